@@ -1,0 +1,125 @@
+"""ctypes binding of libsba_mi355x.so (the C ABI declared in include/sba_mi355x.h).
+
+The library is the only compute path: if it is missing, loading raises and every
+operator call fails loudly.  There is no PyTorch or CPU fallback.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import os
+import threading
+
+import torch
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "csrc", "libsba_mi355x.so")
+
+SBA_DTYPE_F32, SBA_DTYPE_BF16 = 0, 1
+SBA_ABI_VERSION = 1
+
+
+class SbaTensor(C.Structure):
+    _fields_ = [("ptr", C.c_void_p), ("stride_b", C.c_int64), ("stride_h", C.c_int64),
+                ("stride_t", C.c_int64)]
+
+
+class SbaVector(C.Structure):
+    _fields_ = [("ptr", C.c_void_p), ("stride_b", C.c_int64), ("stride_h", C.c_int64)]
+
+
+class SbaParams(C.Structure):
+    _fields_ = [
+        ("struct_size", C.c_uint32), ("dtype", C.c_int32), ("n_seq", C.c_int32),
+        ("n_heads", C.c_int32), ("seq_len", C.c_int32), ("total_tokens", C.c_int32),
+        ("head_dim", C.c_int32), ("attend_current", C.c_int32), ("scale", C.c_float),
+        ("save_for_backward", C.c_int32),
+        ("cu_seqlens", C.c_void_p), ("schedule", C.c_void_p), ("n_schedule", C.c_int32),
+        ("q", SbaTensor), ("k", SbaTensor), ("v", SbaTensor), ("o", SbaTensor),
+        ("rem", SbaVector), ("d_o", SbaTensor), ("d_rem", SbaVector),
+        ("dq", SbaTensor), ("dk", SbaTensor), ("dv", SbaTensor),
+        ("workspace", C.c_void_p), ("workspace_bytes", C.c_size_t), ("stream", C.c_void_p),
+    ]
+
+
+_lib = None
+_lock = threading.Lock()
+
+
+def load() -> C.CDLL:
+    """Load the shared library once; raise if it has not been built."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    with _lock:
+        if _lib is not None:
+            return _lib
+        if not os.path.exists(LIB_PATH):
+            raise RuntimeError(
+                f"{LIB_PATH} is missing: build it with `make -C {os.path.dirname(LIB_PATH)}` "
+                "(or __graft_entry__.build()). There is no fallback path.")
+        lib = C.CDLL(LIB_PATH)
+        lib.sba_abi_version.restype = C.c_int
+        lib.sba_error_string.restype = C.c_char_p
+        lib.sba_error_string.argtypes = [C.c_int]
+        lib.sba_workspace_bytes.restype = C.c_size_t
+        lib.sba_workspace_bytes.argtypes = [C.POINTER(SbaParams)]
+        lib.sba_build_schedule.restype = C.c_int
+        lib.sba_build_schedule.argtypes = [C.POINTER(C.c_int32), C.c_int, C.POINTER(C.c_int32), C.c_int]
+        lib.sba_row_block.restype = C.c_int
+        lib.sba_fwd.restype = C.c_int
+        lib.sba_fwd.argtypes = [C.POINTER(SbaParams)]
+        lib.sba_bwd.restype = C.c_int
+        lib.sba_bwd.argtypes = [C.POINTER(SbaParams)]
+        if lib.sba_abi_version() != SBA_ABI_VERSION:
+            raise RuntimeError("libsba_mi355x.so ABI version mismatch; rebuild it")
+        _lib = lib
+    return _lib
+
+
+EXPORTED_SYMBOLS = ("sba_abi_version", "sba_error_string", "sba_workspace_bytes",
+                    "sba_build_schedule", "sba_row_block", "sba_fwd", "sba_bwd")
+
+
+def check(rc: int, what: str) -> None:
+    if rc != 0:
+        raise RuntimeError(f"{what} failed: {load().sba_error_string(rc).decode()} (code {rc})")
+
+
+def dtype_code(dt: torch.dtype) -> int:
+    if dt == torch.float32:
+        return SBA_DTYPE_F32
+    if dt == torch.bfloat16:
+        return SBA_DTYPE_BF16
+    raise TypeError(f"stick-breaking attention supports float32 and bfloat16, got {dt}")
+
+
+def tensor4(t: torch.Tensor) -> SbaTensor:
+    """[B, H, T, D] view -> descriptor."""
+    return SbaTensor(t.data_ptr(), t.stride(0), t.stride(1), t.stride(2))
+
+
+def tensor3(t: torch.Tensor) -> SbaTensor:
+    """[H, T, D] view -> descriptor (no batch stride)."""
+    return SbaTensor(t.data_ptr(), 0, t.stride(0), t.stride(1))
+
+
+def usable(t: torch.Tensor) -> torch.Tensor:
+    """Kernels need unit stride along D and 16-byte aligned rows; copy otherwise."""
+    ok = t.stride(-1) == 1 and t.data_ptr() % 16 == 0
+    if ok:
+        per16 = 16 // t.element_size()
+        ok = all(s % per16 == 0 for s in t.stride()[:-1])
+    return t if ok else t.contiguous()
+
+
+def build_schedule(cu_host: torch.Tensor) -> torch.Tensor:
+    """Host int32 cu_seqlens (leading 0) -> host int32 [n_jobs, 4] schedule."""
+    lib = load()
+    cu = cu_host.to(torch.int32).contiguous()
+    n_seq = cu.numel() - 1
+    ptr = C.cast(cu.data_ptr(), C.POINTER(C.c_int32))
+    n = lib.sba_build_schedule(ptr, n_seq, None, 0)
+    out = torch.empty((max(n, 1), 4), dtype=torch.int32)
+    got = lib.sba_build_schedule(ptr, n_seq, C.cast(out.data_ptr(), C.POINTER(C.c_int32)), n)
+    assert got == n
+    return out[:n]

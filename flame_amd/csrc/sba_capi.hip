@@ -1,0 +1,171 @@
+// C ABI of libsba_mi355x.so: argument checking, schedule building, kernel dispatch.
+// Declarations and the reference interfaces they replace: include/sba_mi355x.h.
+#include "sba_common.h"
+
+#include <algorithm>
+#include <cstdlib>
+#include <cstring>
+#include <vector>
+
+namespace {
+
+using sba::KParams;
+
+bool force_generic() {
+    const char* e = getenv("SBA_FORCE_GENERIC");
+    return e && e[0] == '1';
+}
+
+// The MFMA kernels cover bf16 with head_dim 64 or 128; everything else takes the
+// generic vector-ALU kernels.
+bool use_mfma(const SbaParams* p) {
+    if (force_generic()) return false;
+    return p->dtype == SBA_DTYPE_BF16 && (p->head_dim == 64 || p->head_dim == 128);
+}
+
+// The MFMA backward is a separate switch so that the two directions can be brought up
+// (and, with SBA_FORCE_GENERIC_BWD=1, cross-checked) independently.
+bool use_mfma_bwd(const SbaParams* p) {
+    const char* e = getenv("SBA_FORCE_GENERIC_BWD");
+    if (e && e[0] == '1') return false;
+    return use_mfma(p) && sba_mfma_bwd_available();
+}
+
+int64_t tab_tokens(const SbaParams* p) {
+    return p->cu_seqlens ? (int64_t)p->total_tokens : (int64_t)p->n_seq * p->seq_len;
+}
+
+int n_key_blocks(const SbaParams* p) { return (p->seq_len + sba::kKeyBlock - 1) / sba::kKeyBlock; }
+
+size_t table_bytes(const SbaParams* p) {
+    size_t b = (size_t)p->n_heads * n_key_blocks(p) * tab_tokens(p) * sizeof(float);
+    return (b + 255) & ~(size_t)255;
+}
+
+size_t generic_acc_bytes(const SbaParams* p) {
+    size_t b = (size_t)2 * tab_tokens(p) * p->n_heads * sba_generic_padded_dim(p->head_dim) * sizeof(float);
+    return (b + 255) & ~(size_t)255;
+}
+
+sba::TensorArg cvt(const SbaTensor& t) { return sba::TensorArg{(char*)t.ptr, t.stride_b, t.stride_h, t.stride_t}; }
+sba::VectorArg cvt(const SbaVector& t) { return sba::VectorArg{(char*)t.ptr, t.stride_b, t.stride_h}; }
+
+int check_common(const SbaParams* p) {
+    if (!p) return SBA_ERR_NULL;
+    if (p->struct_size != sizeof(SbaParams)) return SBA_ERR_ABI;
+    if (p->dtype != SBA_DTYPE_F32 && p->dtype != SBA_DTYPE_BF16) return SBA_ERR_DTYPE;
+    if (p->n_seq <= 0 || p->n_heads <= 0 || p->seq_len <= 0 || p->total_tokens <= 0) return SBA_ERR_SHAPE;
+    if (p->head_dim <= 0 || p->head_dim > 128) return SBA_ERR_SHAPE;
+    if (!p->q.ptr || !p->k.ptr || !p->v.ptr) return SBA_ERR_NULL;
+    if (p->cu_seqlens) {
+        if (!p->schedule || p->n_schedule <= 0) return SBA_ERR_SCHEDULE;
+    } else if (p->total_tokens != p->seq_len) {
+        return SBA_ERR_SHAPE;
+    }
+    return SBA_OK;
+}
+
+KParams make_kparams(const SbaParams* p) {
+    KParams kp;
+    memset(&kp, 0, sizeof(kp));
+    kp.n_seq = p->n_seq; kp.n_heads = p->n_heads; kp.seq_len = p->seq_len;
+    kp.total_tokens = p->total_tokens; kp.head_dim = p->head_dim;
+    kp.attend_current = p->attend_current ? 1 : 0;
+    kp.save = p->save_for_backward ? 1 : 0;
+    kp.scale = p->scale; kp.scale2 = p->scale * sba::kLog2e;
+    kp.cu_seqlens = p->cu_seqlens; kp.schedule = p->schedule;
+    if (p->cu_seqlens) {
+        kp.n_jobs = p->n_schedule;
+    } else {
+        kp.n_jobs = p->n_seq * ((p->seq_len + sba::kRowBlock - 1) / sba::kRowBlock);
+    }
+    kp.q = cvt(p->q); kp.k = cvt(p->k); kp.v = cvt(p->v); kp.o = cvt(p->o);
+    kp.d_o = cvt(p->d_o); kp.dq = cvt(p->dq); kp.dk = cvt(p->dk); kp.dv = cvt(p->dv);
+    kp.rem = cvt(p->rem); kp.d_rem = cvt(p->d_rem);
+    kp.n_kb = n_key_blocks(p);
+    kp.tab_tokens = tab_tokens(p);
+    char* ws = (char*)p->workspace;
+    if (ws && use_mfma(p)) {
+        kp.rtab = (float*)ws;
+        kp.gtab = (float*)(ws + table_bytes(p));
+        ws += 2 * table_bytes(p);
+    }
+    if (ws && !use_mfma_bwd(p)) kp.dkv32 = (float*)ws;
+    return kp;
+}
+
+}  // namespace
+
+extern "C" {
+
+int sba_abi_version(void) { return SBA_ABI_VERSION; }
+
+const char* sba_error_string(int code) {
+    switch (code) {
+        case SBA_OK: return "ok";
+        case SBA_ERR_NULL: return "a required pointer is NULL";
+        case SBA_ERR_SHAPE: return "bad shape: sizes must be positive, head_dim <= 128, dense total_tokens == seq_len";
+        case SBA_ERR_DTYPE: return "unsupported dtype (float32 and bfloat16 only)";
+        case SBA_ERR_WORKSPACE: return "workspace missing or smaller than sba_workspace_bytes()";
+        case SBA_ERR_SCHEDULE: return "packed layout needs a row-block schedule from sba_build_schedule()";
+        case SBA_ERR_LAUNCH: return "kernel launch failed";
+        case SBA_ERR_ABI: return "SbaParams.struct_size does not match this library";
+        default: return "unknown error";
+    }
+}
+
+size_t sba_workspace_bytes(const SbaParams* p) {
+    if (!p || p->n_heads <= 0 || p->seq_len <= 0 || p->head_dim <= 0 || p->head_dim > 128) return 0;
+    size_t b = 0;
+    if (use_mfma(p)) b += 2 * table_bytes(p);
+    if (!use_mfma_bwd(p)) b += generic_acc_bytes(p);
+    return b;
+}
+
+int sba_row_block(void) { return sba::kRowBlock; }
+
+int sba_build_schedule(const int32_t* cu, int n_seq, int32_t* out, int capacity) {
+    if (!cu || n_seq <= 0) return 0;
+    struct J { int32_t tok0, len, rb, doc; };
+    std::vector<J> jobs;
+    for (int s = 0; s < n_seq; ++s) {
+        int32_t len = cu[s + 1] - cu[s];
+        if (len <= 0) continue;
+        int n_rb = (len + sba::kRowBlock - 1) / sba::kRowBlock;
+        for (int rb = 0; rb < n_rb; ++rb) jobs.push_back(J{cu[s], len, rb, s});
+    }
+    // longest sweeps first; a stable order keeps the schedule deterministic
+    std::stable_sort(jobs.begin(), jobs.end(), [](const J& a, const J& b) { return a.rb > b.rb; });
+    int n = (int)jobs.size();
+    if (out && capacity >= n)
+        for (int i = 0; i < n; ++i) {
+            out[4 * i + 0] = jobs[i].tok0; out[4 * i + 1] = jobs[i].len;
+            out[4 * i + 2] = jobs[i].rb;   out[4 * i + 3] = jobs[i].doc;
+        }
+    return n;
+}
+
+int sba_fwd(const SbaParams* p) {
+    int rc = check_common(p);
+    if (rc) return rc;
+    if (!p->o.ptr || !p->rem.ptr) return SBA_ERR_NULL;
+    const bool mfma = use_mfma(p);
+    if (mfma && p->save_for_backward) {
+        if (!p->workspace || p->workspace_bytes < sba_workspace_bytes(p)) return SBA_ERR_WORKSPACE;
+    }
+    KParams kp = make_kparams(p);
+    hipStream_t s = (hipStream_t)p->stream;
+    return mfma ? sba_launch_mfma_fwd(kp, s) : sba_launch_generic_fwd(kp, p->dtype, s);
+}
+
+int sba_bwd(const SbaParams* p) {
+    int rc = check_common(p);
+    if (rc) return rc;
+    if (!p->d_o.ptr || !p->dq.ptr || !p->dk.ptr || !p->dv.ptr) return SBA_ERR_NULL;
+    if (!p->workspace || p->workspace_bytes < sba_workspace_bytes(p)) return SBA_ERR_WORKSPACE;
+    KParams kp = make_kparams(p);
+    hipStream_t s = (hipStream_t)p->stream;
+    return use_mfma_bwd(p) ? sba_launch_mfma_bwd(kp, s) : sba_launch_generic_bwd(kp, p->dtype, s);
+}
+
+}  // extern "C"

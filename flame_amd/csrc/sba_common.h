@@ -1,0 +1,86 @@
+// Shared device/host helpers for the stick-breaking attention kernels (gfx950).
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include "../../include/sba_mi355x.h"
+
+namespace sba {
+
+constexpr int kRowBlock = 128;   // query rows per scheduled job (one workgroup)
+constexpr int kKeyBlock = 64;    // keys per sweep step of the MFMA kernels / carry-table column
+
+// Logits above this (in base-2 units) are clamped: sigmoid(z) differs from 1 by < 2^-30
+// there, so outputs move by < 1e-9, and exp2 of the clamped value cannot overflow.
+constexpr float kMaxLogit2 = 30.0f;
+constexpr float kLog2e = 1.4426950408889634f;
+
+struct TensorArg { char* ptr; int64_t sb, sh, st; };
+struct VectorArg { char* ptr; int64_t sb, sh; };
+
+// Kernel-side copy of SbaParams (by value in the launch).
+struct KParams {
+    int n_seq, n_heads, seq_len, total_tokens, head_dim, attend_current, save, n_jobs;
+    float scale2;                  // scale * log2(e): logits in base-2 units
+    float scale;                   // natural-unit scale (for dq/dk)
+    const int32_t* cu_seqlens;
+    const int32_t* schedule;
+    TensorArg q, k, v, o, d_o, dq, dk, dv;
+    VectorArg rem, d_rem;
+    float* rtab;                   // forward carry table  [H][n_kb][total_tokens] (x n_seq for dense)
+    float* gtab;                   // backward prefix table, same shape
+    float* dkv32;                  // generic path: fp32 dk|dv accumulators
+    int n_kb;                      // carry-table columns = ceil(seq_len / kKeyBlock)
+    int64_t tab_tokens;            // tokens per head in the tables (n_seq*T dense, sumT packed)
+};
+
+struct Job { int tok0, len, rb, seq; };
+
+// blockIdx.x = job * n_heads + head.  Dense jobs are generated arithmetically, longest
+// row-blocks first; packed jobs come from the host-built schedule.
+__device__ inline Job decode_job(const KParams& p, int job) {
+    Job j;
+    if (p.cu_seqlens == nullptr) {
+        int n_rb = (p.seq_len + kRowBlock - 1) / kRowBlock;
+        j.rb = n_rb - 1 - job / p.n_seq;
+        j.seq = job % p.n_seq;
+        j.tok0 = 0;
+        j.len = p.seq_len;
+    } else {
+        const int32_t* s = p.schedule + 4 * (int64_t)job;
+        j.tok0 = s[0]; j.len = s[1]; j.rb = s[2]; j.seq = 0;
+    }
+    return j;
+}
+
+// Token index inside the carry tables.
+__device__ inline int64_t tab_token(const KParams& p, const Job& j, int local) {
+    return (p.cu_seqlens == nullptr) ? (int64_t)j.seq * p.seq_len + local : (int64_t)j.tok0 + local;
+}
+
+__device__ inline float bf16_to_f32(uint16_t b) { return __uint_as_float(((uint32_t)b) << 16); }
+__device__ inline uint16_t f32_to_bf16(float f) {   // round to nearest even
+    uint32_t u = __float_as_uint(f);
+    if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x40);
+    u += 0x7fffu + ((u >> 16) & 1u);
+    return (uint16_t)(u >> 16);
+}
+
+template <typename T> struct Elem;
+template <> struct Elem<float> {
+    __device__ static float load(const char* p, int64_t i) { return ((const float*)p)[i]; }
+    __device__ static void store(char* p, int64_t i, float v) { ((float*)p)[i] = v; }
+};
+template <> struct Elem<uint16_t> {   // bf16 bits
+    __device__ static float load(const char* p, int64_t i) { return bf16_to_f32(((const uint16_t*)p)[i]); }
+    __device__ static void store(char* p, int64_t i, float v) { ((uint16_t*)p)[i] = f32_to_bf16(v); }
+};
+
+}  // namespace sba
+
+// Launchers implemented in the kernel translation units.
+int sba_generic_padded_dim(int D);
+int sba_launch_generic_fwd(const sba::KParams& kp, int dtype, hipStream_t s);
+int sba_launch_generic_bwd(const sba::KParams& kp, int dtype, hipStream_t s);
+int sba_launch_mfma_fwd(const sba::KParams& kp, hipStream_t s);
+int sba_launch_mfma_bwd(const sba::KParams& kp, hipStream_t s);
+bool sba_mfma_bwd_available();

@@ -1,0 +1,177 @@
+// Building blocks of the bf16 MFMA kernels (gfx950): LDS tile layout, global->LDS tile
+// copies, MFMA operand fetches and the per-tile stick-breaking arithmetic.
+//
+// Geometry.  A workgroup is 4 waves; wave w owns 32 query rows.  A sweep step covers
+// 64 keys.  All score tiles are computed TRANSPOSED, S^T = K * Q^T, with
+// v_mfma_f32_32x32x16_bf16: in its 32x32 accumulator layout lane (n = lane%32,
+// h = lane/32) holds column n (one query) and rows 8*(r/4) + 4*h + r%4, r = 0..15.
+// The 64 keys of a step are assigned to the two 32-row tiles t = 0,1 so that
+//     key_local = 32*h + 16*t + r
+// i.e. each lane holds 32 CONSECUTIVE keys of one query in registers (idx = 16*t + r),
+// lower half-wave the left 32 keys, upper half-wave the right 32.  The products along
+// the key axis that stick-breaking needs are then in-register chains plus one
+// cross-half exchange per step, and the packed bf16 weights are directly the B operand of
+// the following MFMAs (O^T += V^T * P^T, dQ^T += K^T * dZ^T).
+//
+// LDS tiles hold 64 rows of D bf16.  Row order is "MFMA order": key_local
+// 32*hh + 16*t + 4*g + i lives in row rho = 32*t + 8*g + 4*hh + i, so that the A-operand
+// fetch of tile t reads rows 32*t + lane%32.  16-byte chunks of a row are XOR-swizzled
+// (see swz()) so that both access patterns used here are bank-conflict free:
+//   * row fetches   (ds_read_b128: 16 consecutive rows, one chunk each) and
+//   * transposing fetches (ds_read_b64_tr_b16: 4 consecutive rows x 64 bytes).
+#pragma once
+#include "sba_common.h"
+
+namespace sba {
+
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2;
+typedef __attribute__((ext_vector_type(2))) float f32x2;
+typedef __attribute__((ext_vector_type(16))) float f32x16;
+typedef __attribute__((ext_vector_type(4))) short s16x4;
+typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
+
+constexpr int kThreads = 256;
+
+__device__ inline int mfma_row_of_key(int kl) {   // key_local -> LDS row
+    return ((kl >> 4) & 1) * 32 + ((kl >> 2) & 3) * 8 + (kl >> 5) * 4 + (kl & 3);
+}
+
+template <int D> __device__ inline int swz(int row);
+template <> __device__ inline int swz<64>(int row) {   // 8 chunks per row
+    int v = (row >> 1) & 7;
+    return ((v & 1) << 2) | (v & 2) | ((v >> 2) & 1);
+}
+template <> __device__ inline int swz<128>(int row) {  // 16 chunks per row
+    return ((row & 3) << 2) | ((row >> 2) & 3);
+}
+
+template <int D> __device__ inline int tile_offset(int row, int chunk) {   // bytes
+    return row * (D * 2) + ((chunk ^ swz<D>(row)) << 4);
+}
+
+// Global -> registers -> LDS copy of one 64-row tile (rows row0..row0+63 of a sequence),
+// split so that the global loads of the next tile overlap the arithmetic on this one.
+template <int D> struct TileCopy {
+    static constexpr int kChunks = 64 * D / 8;                 // 16-byte chunks per tile
+    static constexpr int kPerThread = kChunks / kThreads;      // 2 (D=64) or 4 (D=128)
+    u32x4 regs[kPerThread];
+
+    // rows of the tile in MFMA order when `permute`, natural order otherwise
+    __device__ inline void load(const TensorArg& t, int64_t base, int row0, int len) {
+#pragma unroll
+        for (int r = 0; r < kPerThread; ++r) {
+            int cid = threadIdx.x + r * kThreads;
+            int kl = cid / (D / 8), c = cid % (D / 8);
+            int row = row0 + kl;
+            u32x4 v = {0u, 0u, 0u, 0u};
+            if (row < len) v = *(const u32x4*)(t.ptr + 2 * (base + (int64_t)row * t.st + c * 8));
+            regs[r] = v;
+        }
+    }
+    __device__ inline void store(char* tile) const {
+#pragma unroll
+        for (int r = 0; r < kPerThread; ++r) {
+            int cid = threadIdx.x + r * kThreads;
+            int kl = cid / (D / 8), c = cid % (D / 8);
+            *(u32x4*)(tile + tile_offset<D>(mfma_row_of_key(kl), c)) = regs[r];
+        }
+    }
+};
+
+// A operand, row fetch: lane (m = lane%32, h = lane/32) gets 8 bf16 of row 32*t + m,
+// columns 16*ks + 8*h .. +7.
+template <int D> __device__ inline bf16x8 fetch_rows(const char* tile, int t, int ks, int lane) {
+    int row = 32 * t + (lane & 31);
+    int chunk = 2 * ks + (lane >> 5);
+    return *(const bf16x8*)(tile + tile_offset<D>(row, chunk));
+}
+
+// A operand, transposing fetch: lane (m = lane%32, h = lane/32) gets column 32*db + m of
+// the 8 keys key_local = 32*h + 8*c + j, j = 0..7.  Each ds_read_b64_tr_b16 makes 16
+// lanes read a [4 rows x 16 columns] block (lane s: row s/4, columns 4*(s%4)..+3) and
+// hands lane s column s of it.
+template <int D> __device__ inline bf16x8 fetch_cols(const char* tile, int db, int c, int lane) {
+    const int h = lane >> 5, G1 = (lane >> 4) & 1, s = lane & 15;
+    const int chunk = 4 * db + 2 * G1 + ((s & 3) >> 1);
+    const int sub = (s & 1) << 3;
+    union { s16x4 v[2]; bf16x8 b; } u;
+#pragma unroll
+    for (int a = 0; a < 2; ++a) {
+        int row = 32 * (c >> 1) + 8 * (2 * (c & 1) + a) + 4 * h + (s >> 2);
+        const char* p = tile + tile_offset<D>(row, chunk) + sub;
+        u.v[a] = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+            (__attribute__((address_space(3))) s16x4*)(uintptr_t)(uint32_t)(uintptr_t)p);
+    }
+    return u.b;
+}
+
+// B operand kept in registers for the whole sweep: row `row` of a [rows, D] tensor,
+// columns 16*ks + 8*h .. +7 for every ks.  Rows >= len read as zero.
+template <int D>
+__device__ inline void load_row_frags(bf16x8 (&f)[D / 16], const TensorArg& t, int64_t base, int row,
+                                      int len, int lane) {
+    const int h = lane >> 5;
+#pragma unroll
+    for (int ks = 0; ks < D / 16; ++ks) {
+        u32x4 v = {0u, 0u, 0u, 0u};
+        if (row < len) v = *(const u32x4*)(t.ptr + 2 * (base + (int64_t)row * t.st + 16 * ks + 8 * h));
+        f[ks] = __builtin_bit_cast(bf16x8, v);
+    }
+}
+
+__device__ inline bf16x8 pack8(const float* p) {
+    bf16x8 r;
+#pragma unroll
+    for (int i = 0; i < 8; i += 2) {
+        f32x2 v = {p[i], p[i + 1]};
+        bf16x2 b = __builtin_convertvector(v, bf16x2);
+        r[i] = b[0]; r[i + 1] = b[1];
+    }
+    return r;
+}
+
+__device__ inline f32x16 mfma(bf16x8 a, bf16x8 b, f32x16 c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
+}
+
+// S^T tile pair for one wave: x[16*t + r] = scale2 * (K Q^T)[key_local = 32h+16t+r][query n].
+template <int D>
+__device__ inline void score_tiles(float (&x)[32], const char* ktile, const bf16x8 (&qf)[D / 16],
+                                   float scale2, int lane) {
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+        f32x16 acc = {0};
+#pragma unroll
+        for (int ks = 0; ks < D / 16; ++ks) acc = mfma(fetch_rows<D>(ktile, t, ks, lane), qf[ks], acc);
+#pragma unroll
+        for (int r = 0; r < 16; ++r) x[16 * t + r] = acc[r] * scale2;
+    }
+}
+
+// In-place: x[idx] (base-2 logits, idx = key offset inside this lane's 32 keys; invalid
+// pairs already set to -inf) -> stick-breaking weights of this step, given the carry
+// `R` = product of (1 - beta) over all keys right of this 64-key step.
+//   e = 2^x, u = 1/(1+e);  local chain right-to-left;  one exchange between half-waves.
+// Outputs: x[idx] = A (attention weight); beta[idx] when kNeedBeta; R updated to the carry
+// for the next (left) step.
+template <bool kNeedBeta>
+__device__ inline void stick_weights(float (&x)[32], float (&beta)[kNeedBeta ? 32 : 1], float& R, int lane) {
+    float L = 1.0f;
+#pragma unroll
+    for (int idx = 31; idx >= 0; --idx) {
+        float e = __builtin_amdgcn_exp2f(fminf(x[idx], kMaxLogit2));
+        float u = __builtin_amdgcn_rcpf(1.0f + e);
+        L *= u;
+        x[idx] = e * L;
+        if (kNeedBeta) beta[idx] = e * u;
+    }
+    const float other = __shfl_xor(L, 32);
+    // upper half-wave holds the right 32 keys: its chain starts from R itself
+    const float F = (lane >= 32) ? R : R * other;
+#pragma unroll
+    for (int idx = 0; idx < 32; ++idx) x[idx] *= F;
+    R = R * L * other;
+}
+
+}  // namespace sba

@@ -1,0 +1,120 @@
+// bf16 MFMA forward kernel (head_dim 64 / 128).
+// Replaces the reference's `_forward_one_row` sweep (sb_varlen/sb_varlen_fwd.py:81-215):
+// one workgroup per (sequence, head, 128-query row-block), keys swept right-to-left from
+// the diagonal in steps of 64, K/V tiles double-buffered in LDS, running product of
+// (1 - beta) per query in a register.  Layout and arithmetic: sba_mfma.h.
+#include "sba_mfma.h"
+
+namespace sba {
+
+template <int D>
+__global__ __launch_bounds__(kThreads) void mfma_fwd_kernel(KParams p) {
+    constexpr int kTile = 64 * D * 2;            // bytes per K or V tile
+    __shared__ __attribute__((aligned(16))) char lds[4 * kTile];   // K0 V0 K1 V1
+
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int n = lane & 31, h = lane >> 5;
+    const int head = blockIdx.x % p.n_heads;
+    const Job job = decode_job(p, blockIdx.x / p.n_heads);
+    const int strict = p.attend_current ? 0 : 1;
+    const int m0 = job.rb * kRowBlock;
+    const int q0w = m0 + 32 * wave;              // first query of this wave
+    const int qi = q0w + n;                      // this lane's query
+    const int64_t qbase = (int64_t)job.seq * p.q.sb + (int64_t)head * p.q.sh + (int64_t)job.tok0 * p.q.st;
+    const int64_t kbase = (int64_t)job.seq * p.k.sb + (int64_t)head * p.k.sh + (int64_t)job.tok0 * p.k.st;
+    const int64_t vbase = (int64_t)job.seq * p.v.sb + (int64_t)head * p.v.sh + (int64_t)job.tok0 * p.v.st;
+
+    bf16x8 qf[D / 16];
+    load_row_frags<D>(qf, p.q, qbase, qi, job.len, lane);
+
+    f32x16 oacc[D / 32];
+#pragma unroll
+    for (int db = 0; db < D / 32; ++db) oacc[db] = f32x16{0};
+    float R = 1.0f;
+
+    const int imax = min(m0 + kRowBlock - 1, job.len - 1);
+    const int kmax = imax - strict;                       // last key any row of the block sees
+    const int n_steps = kmax >= 0 ? kmax / kKeyBlock + 1 : 0;
+    const int64_t tabtok = tab_token(p, job, qi);
+
+    TileCopy<D> kc, vc;
+    if (n_steps > 0) {
+        kc.load(p.k, kbase, (n_steps - 1) * kKeyBlock, job.len);
+        vc.load(p.v, vbase, (n_steps - 1) * kKeyBlock, job.len);
+        kc.store(lds);
+        vc.store(lds + kTile);
+    }
+    __syncthreads();
+
+    for (int step = n_steps - 1, buf = 0; step >= 0; --step, buf ^= 1) {
+        const char* ktile = lds + buf * 2 * kTile;
+        const char* vtile = ktile + kTile;
+        const bool more = step > 0;
+        if (more) {
+            kc.load(p.k, kbase, (step - 1) * kKeyBlock, job.len);
+            vc.load(p.v, vbase, (step - 1) * kKeyBlock, job.len);
+        }
+        const int key0 = step * kKeyBlock;
+        // whole step right of this wave's last query: nothing visible
+        const bool skip = key0 + strict > q0w + 31;
+        if (!skip) {
+            float x[32];
+            score_tiles<D>(x, ktile, qf, p.scale2, lane);
+            if (key0 + 63 + strict > q0w) {     // diagonal region: mask invisible pairs
+#pragma unroll
+                for (int idx = 0; idx < 32; ++idx) {
+                    int j = key0 + 32 * h + idx;
+                    if (j + strict > qi) x[idx] = -INFINITY;
+                }
+            }
+            if (p.save && h == 0 && qi < job.len)
+                p.rtab[((int64_t)head * p.n_kb + step) * p.tab_tokens + tabtok] = R;
+            float dummy[1];
+            stick_weights<false>(x, dummy, R, lane);
+            bf16x8 pf[4];
+#pragma unroll
+            for (int c = 0; c < 4; ++c) pf[c] = pack8(&x[8 * c]);
+#pragma unroll
+            for (int db = 0; db < D / 32; ++db)
+#pragma unroll
+                for (int c = 0; c < 4; ++c)
+                    oacc[db] = mfma(fetch_cols<D>(vtile, db, c, lane), pf[c], oacc[db]);
+        }
+        if (more) {
+            kc.store(lds + (buf ^ 1) * 2 * kTile);
+            vc.store(lds + (buf ^ 1) * 2 * kTile + kTile);
+        }
+        __syncthreads();
+    }
+
+    if (qi < job.len) {
+        const int64_t obase = (int64_t)job.seq * p.o.sb + (int64_t)head * p.o.sh + (int64_t)(job.tok0 + qi) * p.o.st;
+#pragma unroll
+        for (int db = 0; db < D / 32; ++db)
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                // rows d = 32*db + 8*g + 4*h + 0..3 of O^T, column = this query
+                f32x2 a = {oacc[db][4 * g], oacc[db][4 * g + 1]};
+                f32x2 b = {oacc[db][4 * g + 2], oacc[db][4 * g + 3]};
+                bf16x2 pa = __builtin_convertvector(a, bf16x2), pb = __builtin_convertvector(b, bf16x2);
+                uint2 w;
+                w.x = __builtin_bit_cast(uint32_t, pa);
+                w.y = __builtin_bit_cast(uint32_t, pb);
+                *(uint2*)(p.o.ptr + 2 * (obase + 32 * db + 8 * g + 4 * h)) = w;
+            }
+        if (h == 0)
+            Elem<uint16_t>::store(p.rem.ptr, (int64_t)job.seq * p.rem.sb + (int64_t)head * p.rem.sh + job.tok0 + qi, R);
+    }
+}
+
+}  // namespace sba
+
+int sba_launch_mfma_fwd(const sba::KParams& kp, hipStream_t s) {
+    using namespace sba;
+    dim3 grid((unsigned)kp.n_jobs * kp.n_heads);
+    if (kp.head_dim == 64)
+        hipLaunchKernelGGL((mfma_fwd_kernel<64>), grid, dim3(kThreads), 0, s, kp);
+    else
+        hipLaunchKernelGGL((mfma_fwd_kernel<128>), grid, dim3(kThreads), 0, s, kp);
+    return hipGetLastError() == hipSuccess ? SBA_OK : SBA_ERR_LAUNCH;
+}

@@ -1,0 +1,134 @@
+/*
+ * C ABI of libsba_mi355x.so: stick-breaking attention for AMD MI355X (gfx950).
+ *
+ * Plain pointers and sizes only; no torch types.  All tensor pointers are device
+ * pointers (HIP), all launches are asynchronous on `stream`, nothing is allocated,
+ * nothing synchronises, and no global state is kept, so every entry point may be called
+ * from any thread.  Return value: 0 on success, a negative SBA_ERR_* code otherwise
+ * (sba_error_string() gives the text).
+ *
+ * The reference has no native code; what each entry point replaces is the Python host
+ * launcher plus the Triton kernel it starts (paths relative to the reference tree,
+ * custom_models/sba/stickbreaking_attention/):
+ *
+ *   sba_fwd  <-  sb_attn/sb_fwd.py:139-253   (_fwd / _compileable_fwd -> dense _forward)
+ *                sb_varlen/sb_varlen_fwd.py:408-516 (varlen_fwd -> varlen _forward)
+ *   sba_bwd  <-  sb_attn/sb_bwd.py:163-297   (_bwd / _compileable_backward -> dense _backward)
+ *                sb_varlen/sb_varlen_bwd.py:459-615 (varlen_bwd -> varlen _backward)
+ *
+ * Tensor layout.  One descriptor covers both reference layouts:
+ *   dense  [B, H, T, D]  : n_seq = B, seq_len = T, cu_seqlens = NULL,
+ *                          element (b,h,t,d) at  base + b*stride_b + h*stride_h + t*stride_t + d
+ *   packed [H, sumT, D]  : n_seq = number of documents, cu_seqlens = device int32[n_seq+1]
+ *                          with cu_seqlens[0] == 0, stride_b = 0,
+ *                          element (h,t,d) at    base + h*stride_h + t*stride_t + d
+ * Strides are in elements; the innermost (D) stride is 1.
+ */
+#ifndef SBA_MI355X_H
+#define SBA_MI355X_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define SBA_ABI_VERSION 1
+
+enum { SBA_DTYPE_F32 = 0, SBA_DTYPE_BF16 = 1 };
+
+enum {
+    SBA_OK = 0,
+    SBA_ERR_NULL = -1,        /* a required pointer is NULL */
+    SBA_ERR_SHAPE = -2,       /* non-positive size, head_dim unsupported, bad strides */
+    SBA_ERR_DTYPE = -3,       /* unknown dtype */
+    SBA_ERR_WORKSPACE = -4,   /* workspace missing or too small */
+    SBA_ERR_SCHEDULE = -5,    /* packed layout without a row-block schedule */
+    SBA_ERR_LAUNCH = -6,      /* hipGetLastError() after a launch was not hipSuccess */
+    SBA_ERR_ABI = -7          /* struct_size does not match this library */
+};
+
+/* One tensor of q/k/v/o/do/dq/dk/dv shape. */
+typedef struct SbaTensor {
+    void*   ptr;
+    int64_t stride_b;   /* 0 for the packed layout */
+    int64_t stride_h;
+    int64_t stride_t;
+} SbaTensor;
+
+/* One per-token vector (rem, drem): element (b,h,t) at ptr + b*stride_b + h*stride_h + t. */
+typedef struct SbaVector {
+    void*   ptr;
+    int64_t stride_b;
+    int64_t stride_h;
+} SbaVector;
+
+typedef struct SbaParams {
+    uint32_t struct_size;      /* = sizeof(SbaParams); checked */
+    int32_t  dtype;            /* SBA_DTYPE_*: element type of q,k,v,o,rem,do,drem,dq,dk,dv */
+    int32_t  n_seq;            /* B (dense) or number of documents (packed) */
+    int32_t  n_heads;
+    int32_t  seq_len;          /* T (dense) or max document length (packed) */
+    int32_t  total_tokens;     /* T (dense) or sumT (packed) */
+    int32_t  head_dim;         /* D */
+    int32_t  attend_current;   /* 0: keys j < i;  1: keys j <= i */
+    float    scale;            /* logit scale ("inv_temp") in natural-log units */
+    int32_t  save_for_backward;/* forward only: also fill the carry table in workspace */
+
+    const int32_t* cu_seqlens; /* device, n_seq+1 entries, or NULL for dense */
+    const int32_t* schedule;   /* device, from sba_build_schedule(); packed layout only */
+    int32_t  n_schedule;       /* number of row-block jobs in `schedule` */
+
+    SbaTensor q, k, v;         /* inputs */
+    SbaTensor o;               /* forward output            / backward: unused */
+    SbaVector rem;             /* forward output            / backward: unused */
+    SbaTensor d_o;             /* backward input  (grad of o) */
+    SbaVector d_rem;           /* backward input  (grad of rem); ptr may be NULL = zeros */
+    SbaTensor dq, dk, dv;      /* backward outputs */
+
+    void*    workspace;        /* device scratch, see sba_workspace_bytes() */
+    size_t   workspace_bytes;
+    void*    stream;           /* hipStream_t */
+} SbaParams;
+
+/* Library identity: SBA_ABI_VERSION it was built with. */
+int sba_abi_version(void);
+
+/* Text for an SBA_ERR_* code (static storage). */
+const char* sba_error_string(int code);
+
+/*
+ * Bytes of device workspace the pair (sba_fwd with save_for_backward, sba_bwd) needs for
+ * this problem.  The forward writes its per-key-block carry table there and the backward
+ * reads it back, so the SAME buffer, untouched in between, must be given to both calls
+ * (the Python layer keeps it in the autograd context the way the reference keeps
+ * neg_log_acc, sb_attn/__init__.py:30).  Only the size fields of `p` are read.
+ */
+size_t sba_workspace_bytes(const SbaParams* p);
+
+/*
+ * Row-block schedule for the packed layout, built on the host from host cu_seqlens
+ * (n_seq+1 entries, leading 0).  Writes up to `capacity` jobs of 4 int32 each
+ * {first_token, doc_len, row_block, doc_index} into `out` (host memory), longest
+ * row-blocks first, and returns the number of jobs (or the number needed when
+ * `out` is NULL or capacity is too small).  The caller copies it to the device and passes
+ * it as SbaParams.schedule.  Replaces the reference's 3-D launch grid
+ * (n_docs, ceil(H/2), ceil(max_len/64)+1) and its long/short head pairing
+ * (sb_varlen_fwd.py:288-289, 472-475).
+ */
+int sba_build_schedule(const int32_t* cu_seqlens_host, int n_seq, int32_t* out, int capacity);
+
+/* Rows of queries one scheduled job covers (the kernels' row-block height). */
+int sba_row_block(void);
+
+/* Forward: o, rem (and the carry table when save_for_backward). */
+int sba_fwd(const SbaParams* p);
+
+/* Backward: dq, dk, dv from d_o, d_rem, q, k, v and the forward's carry table. */
+int sba_bwd(const SbaParams* p);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* SBA_MI355X_H */

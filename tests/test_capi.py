@@ -1,0 +1,87 @@
+"""CPU tests of the C-ABI shared library: it loads, exports every symbol the header
+declares, and its host-only entry points (schedule builder, argument checks) behave."""
+import ctypes as C
+import os
+import re
+
+import pytest
+import torch
+
+from flame_amd import _lib
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+@pytest.fixture(scope="module")
+def lib():
+    if not os.path.exists(_lib.LIB_PATH):
+        import __graft_entry__
+        __graft_entry__.build()
+    return _lib.load()
+
+
+def test_exports_every_declared_symbol(lib):
+    header = open(os.path.join(ROOT, "include", "sba_mi355x.h")).read()
+    header = re.sub(r"/\*.*?\*/", "", header, flags=re.S)
+    declared = set(re.findall(r"\b(sba_[a-z_]+)\s*\(", header))
+    assert declared == set(_lib.EXPORTED_SYMBOLS)
+    for name in declared:
+        assert getattr(lib, name) is not None
+
+
+def test_abi_version_and_struct_size(lib):
+    assert lib.sba_abi_version() == 1
+    p = _lib.SbaParams()
+    p.struct_size = C.sizeof(_lib.SbaParams) - 8
+    assert lib.sba_fwd(C.byref(p)) == -7          # SBA_ERR_ABI, before anything touches a GPU
+    assert b"struct_size" in lib.sba_error_string(-7)
+
+
+def test_argument_checks_without_gpu(lib):
+    p = _lib.SbaParams()
+    p.struct_size = C.sizeof(_lib.SbaParams)
+    p.dtype = 7
+    assert lib.sba_fwd(C.byref(p)) == -3          # dtype
+    p.dtype = _lib.SBA_DTYPE_BF16
+    assert lib.sba_fwd(C.byref(p)) == -2          # shape (all zero)
+    p.n_seq, p.n_heads, p.seq_len, p.total_tokens, p.head_dim = 1, 2, 64, 64, 256
+    assert lib.sba_fwd(C.byref(p)) == -2          # head_dim > 128
+    p.head_dim = 64
+    assert lib.sba_fwd(C.byref(p)) == -1          # NULL q/k/v
+    assert lib.sba_fwd(None) == -1
+    assert lib.sba_row_block() == 128
+
+
+def test_workspace_bytes(lib):
+    p = _lib.SbaParams()
+    p.struct_size = C.sizeof(_lib.SbaParams)
+    p.dtype = _lib.SBA_DTYPE_BF16
+    p.n_seq, p.n_heads, p.seq_len, p.total_tokens, p.head_dim = 1, 16, 4096, 4096, 64
+    n = lib.sba_workspace_bytes(C.byref(p))
+    assert n >= 2 * 16 * 64 * 4096 * 4            # two carry tables [H][T/64][T] fp32
+    p.dtype = _lib.SBA_DTYPE_F32
+    assert lib.sba_workspace_bytes(C.byref(p)) == 2 * 4096 * 16 * 64 * 4
+
+
+def test_schedule_builder(lib):
+    cu = torch.tensor([0, 100, 400, 401, 1000, 1000], dtype=torch.int32)   # last doc empty
+    s = _lib.build_schedule(cu)
+    jobs = [tuple(r) for r in s.tolist()]
+    # every (doc, row_block) exactly once, none for the empty document
+    expect = {(0, 100, 0, 0), (100, 300, 0, 1), (100, 300, 1, 1), (100, 300, 2, 1), (400, 1, 0, 2)}
+    expect |= {(401, 599, rb, 3) for rb in range(5)}
+    assert set(jobs) == expect and len(jobs) == len(expect)
+    rbs = [j[2] for j in jobs]
+    assert rbs == sorted(rbs, reverse=True)       # longest sweeps first
+    # capacity too small: returns the count needed and writes nothing
+    out = torch.full((2, 4), -1, dtype=torch.int32)
+    n = lib.sba_build_schedule(C.cast(cu.data_ptr(), C.POINTER(C.c_int32)), 5,
+                               C.cast(out.data_ptr(), C.POINTER(C.c_int32)), 2)
+    assert n == len(expect) and bool((out == -1).all())
+
+
+def test_op_refuses_cpu_tensors():
+    from flame_amd import sb_attn
+    q = torch.zeros(1, 1, 4, 8)
+    with pytest.raises(RuntimeError, match="GPU only"):
+        sb_attn(q, q, q)
