@@ -174,4 +174,64 @@ __device__ inline void stick_weights(float (&x)[32], float (&beta)[kNeedBeta ? 3
     R = R * L * other;
 }
 
+// Transposing fetch from a tile whose rows are in NATURAL order (Q, dO, and the weight
+// tiles of the key-owner pass): lane (m = lane%32, h = lane/32) gets column 32*cb + m of
+// rows row0 + 8*h + j, j = 0..7.  ROWD is the row length in bf16 (selects the swizzle).
+template <int ROWD> __device__ inline bf16x8 fetch_cols_nat(const char* tile, int row0, int cb, int lane) {
+    const int h = lane >> 5, G1 = (lane >> 4) & 1, s = lane & 15;
+    const int chunk = 4 * cb + 2 * G1 + ((s & 3) >> 1);
+    const int sub = (s & 1) << 3;
+    union { s16x4 v[2]; bf16x8 b; } u;
+#pragma unroll
+    for (int a = 0; a < 2; ++a) {
+        int row = row0 + 8 * h + 4 * a + (s >> 2);
+        const char* p = tile + tile_offset<ROWD>(row, chunk) + sub;
+        u.v[a] = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+            (__attribute__((address_space(3))) s16x4*)(uintptr_t)(uint32_t)(uintptr_t)p);
+    }
+    return u.b;
+}
+
+// Row fetch from a natural-order tile: 8 bf16 of row `row`, columns 16*ks + 8*h .. +7.
+template <int ROWD> __device__ inline bf16x8 fetch_row_nat(const char* tile, int row, int ks, int lane) {
+    return *(const bf16x8*)(tile + tile_offset<ROWD>(row, 2 * ks + (lane >> 5)));
+}
+
+// dP^T tile pair: dp[16*t + r] = (V dO^T)[key_local][query] - drem[query].
+template <int D>
+__device__ inline void dp_tiles(float (&dp)[32], const char* vtile, const bf16x8 (&dof)[D / 16], float dr,
+                                int lane) {
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+        f32x16 acc;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[r] = -dr;
+#pragma unroll
+        for (int ks = 0; ks < D / 16; ++ks) acc = mfma(fetch_rows<D>(vtile, t, ks, lane), dof[ks], acc);
+#pragma unroll
+        for (int r = 0; r < 16; ++r) dp[16 * t + r] = acc[r];
+    }
+}
+
+// Gradient of the logits for one step.  In: a[idx] attention weights, beta[idx],
+// dp[idx] = dO.v - drem, Gc = sum of g over all keys LEFT of this step.
+// Out: dp[idx] <- dz = g - beta * prefix_sum(g);  Gc advanced past this step.
+__device__ inline void logit_grads(const float (&a)[32], const float (&beta)[32], float (&dp)[32], float& Gc,
+                                   int lane) {
+    float c = 0.f;
+    float pre[32];
+#pragma unroll
+    for (int idx = 0; idx < 32; ++idx) {
+        dp[idx] = a[idx] * dp[idx];     // g
+        c += dp[idx];
+        pre[idx] = c;
+    }
+    const float other = __shfl_xor(c, 32);
+    // lower half-wave holds the left 32 keys
+    const float F = (lane >= 32) ? Gc + other : Gc;
+#pragma unroll
+    for (int idx = 0; idx < 32; ++idx) dp[idx] = dp[idx] - beta[idx] * (pre[idx] + F);
+    Gc = Gc + c + other;
+}
+
 }  // namespace sba
