@@ -1,0 +1,176 @@
+"""Benchmark of the stick-breaking attention hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload cfg2|cfg3|cfg4]
+
+A step is one forward + backward of the operator through its public autograd API on
+synthetic inputs already resident in HBM.  Prints ONE JSON line.
+"""
+import argparse
+import json
+import math
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+BF16_MFMA_PEAK_TFLOPS = 2516.6     # 256 CU x 2.4 GHz x 4096 FLOP/clk/CU (dense bf16)
+
+
+def _lognormal_lengths(total, seed, median=600.0, sigma=1.0, lo=16, hi=4096):
+    import torch
+    g = torch.Generator().manual_seed(seed)
+    lens, s = [], 0
+    while s < total:
+        L = int(round(math.exp(math.log(median) + sigma * torch.randn((), generator=g).item())))
+        L = max(lo, min(hi, L))
+        L = min(L, total - s)
+        if L < lo and lens:
+            lens[-1] += L       # a truncated tail shorter than `lo` joins the previous document
+        else:
+            lens.append(L)
+        s += L
+    return lens
+
+
+def make_workload(name, device):
+    """Returns (description, step_fn inputs, number of allowed pairs P, tokens, d)."""
+    import torch
+    g = torch.Generator().manual_seed(0)
+
+    def rn(shape, scale):
+        return (torch.randn(shape, generator=g) * scale).to(torch.bfloat16).to(device)
+
+    if name == "cfg2":
+        B, H, T, D = 1, 16, 4096, 64
+        q, k, v = rn((B, H, T, D), 0.5), rn((B, H, T, D), 0.5), rn((B, H, T, D), 0.5)
+        do = rn((B, H, T, D), 1.0)
+        pairs = B * H * T * (T - 1) // 2
+        desc = {"workload": "cfg2: dense causal fwd+bwd B=1 H=16 T=4096 d=64 bf16", "B": B, "H": H, "T": T, "d": D}
+        return desc, (q, k, v, do, None, None), pairs, B * T, D, H
+    if name == "cfg4":
+        B, H, T, D = 1, 16, 16384, 128
+        q, k, v = rn((B, H, T, D), 0.5), rn((B, H, T, D), 0.5), rn((B, H, T, D), 1.0)
+        # 1% of the key rows of every head get 3*u added, u a seeded unit vector per head
+        n_sel = T // 100
+        for h in range(H):
+            sel = torch.randperm(T, generator=g)[:n_sel].to(device)
+            u = torch.randn(D, generator=g)
+            u = (3.0 * u / u.norm()).to(torch.bfloat16).to(device)
+            k[0, h, sel] += u
+        do = rn((B, H, T, D), 1.0)
+        pairs = B * H * T * (T - 1) // 2
+        desc = {"workload": "cfg4: dense causal fwd+bwd B=1 H=16 T=16384 d=128 bf16, 1% boosted keys",
+                "B": B, "H": H, "T": T, "d": D}
+        return desc, (q, k, v, do, None, None), pairs, B * T, D, H
+    if name == "cfg3":
+        H, N, D = 16, 65536, 64
+        lens = _lognormal_lengths(N, seed=0)
+        cu = [0]
+        for L in lens:
+            cu.append(cu[-1] + L)
+        q, k, v = rn((H, N, D), 0.5), rn((H, N, D), 0.5), rn((H, N, D), 0.5)
+        do = rn((H, N, D), 1.0)
+        pairs = H * sum(L * (L - 1) // 2 for L in lens)
+        cu_t = torch.tensor(cu, dtype=torch.int32, device=device)
+        desc = {"workload": "cfg3: packed varlen fwd+bwd H=16 d=64 bf16, 65536 tokens, lognormal docs",
+                "H": H, "tokens": N, "d": D, "n_docs": len(lens), "max_len": max(lens)}
+        return desc, (q, k, v, do, cu_t, max(lens)), pairs, N, D, H
+    raise SystemExit(f"unknown workload {name}")
+
+
+def cpu_baseline(name, budget_heads=2):
+    """The oracle (a PyTorch restatement of the reference formula) timed on the host cores:
+    fwd+bwd of `budget_heads` heads of the cfg2 problem, scaled to TFLOP/s."""
+    import torch
+    from oracle import sb_oracle as O
+    torch.set_num_threads(min(os.cpu_count() or 1, 16))
+    T, D = 4096, 64
+    g = torch.Generator().manual_seed(1)
+    q, k, v = ((torch.randn(1, budget_heads, T, D, generator=g) * 0.5).to(torch.bfloat16) for _ in range(3))
+    do = torch.randn(1, budget_heads, T, D, generator=g).to(torch.bfloat16)
+    O.sb_attn_grads_oracle(q[:, :1, :512], k[:, :1, :512], v[:, :1, :512], do[:, :1, :512])   # warm-up
+    t0 = time.perf_counter()
+    for h in range(budget_heads):
+        O.sb_attn_grads_oracle(q[:, h:h + 1], k[:, h:h + 1], v[:, h:h + 1], do[:, h:h + 1])
+    dt = time.perf_counter() - t0
+    pairs = budget_heads * T * (T - 1) // 2
+    return {"value": round(12 * D * pairs / dt / 1e12, 5), "unit": "TFLOP/s", "cores": torch.get_num_threads(),
+            "kind": "port",
+            "sample": f"oracle/sb_oracle.py (torch fp32) fwd+bwd of {budget_heads} of 16 heads of cfg2 "
+                      f"(T=4096, d=64), one head at a time, {dt:.2f} s; same 12*d*P FLOP count",
+            "tokens_per_s": round(T / (dt * 16 / budget_heads), 1)}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--workload", default="cfg2", choices=["cfg2", "cfg3", "cfg4"])
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        raise SystemExit("bench.py measures one GPU: the operator has no cross-GPU part "
+                         "(heads and documents shard with no exchange); run with --gpus 1")
+
+    import torch
+    from flame_amd import sb_attn, sb_attn_varlen
+    from flame_amd.stickbreaking_attention import profiling
+
+    dev = torch.device("cuda:0")
+    desc, (q, k, v, do, cu, max_len), pairs, tokens, D, H = make_workload(args.workload, dev)
+    q.requires_grad_(True), k.requires_grad_(True), v.requires_grad_(True)
+
+    def step():
+        q.grad = k.grad = v.grad = None
+        if cu is None:
+            o, _ = sb_attn(q, k, v)
+        else:
+            o, _ = sb_attn_varlen(q, k, v, cu, max_len)
+        torch.autograd.backward([o], [do])
+
+    for _ in range(args.warmup):
+        step()
+    timer = profiling.KernelTimer()
+    profiling.install(timer)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    profiling.install(None)
+
+    ms = dt * 1e3 / args.steps
+    f_fb = 12.0 * D * pairs
+    tflops = f_fb / (ms * 1e-3) / 1e12
+    kern = {name: sum(v_) / len(v_) for name, v_ in timer.durations_ms().items()}
+    # algorithmic FLOPs per launch: each of the three kernels carries two of the six
+    # counted products (4*d*P); recomputed products are not counted
+    per_kernel_flops = 4.0 * D * pairs
+    dom = max(kern, key=kern.get)
+    achieved = per_kernel_flops / (kern[dom] * 1e-3) / 1e12
+    out = {
+        "metric": "sb_attn_fwd_bwd_tflops", "value": round(tflops, 2), "unit": "TFLOP/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms, 4),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16",
+        "data": "synthetic", "config": desc,
+        "pct_of_bf16_mfma_peak": round(100 * tflops / BF16_MFMA_PEAK_TFLOPS, 2),
+        "tokens_per_s": round(tokens / (ms * 1e-3), 1),
+        "flops_convention": "12*d*P, P = allowed (query,key) pairs; recompute not counted",
+        "kernel_ms": {n: round(t, 4) for n, t in kern.items()},
+        "fwd_tflops": round(4.0 * D * pairs / (kern.get("fwd", float("nan")) * 1e-3) / 1e12, 2),
+        "roofline": {"bound": "mfma", "kernel": dom, "achieved": round(achieved, 2),
+                     "peak": BF16_MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
+                     "frac": round(achieved / BF16_MFMA_PEAK_TFLOPS, 4), "traffic": None},
+    }
+    if not args.no_cpu_baseline:
+        out["cpu_baseline"] = cpu_baseline(args.workload)
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

@@ -32,7 +32,7 @@ class SbaParams(C.Structure):
         ("struct_size", C.c_uint32), ("dtype", C.c_int32), ("n_seq", C.c_int32),
         ("n_heads", C.c_int32), ("seq_len", C.c_int32), ("total_tokens", C.c_int32),
         ("head_dim", C.c_int32), ("attend_current", C.c_int32), ("scale", C.c_float),
-        ("save_for_backward", C.c_int32),
+        ("save_for_backward", C.c_int32), ("bwd_phases", C.c_int32),
         ("cu_seqlens", C.c_void_p), ("schedule", C.c_void_p), ("n_schedule", C.c_int32),
         ("q", SbaTensor), ("k", SbaTensor), ("v", SbaTensor), ("o", SbaTensor),
         ("rem", SbaVector), ("d_o", SbaTensor), ("d_rem", SbaVector),

@@ -162,10 +162,13 @@ int sba_bwd(const SbaParams* p) {
     int rc = check_common(p);
     if (rc) return rc;
     if (!p->d_o.ptr || !p->dq.ptr || !p->dk.ptr || !p->dv.ptr) return SBA_ERR_NULL;
+    if (p->bwd_phases < 0 || p->bwd_phases > 2) return SBA_ERR_SHAPE;
     if (!p->workspace || p->workspace_bytes < sba_workspace_bytes(p)) return SBA_ERR_WORKSPACE;
     KParams kp = make_kparams(p);
     hipStream_t s = (hipStream_t)p->stream;
-    return use_mfma_bwd(p) ? sba_launch_mfma_bwd(kp, s) : sba_launch_generic_bwd(kp, p->dtype, s);
+    // the generic backward is one piece: it all runs in phase 1
+    if (!use_mfma_bwd(p) && p->bwd_phases == 2) return SBA_OK;
+    return use_mfma_bwd(p) ? sba_launch_mfma_bwd(kp, p->bwd_phases, s) : sba_launch_generic_bwd(kp, p->dtype, s);
 }
 
 }  // extern "C"

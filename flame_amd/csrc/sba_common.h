@@ -82,5 +82,5 @@ int sba_generic_padded_dim(int D);
 int sba_launch_generic_fwd(const sba::KParams& kp, int dtype, hipStream_t s);
 int sba_launch_generic_bwd(const sba::KParams& kp, int dtype, hipStream_t s);
 int sba_launch_mfma_fwd(const sba::KParams& kp, hipStream_t s);
-int sba_launch_mfma_bwd(const sba::KParams& kp, hipStream_t s);
+int sba_launch_mfma_bwd(const sba::KParams& kp, int phases, hipStream_t s);
 bool sba_mfma_bwd_available();

@@ -264,15 +264,16 @@ __global__ __launch_bounds__(kThreads) void mfma_bwd_dkv_kernel(KParams p) {
 
 bool sba_mfma_bwd_available() { return true; }
 
-int sba_launch_mfma_bwd(const sba::KParams& kp, hipStream_t s) {
+int sba_launch_mfma_bwd(const sba::KParams& kp, int phases, hipStream_t s) {
     using namespace sba;
     dim3 grid((unsigned)kp.n_jobs * kp.n_heads);
+    const bool p1 = phases != 2, p2 = phases != 1;
     if (kp.head_dim == 64) {
-        hipLaunchKernelGGL((mfma_bwd_dq_kernel<64>), grid, dim3(kThreads), 0, s, kp);
-        hipLaunchKernelGGL((mfma_bwd_dkv_kernel<64>), grid, dim3(kThreads), 0, s, kp);
+        if (p1) hipLaunchKernelGGL((mfma_bwd_dq_kernel<64>), grid, dim3(kThreads), 0, s, kp);
+        if (p2) hipLaunchKernelGGL((mfma_bwd_dkv_kernel<64>), grid, dim3(kThreads), 0, s, kp);
     } else {
-        hipLaunchKernelGGL((mfma_bwd_dq_kernel<128>), grid, dim3(kThreads), 0, s, kp);
-        hipLaunchKernelGGL((mfma_bwd_dkv_kernel<128>), grid, dim3(kThreads), 0, s, kp);
+        if (p1) hipLaunchKernelGGL((mfma_bwd_dq_kernel<128>), grid, dim3(kThreads), 0, s, kp);
+        if (p2) hipLaunchKernelGGL((mfma_bwd_dkv_kernel<128>), grid, dim3(kThreads), 0, s, kp);
     }
     return hipGetLastError() == hipSuccess ? SBA_OK : SBA_ERR_LAUNCH;
 }

@@ -1,0 +1,63 @@
+"""Optional per-kernel timing of the operator.
+
+A benchmark installs a ``KernelTimer``; the launch helpers then record an event on the
+launch stream before and after every kernel (the backward is issued as its two kernels,
+one C call each, via SbaParams.bwd_phases).  With no timer installed -- the normal
+case -- nothing is recorded and the backward is a single C call.
+"""
+from __future__ import annotations
+
+import ctypes as C
+from collections import defaultdict
+from typing import Optional
+
+import torch
+
+from .. import _lib
+
+_TIMER: Optional["KernelTimer"] = None
+
+
+class KernelTimer:
+    """Collects (name, start_event, end_event) triples; durations after a synchronize."""
+
+    def __init__(self):
+        self._last = None
+        self._spans = []
+
+    def mark(self, name: str):
+        ev = torch.cuda.Event(enable_timing=True)
+        ev.record()                      # torch's current stream = the stream we launch on
+        if name != "start" and self._last is not None:
+            self._spans.append((name, self._last, ev))
+        self._last = ev
+
+    def durations_ms(self):
+        out = defaultdict(list)
+        for name, a, b in self._spans:
+            out[name].append(a.elapsed_time(b))
+        return dict(out)
+
+
+def install(timer: Optional[KernelTimer]):
+    global _TIMER
+    _TIMER = timer
+
+
+def mark(name: str):
+    if _TIMER is not None:
+        _TIMER.mark(name)
+
+
+def launch_bwd(lib, p):
+    if _TIMER is None:
+        _lib.check(lib.sba_bwd(C.byref(p)), "sba_bwd")
+        return
+    mark("start")
+    p.bwd_phases = 1
+    _lib.check(lib.sba_bwd(C.byref(p)), "sba_bwd")
+    mark("bwd_dq")
+    p.bwd_phases = 2
+    _lib.check(lib.sba_bwd(C.byref(p)), "sba_bwd")
+    mark("bwd_dkv")
+    p.bwd_phases = 0

@@ -13,6 +13,7 @@ import math
 import torch
 
 from .. import _lib
+from . import profiling
 
 
 def _launch_fwd(q, k, v, inv_temp, attend_current, need_grad):
@@ -35,7 +36,9 @@ def _launch_fwd(q, k, v, inv_temp, attend_current, need_grad):
         ws = torch.empty(max(nbytes, 16), dtype=torch.uint8, device=q.device)
         p.workspace, p.workspace_bytes = ws.data_ptr(), nbytes
     p.stream = torch.cuda.current_stream(q.device).cuda_stream
+    profiling.mark("start")
     _lib.check(lib.sba_fwd(C.byref(p)), "sba_fwd")
+    profiling.mark("fwd")
     return o, rem, ws
 
 
@@ -58,7 +61,7 @@ def _launch_bwd(do, drem, q, k, v, ws, inv_temp, attend_current):
     p.dq, p.dk, p.dv = _lib.tensor4(dq), _lib.tensor4(dk), _lib.tensor4(dv)
     p.workspace, p.workspace_bytes = ws.data_ptr(), lib.sba_workspace_bytes(C.byref(p))
     p.stream = torch.cuda.current_stream(q.device).cuda_stream
-    _lib.check(lib.sba_bwd(C.byref(p)), "sba_bwd")
+    profiling.launch_bwd(lib, p)
     return dq, dk, dv
 
 

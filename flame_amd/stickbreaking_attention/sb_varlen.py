@@ -15,6 +15,7 @@ from collections import OrderedDict
 import torch
 
 from .. import _lib
+from . import profiling
 
 _SCHEDULES: "OrderedDict[tuple, tuple]" = OrderedDict()
 _MAX_CACHED = 16
@@ -86,7 +87,9 @@ class StickBreakingAttention(torch.autograd.Function):
                 nbytes = lib.sba_workspace_bytes(C.byref(p))
                 ws = torch.empty(max(nbytes, 16), dtype=torch.uint8, device=q.device)
                 p.workspace, p.workspace_bytes = ws.data_ptr(), nbytes
+            profiling.mark("start")
             _lib.check(lib.sba_fwd(C.byref(p)), "sba_fwd")
+            profiling.mark("fwd")
         if need_grad:
             ctx.save_for_backward(q, k, v, ws, cu_seqlens)
         ctx.logit_scale = inv_temp
@@ -114,7 +117,7 @@ class StickBreakingAttention(torch.autograd.Function):
                 p.d_rem = _lib.SbaVector(drem.data_ptr(), 0, drem.stride(0))
             p.dq, p.dk, p.dv = _lib.tensor3(dq), _lib.tensor3(dk), _lib.tensor3(dv)
             p.workspace, p.workspace_bytes = ws.data_ptr(), lib.sba_workspace_bytes(C.byref(p))
-            _lib.check(lib.sba_bwd(C.byref(p)), "sba_bwd")
+            profiling.launch_bwd(lib, p)
         return dq, dk, dv, None, None, None, None
 
 

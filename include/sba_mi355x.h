@@ -75,6 +75,9 @@ typedef struct SbaParams {
     int32_t  attend_current;   /* 0: keys j < i;  1: keys j <= i */
     float    scale;            /* logit scale ("inv_temp") in natural-log units */
     int32_t  save_for_backward;/* forward only: also fill the carry table in workspace */
+    int32_t  bwd_phases;       /* backward only: 0 = whole backward; 1 = first kernel only (dq and the
+                                  prefix table), 2 = second kernel only (dk, dv; needs phase 1 done on
+                                  the same workspace).  Lets a profiler time the kernels one by one */
 
     const int32_t* cu_seqlens; /* device, n_seq+1 entries, or NULL for dense */
     const int32_t* schedule;   /* device, from sba_build_schedule(); packed layout only */
