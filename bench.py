@@ -81,7 +81,7 @@ def make_workload(name, device):
     raise SystemExit(f"unknown workload {name}")
 
 
-def cpu_baseline(name, budget_heads=2):
+def cpu_baseline(name, budget_heads=16, reps=3):
     """The oracle (a PyTorch restatement of the reference formula) timed on the host cores:
     fwd+bwd of `budget_heads` heads of the cfg2 problem, scaled to TFLOP/s."""
     import torch
@@ -93,15 +93,57 @@ def cpu_baseline(name, budget_heads=2):
     do = torch.randn(1, budget_heads, T, D, generator=g).to(torch.bfloat16)
     O.sb_attn_grads_oracle(q[:, :1, :512], k[:, :1, :512], v[:, :1, :512], do[:, :1, :512])   # warm-up
     t0 = time.perf_counter()
-    for h in range(budget_heads):
-        O.sb_attn_grads_oracle(q[:, h:h + 1], k[:, h:h + 1], v[:, h:h + 1], do[:, h:h + 1])
-    dt = time.perf_counter() - t0
+    for _ in range(reps):
+        for h in range(budget_heads):
+            O.sb_attn_grads_oracle(q[:, h:h + 1], k[:, h:h + 1], v[:, h:h + 1], do[:, h:h + 1])
+    dt = (time.perf_counter() - t0) / reps
     pairs = budget_heads * T * (T - 1) // 2
     return {"value": round(12 * D * pairs / dt / 1e12, 5), "unit": "TFLOP/s", "cores": torch.get_num_threads(),
             "kind": "port",
             "sample": f"oracle/sb_oracle.py (torch fp32) fwd+bwd of {budget_heads} of 16 heads of cfg2 "
-                      f"(T=4096, d=64), one head at a time, {dt:.2f} s; same 12*d*P FLOP count",
+                      f"(T=4096, d=64), one head at a time, {reps} repetitions, {dt:.2f} s each; "
+                      f"same 12*d*P FLOP count",
             "tokens_per_s": round(T / (dt * 16 / budget_heads), 1)}
+
+
+def bench_model(args, dev):
+    """BASELINE config 5: full SBA-340M training step, one packed row of 8192 tokens."""
+    import torch
+    from flame_amd.modeling_sba import SBAConfig, SBAForCausalLM
+    from flame_amd.train_step import make_optimizer, train_step
+    torch.manual_seed(0)
+    cfg = SBAConfig()
+    model = SBAForCausalLM(cfg).to(dev)
+    opt = make_optimizer(model)
+    N = 8192
+    lens = _lognormal_lengths(N, seed=0)
+    cu = [0]
+    for L in lens:
+        cu.append(cu[-1] + L)
+    cu_t = torch.tensor(cu, dtype=torch.int32, device=dev)
+    ids = torch.randint(0, cfg.vocab_size, (1, N), device=dev)
+    for _ in range(args.warmup):
+        train_step(model, opt, ids, ids, cu_t, max(lens))
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        loss, _ = train_step(model, opt, ids, ids, cu_t, max(lens))
+    torch.cuda.synchronize()
+    ms = (time.perf_counter() - t0) * 1e3 / args.steps
+    n_noemb = model.num_parameters(exclude_embeddings=True)
+    # flame's accounting (flame/tools/utils.py:39): 6*(N - N_emb) + 12*l*h*q*t FLOPs per token
+    flops_tok = 6 * n_noemb + 12 * cfg.num_hidden_layers * cfg.num_heads * (cfg.hidden_size // cfg.num_heads) * N
+    out = {
+        "metric": "sba_340m_train_tokens_per_s", "value": round(N / (ms * 1e-3), 1), "unit": "tokens/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms, 3),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": "cfg5: SBA-340M train step (24 layers, hidden 1024, 16x64 heads, MLP 2816, "
+                               "vocab 32000), AdamW, bf16 autocast, one packed varlen row of 8192 tokens",
+                   "params_M": round(model.num_parameters() / 1e6, 1), "n_docs": len(lens), "max_len": max(lens)},
+        "final_loss": round(float(loss), 4),
+        "mfu_flame_convention": round(flops_tok * N / (ms * 1e-3) / 1e12 / BF16_MFMA_PEAK_TFLOPS, 4),
+    }
+    print(json.dumps(out))
 
 
 def main():
@@ -109,7 +151,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--workload", default="cfg2", choices=["cfg2", "cfg3", "cfg4"])
+    ap.add_argument("--workload", default="cfg2", choices=["cfg2", "cfg3", "cfg4", "cfg5"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -121,6 +163,8 @@ def main():
     from flame_amd.stickbreaking_attention import profiling
 
     dev = torch.device("cuda:0")
+    if args.workload == "cfg5":
+        return bench_model(args, dev)
     desc, (q, k, v, do, cu, max_len), pairs, tokens, D, H = make_workload(args.workload, dev)
     q.requires_grad_(True), k.requires_grad_(True), v.requires_grad_(True)
 

@@ -35,8 +35,17 @@ struct KParams {
 
 struct Job { int tok0, len, rb, seq; };
 
-// blockIdx.x = job * n_heads + head.  Dense jobs are generated arithmetically, longest
-// row-blocks first; packed jobs come from the host-built schedule.
+// Workgroup -> (job, head).  blockIdx.x = slot * n_heads + head, so that consecutive
+// workgroups (which the dispatcher deals round-robin to the 8 XCDs) are different heads of
+// the same job and a head stays on one XCD's L2.  Jobs are sorted by decreasing sweep
+// length (longest first); `longest_last` walks the list from its other end (the key-owner
+// pass, whose work grows as the row-block index falls).
+__device__ inline int order_job(int slot, int n_jobs, bool longest_last) {
+    return longest_last ? n_jobs - 1 - slot : slot;
+}
+
+// Dense jobs are generated arithmetically (row-blocks in decreasing order); packed jobs
+// come from the host-built schedule, which has the same order.
 __device__ inline Job decode_job(const KParams& p, int job) {
     Job j;
     if (p.cu_seqlens == nullptr) {

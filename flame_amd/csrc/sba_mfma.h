@@ -152,7 +152,11 @@ __device__ inline void score_tiles(float (&x)[32], const char* ktile, const bf16
 // In-place: x[idx] (base-2 logits, idx = key offset inside this lane's 32 keys; invalid
 // pairs already set to -inf) -> stick-breaking weights of this step, given the carry
 // `R` = product of (1 - beta) over all keys right of this 64-key step.
-//   e = 2^x, u = 1/(1+e);  local chain right-to-left;  one exchange between half-waves.
+//   e = 2^x, u = 1/(1+e) = 1 - beta;  a = beta * (product of u right of the key).
+// e may overflow to +inf for huge logits: then u = 0 and beta = 1 exactly, no NaN, so no
+// clamp is needed; -inf (masked) gives e = 0, u = 1, beta = 0.
+// The chain runs right-to-left inside the lane's 32 keys from 1; one exchange between
+// the half-waves supplies the factor the lower (left) half is missing.
 // Outputs: x[idx] = A (attention weight); beta[idx] when kNeedBeta; R updated to the carry
 // for the next (left) step.
 template <bool kNeedBeta>
@@ -160,11 +164,12 @@ __device__ inline void stick_weights(float (&x)[32], float (&beta)[kNeedBeta ? 3
     float L = 1.0f;
 #pragma unroll
     for (int idx = 31; idx >= 0; --idx) {
-        float e = __builtin_amdgcn_exp2f(fminf(x[idx], kMaxLogit2));
+        float e = __builtin_amdgcn_exp2f(x[idx]);
         float u = __builtin_amdgcn_rcpf(1.0f + e);
+        float b = 1.0f - u;
+        x[idx] = b * L;
         L *= u;
-        x[idx] = e * L;
-        if (kNeedBeta) beta[idx] = e * u;
+        if (kNeedBeta) beta[idx] = b;
     }
     const float other = __shfl_xor(L, 32);
     // upper half-wave holds the right 32 keys: its chain starts from R itself
@@ -172,6 +177,15 @@ __device__ inline void stick_weights(float (&x)[32], float (&beta)[kNeedBeta ? 3
 #pragma unroll
     for (int idx = 0; idx < 32; ++idx) x[idx] *= F;
     R = R * L * other;
+}
+
+// Sets the logits of invisible (query, key) pairs of a diagonal step to -inf.
+__device__ inline void mask_step(float (&x)[32], int key_first, int qi, int strict) {
+    // key_first = first key of this lane's 32; key j visible iff j + strict <= qi
+    const int nvis = qi - strict - key_first + 1;      // visible keys among idx 0..31
+#pragma unroll
+    for (int idx = 0; idx < 32; ++idx)
+        if (idx >= nvis) x[idx] = -INFINITY;
 }
 
 // Transposing fetch from a tile whose rows are in NATURAL order (Q, dO, and the weight
@@ -216,6 +230,8 @@ __device__ inline void dp_tiles(float (&dp)[32], const char* vtile, const bf16x8
 // Gradient of the logits for one step.  In: a[idx] attention weights, beta[idx],
 // dp[idx] = dO.v - drem, Gc = sum of g over all keys LEFT of this step.
 // Out: dp[idx] <- dz = g - beta * prefix_sum(g);  Gc advanced past this step.
+// The inclusive prefix runs left-to-right inside the lane's 32 keys from 0; the upper
+// (right) half-wave then adds the lower half's total.
 __device__ inline void logit_grads(const float (&a)[32], const float (&beta)[32], float (&dp)[32], float& Gc,
                                    int lane) {
     float c = 0.f;
@@ -227,10 +243,9 @@ __device__ inline void logit_grads(const float (&a)[32], const float (&beta)[32]
         pre[idx] = c;
     }
     const float other = __shfl_xor(c, 32);
-    // lower half-wave holds the left 32 keys
     const float F = (lane >= 32) ? Gc + other : Gc;
 #pragma unroll
-    for (int idx = 0; idx < 32; ++idx) dp[idx] = dp[idx] - beta[idx] * (pre[idx] + F);
+    for (int idx = 0; idx < 32; ++idx) dp[idx] = __builtin_fmaf(-beta[idx], pre[idx] + F, dp[idx]);
     Gc = Gc + c + other;
 }
 

@@ -25,10 +25,11 @@ __global__ __launch_bounds__(kThreads) void mfma_bwd_dq_kernel(KParams p) {
     constexpr int kTile = 64 * D * 2;
     __shared__ __attribute__((aligned(16))) char lds[4 * kTile];   // K0 V0 K1 V1
 
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);   // wave-uniform, keep it scalar
     const int n = lane & 31, h = lane >> 5;
     const int head = blockIdx.x % p.n_heads;
-    const Job job = decode_job(p, blockIdx.x / p.n_heads);
+    const Job job = decode_job(p, order_job(blockIdx.x / p.n_heads, p.n_jobs, false));
     const int strict = p.attend_current ? 0 : 1;
     const int m0 = job.rb * kRowBlock;
     const int q0w = m0 + 32 * wave;
@@ -80,11 +81,7 @@ __global__ __launch_bounds__(kThreads) void mfma_bwd_dq_kernel(KParams p) {
             float x[32], beta[32], dp[32];
             score_tiles<D>(x, ktile, qf, p.scale2, lane);
             if (key0 + 63 + strict > q0w) {
-#pragma unroll
-                for (int idx = 0; idx < 32; ++idx) {
-                    int j = key0 + 32 * h + idx;
-                    if (j + strict > qi) x[idx] = -INFINITY;
-                }
+mask_step(x, key0 + 32 * h, qi, strict);
             }
             float R = row_ok ? p.rtab[tix] : 1.0f;
             stick_weights<true>(x, beta, R, lane);
@@ -150,11 +147,12 @@ __global__ __launch_bounds__(kThreads) void mfma_bwd_dkv_kernel(KParams p) {
     char* zp = dotile + kQTile;                // bf16 attention weights
     char* zd = zp + kZTile;                    // bf16 dz
 
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);   // wave-uniform, keep it scalar
     const int n = lane & 31, h = lane >> 5;
     const int head = blockIdx.x % p.n_heads;
     // longest key blocks (leftmost) first: walk the row-block schedule backwards
-    const Job job = decode_job(p, p.n_jobs - 1 - (int)(blockIdx.x / p.n_heads));
+    const Job job = decode_job(p, order_job(blockIdx.x / p.n_heads, p.n_jobs, true));
     const int strict = p.attend_current ? 0 : 1;
     const int64_t qbase = (int64_t)job.seq * p.q.sb + (int64_t)head * p.q.sh + (int64_t)job.tok0 * p.q.st;
     const int64_t kbase = (int64_t)job.seq * p.k.sb + (int64_t)head * p.k.sh + (int64_t)job.tok0 * p.k.st;
@@ -203,11 +201,7 @@ __global__ __launch_bounds__(kThreads) void mfma_bwd_dkv_kernel(KParams p) {
                 float beta[32];
                 score_tiles<D>(x, ktile, qf, p.scale2, lane);
                 if (key0 + 63 + strict > q0w) {
-#pragma unroll
-                    for (int idx = 0; idx < 32; ++idx) {
-                        int j = key0 + 32 * h + idx;
-                        if (j + strict > qi) x[idx] = -INFINITY;
-                    }
+mask_step(x, key0 + 32 * h, qi, strict);
                 }
                 const int64_t tix = ((int64_t)head * p.n_kb + kb) * p.tab_tokens + tab_token(p, job, qi);
                 float R = row_ok ? p.rtab[tix] : 1.0f;

@@ -12,10 +12,11 @@ __global__ __launch_bounds__(kThreads) void mfma_fwd_kernel(KParams p) {
     constexpr int kTile = 64 * D * 2;            // bytes per K or V tile
     __shared__ __attribute__((aligned(16))) char lds[4 * kTile];   // K0 V0 K1 V1
 
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);   // wave-uniform, keep it scalar
     const int n = lane & 31, h = lane >> 5;
     const int head = blockIdx.x % p.n_heads;
-    const Job job = decode_job(p, blockIdx.x / p.n_heads);
+    const Job job = decode_job(p, order_job(blockIdx.x / p.n_heads, p.n_jobs, false));
     const int strict = p.attend_current ? 0 : 1;
     const int m0 = job.rb * kRowBlock;
     const int q0w = m0 + 32 * wave;              // first query of this wave
@@ -61,11 +62,7 @@ __global__ __launch_bounds__(kThreads) void mfma_fwd_kernel(KParams p) {
             float x[32];
             score_tiles<D>(x, ktile, qf, p.scale2, lane);
             if (key0 + 63 + strict > q0w) {     // diagonal region: mask invisible pairs
-#pragma unroll
-                for (int idx = 0; idx < 32; ++idx) {
-                    int j = key0 + 32 * h + idx;
-                    if (j + strict > qi) x[idx] = -INFINITY;
-                }
+mask_step(x, key0 + 32 * h, qi, strict);
             }
             if (p.save && h == 0 && qi < job.len)
                 p.rtab[((int64_t)head * p.n_kb + step) * p.tab_tokens + tabtok] = R;

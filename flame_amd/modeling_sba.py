@@ -1,0 +1,119 @@
+"""SBA language model for the single-GPU training step (BASELINE config 5).
+
+Plain-PyTorch counterpart of custom_models/sba/modeling_sba.py:34-407 and config_sba.py:
+pre-norm blocks [RMSNorm -> SBA -> +res -> RMSNorm -> SwiGLU MLP -> +res]
+(modeling_sba.py:73-90, the non-fused branch :85-88), final norm, untied lm_head, labels
+shifted left by one with the last position ignored (modeling_sba.py:391), mean
+cross-entropy.  The reference builds its norm, MLP and loss from the `fla` package, which
+is not part of the reference tree; the non-fused PyTorch equivalents are used
+(nn.RMSNorm, explicit SwiGLU, F.cross_entropy).  MLP width follows fla's GatedMLP rule
+for hidden_ratio=4: 2/3 * 4 * hidden rounded up to a multiple of 256 (2816 for 1024).
+"""
+from __future__ import annotations
+
+import math
+from dataclasses import dataclass
+from typing import Optional
+
+import torch
+import torch.nn as nn
+import torch.nn.functional as F
+
+from .sba_layer import SBA
+
+
+@dataclass
+class SBAConfig:
+    # defaults = configs/sba_340m.json of the reference
+    hidden_size: int = 1024
+    num_hidden_layers: int = 24
+    num_heads: int = 16
+    hidden_ratio: int = 4
+    intermediate_size: Optional[int] = None
+    initializer_range: float = 0.006
+    norm_eps: float = 1e-6
+    vocab_size: int = 32000
+    qkv_bias: bool = False
+    tie_word_embeddings: bool = False
+
+    def mlp_width(self) -> int:
+        if self.intermediate_size is not None:
+            return self.intermediate_size
+        w = int(self.hidden_size * self.hidden_ratio * 2 / 3)
+        return 256 * ((w + 255) // 256)
+
+
+class SBAMLP(nn.Module):
+    def __init__(self, cfg: SBAConfig):
+        super().__init__()
+        w = cfg.mlp_width()
+        self.gate_proj = nn.Linear(cfg.hidden_size, w, bias=False)
+        self.up_proj = nn.Linear(cfg.hidden_size, w, bias=False)
+        self.down_proj = nn.Linear(w, cfg.hidden_size, bias=False)
+
+    def forward(self, x):
+        return self.down_proj(F.silu(self.gate_proj(x)) * self.up_proj(x))
+
+
+class SBABlock(nn.Module):
+    def __init__(self, cfg: SBAConfig, layer_idx: int):
+        super().__init__()
+        self.attn_norm = nn.RMSNorm(cfg.hidden_size, eps=cfg.norm_eps)
+        self.attn = SBA(hidden_size=cfg.hidden_size, num_heads=cfg.num_heads, qkv_bias=cfg.qkv_bias,
+                        layer_idx=layer_idx)
+        self.mlp_norm = nn.RMSNorm(cfg.hidden_size, eps=cfg.norm_eps)
+        self.mlp = SBAMLP(cfg)
+
+    def forward(self, x, **kwargs):
+        h, _, _ = self.attn(self.attn_norm(x), **kwargs)
+        x = x + h
+        return x + self.mlp(self.mlp_norm(x))
+
+
+class SBAModel(nn.Module):
+    def __init__(self, cfg: SBAConfig):
+        super().__init__()
+        self.embeddings = nn.Embedding(cfg.vocab_size, cfg.hidden_size)
+        self.layers = nn.ModuleList([SBABlock(cfg, i) for i in range(cfg.num_hidden_layers)])
+        self.norm = nn.RMSNorm(cfg.hidden_size, eps=cfg.norm_eps)
+
+    def forward(self, input_ids, **kwargs):
+        x = self.embeddings(input_ids)
+        for layer in self.layers:
+            x = layer(x, **kwargs)
+        return self.norm(x)
+
+
+class SBAForCausalLM(nn.Module):
+    def __init__(self, cfg: SBAConfig):
+        super().__init__()
+        self.config = cfg
+        self.model = SBAModel(cfg)
+        self.lm_head = nn.Linear(cfg.hidden_size, cfg.vocab_size, bias=False)
+        self.apply(self._init_weights)
+        if cfg.tie_word_embeddings:
+            self.lm_head.weight = self.model.embeddings.weight
+
+    def _init_weights(self, m):
+        # modeling_sba.py:120-127: N(0, initializer_range) for Linear and Embedding
+        if isinstance(m, nn.Linear):
+            nn.init.normal_(m.weight, mean=0.0, std=self.config.initializer_range)
+            if m.bias is not None:
+                nn.init.zeros_(m.bias)
+        elif isinstance(m, nn.Embedding):
+            nn.init.normal_(m.weight, mean=0.0, std=self.config.initializer_range)
+
+    def forward(self, input_ids, labels=None, **kwargs):
+        h = self.model(input_ids, **kwargs)
+        logits = self.lm_head(h)
+        loss = None
+        if labels is not None:
+            shifted = torch.cat((labels[..., 1:], torch.full_like(labels[:, :1], -100)), 1)
+            loss = F.cross_entropy(logits.view(shifted.numel(), -1).float(), shifted.view(-1), ignore_index=-100)
+        return loss, logits
+
+    def num_parameters(self, exclude_embeddings=False):
+        n = sum(p.numel() for p in self.parameters())
+        if exclude_embeddings:
+            n -= self.model.embeddings.weight.numel()
+        return n

@@ -19,7 +19,7 @@ from . import profiling
 def _launch_fwd(q, k, v, inv_temp, attend_current, need_grad):
     lib = _lib.load()
     B, H, T, D = q.shape
-    o = torch.empty((B, H, T, D), dtype=q.dtype, device=q.device)
+    o = torch.empty_like(q)          # same strides as q (sb_fwd.py:144 does the same)
     rem = torch.empty((B, H, T), dtype=q.dtype, device=q.device)
     p = _lib.SbaParams()
     p.struct_size = C.sizeof(_lib.SbaParams)
@@ -45,9 +45,7 @@ def _launch_fwd(q, k, v, inv_temp, attend_current, need_grad):
 def _launch_bwd(do, drem, q, k, v, ws, inv_temp, attend_current):
     lib = _lib.load()
     B, H, T, D = q.shape
-    dq, dk, dv = torch.empty_like(q, memory_format=torch.contiguous_format), \
-        torch.empty_like(k, memory_format=torch.contiguous_format), \
-        torch.empty_like(v, memory_format=torch.contiguous_format)
+    dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
     p = _lib.SbaParams()
     p.struct_size = C.sizeof(_lib.SbaParams)
     p.dtype = _lib.dtype_code(q.dtype)

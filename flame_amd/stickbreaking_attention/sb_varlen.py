@@ -75,7 +75,7 @@ class StickBreakingAttention(torch.autograd.Function):
         q, k, v = _lib.usable(q), _lib.usable(k), _lib.usable(v)
         entry = _schedule_for(cu_seqlens)
         H, N, D = q.shape
-        o = torch.empty((H, N, D), dtype=q.dtype, device=q.device)
+        o = torch.empty_like(q)
         rem = torch.empty((H, N), dtype=q.dtype, device=q.device)
         ws = None
         if entry[2] > 0:
@@ -103,9 +103,7 @@ class StickBreakingAttention(torch.autograd.Function):
         lib = _lib.load()
         q, k, v, ws, cu_seqlens = ctx.saved_tensors
         entry = _schedule_for(cu_seqlens)
-        dq = torch.empty_like(q, memory_format=torch.contiguous_format)
-        dk = torch.empty_like(k, memory_format=torch.contiguous_format)
-        dv = torch.empty_like(v, memory_format=torch.contiguous_format)
+        dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
         if entry[2] > 0:
             if do is None:
                 do = torch.zeros_like(q)

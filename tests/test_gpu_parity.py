@@ -216,3 +216,68 @@ def test_row_mass_invariant_at_config2_size():
     # one head against the oracle
     o_ref, rem_ref = O.sb_attn_oracle(q[:, :1].cpu(), k[:, :1].cpu(), v[:, :1].cpu())
     assert max_abs(o[:, :1].float().cpu(), o_ref) <= 2e-2
+
+
+def test_backward_is_bitwise_repeatable_and_matches_generic_path():
+    # the MFMA backward has no atomics: two runs give identical bits; the generic kernels
+    # (a second, independent implementation) agree within the gradient tolerance
+    sb_attn, _ = _ops()
+    q, k, v, do = (randn((1, 4, 600, 64), 90 + i, 0.5, torch.bfloat16).cuda() for i in range(4))
+    drem = randn((1, 4, 600), 95, 1.0, torch.bfloat16).cuda()
+
+    def grads():
+        qq, kk, vv = (x.clone().requires_grad_(True) for x in (q, k, v))
+        o, rem = sb_attn(qq, kk, vv)
+        torch.autograd.backward([o, rem], [do, drem])
+        return qq.grad, kk.grad, vv.grad
+
+    g1, g2 = grads(), grads()
+    assert all(torch.equal(a, b) for a, b in zip(g1, g2))
+    os.environ["SBA_FORCE_GENERIC"] = "1"
+    try:
+        g3 = grads()
+    finally:
+        del os.environ["SBA_FORCE_GENERIC"]
+    for a, b in zip(g1, g3):
+        assert rel_l2(a.float(), b.float()) <= 2e-2
+
+
+def test_sba_model_loss_matches_oracle_attention():
+    # model wiring on the GPU: same weights, HIP operator (bf16 autocast) vs CPU oracle (fp32)
+    from flame_amd.modeling_sba import SBAConfig, SBAForCausalLM
+    cfg = SBAConfig(hidden_size=256, num_hidden_layers=2, num_heads=4, vocab_size=512)
+    torch.manual_seed(0)
+    ref = SBAForCausalLM(cfg)
+    for layer in ref.model.layers:
+        layer.attn.attn_fn = lambda q, k, v, t: O.sb_attn_oracle(q, k, v)
+        layer.attn.attn_varlen_fn = lambda q, k, v, cu, ml: O.sb_attn_varlen_oracle(q, k, v, cu)
+    gpu = SBAForCausalLM(cfg)
+    gpu.load_state_dict(ref.state_dict())
+    gpu.cuda()
+    ids = torch.randint(0, 512, (1, 384))
+    cu = torch.tensor([0, 100, 101, 300, 384], dtype=torch.int32)
+    loss_ref, _ = ref(ids, labels=ids, cu_seqlens=cu)
+    with torch.autocast("cuda", dtype=torch.bfloat16):
+        loss_gpu, _ = gpu(ids.cuda(), labels=ids.cuda(), cu_seqlens=cu.cuda(), max_seqlen=199)
+        loss_dense, _ = gpu(ids.cuda(), labels=ids.cuda())
+    loss_ref_dense, _ = ref(ids, labels=ids)
+    assert abs(float(loss_gpu) - float(loss_ref)) <= 2e-2
+    assert abs(float(loss_dense) - float(loss_ref_dense)) <= 2e-2
+    loss_gpu.backward()
+    assert all(torch.isfinite(p.grad).all() for p in gpu.parameters())
+
+
+def test_sba_340m_width_train_step_runs():
+    # config-5 style step at the 340M width (4 of the 24 layers to keep the test short):
+    # packed varlen row, bf16 autocast, AdamW; loss finite and falling on a repeated batch
+    from flame_amd.modeling_sba import SBAConfig, SBAForCausalLM
+    from flame_amd.train_step import make_optimizer, train_step
+    torch.manual_seed(0)
+    model = SBAForCausalLM(SBAConfig(num_hidden_layers=4)).cuda()
+    opt = make_optimizer(model, lr=1e-3)
+    lens = lognormal_lengths(2048, seed=1)
+    cu = cu_from_lengths(lens).cuda()
+    ids = torch.randint(0, 32000, (1, 2048), device="cuda")
+    losses = [float(train_step(model, opt, ids, ids, cu, max(lens))[0]) for _ in range(4)]
+    print("losses", losses, flush=True)
+    assert all(math.isfinite(x) for x in losses) and losses[-1] < losses[0]

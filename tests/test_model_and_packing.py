@@ -1,0 +1,84 @@
+"""Host-side logic around the operator: the SBA layer/model wiring (with the CPU oracle
+standing in for the HIP operator) and the cu_seqlens convention."""
+import pytest
+import torch
+
+from flame_amd.modeling_sba import SBAConfig, SBAForCausalLM
+from flame_amd.packing import cu_seqlens_from_tokens, split_by_context_len
+from oracle import sb_oracle as O
+
+
+def _oracle_model(cfg, seed=0):
+    torch.manual_seed(seed)
+    m = SBAForCausalLM(cfg)
+    for layer in m.model.layers:
+        layer.attn.attn_fn = lambda q, k, v, t: O.sb_attn_oracle(q, k, v)
+        layer.attn.attn_varlen_fn = lambda q, k, v, cu, ml: O.sb_attn_varlen_oracle(q, k, v, cu)
+    return m
+
+
+def test_340m_config_shape():
+    cfg = SBAConfig()
+    assert (cfg.hidden_size, cfg.num_hidden_layers, cfg.num_heads, cfg.vocab_size) == (1024, 24, 16, 32000)
+    assert cfg.mlp_width() == 2816
+    n = 32000 * 1024 * 2 + 24 * (4 * 1024 * 1024 + 3 * 1024 * 2816 + 2 * 1024) + 1024
+    assert abs(n / 1e6 - 373.9) < 0.1          # ~374 M parameters
+
+
+def test_model_wiring_dense_vs_packed_single_document():
+    cfg = SBAConfig(hidden_size=64, num_hidden_layers=2, num_heads=2, vocab_size=97)
+    m = _oracle_model(cfg)
+    ids = torch.randint(0, 97, (1, 40))
+    loss_dense, logits_dense = m(ids, labels=ids)
+    loss_packed, logits_packed = m(ids, labels=ids, cu_seqlens=torch.tensor([0, 40]))
+    assert torch.allclose(logits_dense, logits_packed, atol=1e-5)
+    assert torch.allclose(loss_dense, loss_packed, atol=1e-6)
+    loss_dense.backward()
+    assert all(torch.isfinite(p.grad).all() for p in m.parameters())
+
+
+def test_packed_documents_do_not_see_each_other():
+    cfg = SBAConfig(hidden_size=64, num_hidden_layers=2, num_heads=2, vocab_size=97)
+    m = _oracle_model(cfg)
+    a, b = torch.randint(0, 97, (1, 17)), torch.randint(0, 97, (1, 23))
+    _, la = m(a)
+    _, lb = m(b)
+    _, lab = m(torch.cat([a, b], 1), cu_seqlens=torch.tensor([0, 17, 40]))
+    assert torch.allclose(lab[:, :17], la, atol=1e-5) and torch.allclose(lab[:, 17:], lb, atol=1e-5)
+
+
+def test_label_shift_ignores_last_position():
+    cfg = SBAConfig(hidden_size=32, num_hidden_layers=1, num_heads=2, vocab_size=11)
+    m = _oracle_model(cfg)
+    ids = torch.randint(0, 11, (2, 9))
+    loss, logits = m(ids, labels=ids)
+    ref = torch.nn.functional.cross_entropy(logits[:, :-1].reshape(-1, 11), ids[:, 1:].reshape(-1))
+    assert torch.allclose(loss, ref, atol=1e-6)
+
+
+def test_kv_heads_must_equal_heads():
+    from flame_amd.sba_layer import SBA
+    with pytest.raises(ValueError):
+        SBA(hidden_size=64, num_heads=4, num_kv_heads=2)
+
+
+def test_cu_seqlens_from_bos():
+    ids = torch.tensor([[1, 5, 6, 1, 7, 1, 8, 9, 9]])
+    assert cu_seqlens_from_tokens(ids, bos_token_id=1).tolist() == [0, 3, 5, 9]
+    # a row that does not start with BOS still starts a document at 0
+    assert cu_seqlens_from_tokens(ids[:, 1:], bos_token_id=1).tolist() == [0, 2, 4, 8]
+    assert cu_seqlens_from_tokens(ids, bos_token_id=1).dtype == torch.int32
+
+
+def test_cu_seqlens_from_eos():
+    ids = torch.tensor([5, 6, 2, 7, 2, 8, 9])
+    assert cu_seqlens_from_tokens(ids, eos_token_id=2).tolist() == [0, 3, 5, 7]
+    assert cu_seqlens_from_tokens(torch.tensor([5, 6, 2]), eos_token_id=2).tolist() == [0, 3]
+    with pytest.raises(ValueError):
+        cu_seqlens_from_tokens(ids)
+
+
+def test_context_len_rechunking():
+    cu = torch.tensor([0, 10, 13, 30], dtype=torch.int32)
+    assert split_by_context_len(cu, 8).tolist() == [0, 8, 10, 13, 21, 29, 30]
+    assert cu_seqlens_from_tokens(torch.tensor([1] + [3] * 19), bos_token_id=1, context_len=8).tolist() == [0, 8, 16, 20]
