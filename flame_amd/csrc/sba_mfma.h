@@ -135,18 +135,34 @@ __device__ inline f32x16 mfma(bf16x8 a, bf16x8 b, f32x16 c) {
     return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
 }
 
-// S^T tile pair for one wave: x[16*t + r] = scale2 * (K Q^T)[key_local = 32h+16t+r][query n].
+// S^T tile pair for one wave, raw MFMA accumulators (no vector-ALU instruction touches
+// them here, so the matrix cores run ahead of whatever vector work follows):
+// raw[t][r] = (K Q^T)[key_local = 32h + 16t + r][query n].
 template <int D>
-__device__ inline void score_tiles(float (&x)[32], const char* ktile, const bf16x8 (&qf)[D / 16],
-                                   float scale2, int lane) {
+__device__ inline void score_raw(f32x16 (&raw)[2], const char* ktile, const bf16x8 (&qf)[D / 16], int lane) {
 #pragma unroll
     for (int t = 0; t < 2; ++t) {
         f32x16 acc = {0};
 #pragma unroll
         for (int ks = 0; ks < D / 16; ++ks) acc = mfma(fetch_rows<D>(ktile, t, ks, lane), qf[ks], acc);
-#pragma unroll
-        for (int r = 0; r < 16; ++r) x[16 * t + r] = acc[r] * scale2;
+        raw[t] = acc;
     }
+}
+
+// base-2 logits from the raw accumulators: x[16*t + r] = scale2 * raw[t][r].
+__device__ inline void scale_scores(float (&x)[32], const f32x16 (&raw)[2], float scale2) {
+#pragma unroll
+    for (int t = 0; t < 2; ++t)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) x[16 * t + r] = raw[t][r] * scale2;
+}
+
+template <int D>
+__device__ inline void score_tiles(float (&x)[32], const char* ktile, const bf16x8 (&qf)[D / 16],
+                                   float scale2, int lane) {
+    f32x16 raw[2];
+    score_raw<D>(raw, ktile, qf, lane);
+    scale_scores(x, raw, scale2);
 }
 
 // In-place: x[idx] (base-2 logits, idx = key offset inside this lane's 32 keys; invalid
@@ -230,23 +246,41 @@ __device__ inline void dp_tiles(float (&dp)[32], const char* vtile, const bf16x8
 // Gradient of the logits for one step.  In: a[idx] attention weights, beta[idx],
 // dp[idx] = dO.v - drem, Gc = sum of g over all keys LEFT of this step.
 // Out: dp[idx] <- dz = g - beta * prefix_sum(g);  Gc advanced past this step.
-// The inclusive prefix runs left-to-right inside the lane's 32 keys from 0; the upper
-// (right) half-wave then adds the lower half's total.
+// The inclusive prefix runs left-to-right inside the lane's 32 keys; the upper (right)
+// half-wave adds the lower half's total.  kLowReg trades one more add per element for
+// not keeping the 32 prefix values alive (two passes: sum, then running prefix).
+template <bool kLowReg>
 __device__ inline void logit_grads(const float (&a)[32], const float (&beta)[32], float (&dp)[32], float& Gc,
                                    int lane) {
     float c = 0.f;
-    float pre[32];
+    if (kLowReg) {
 #pragma unroll
-    for (int idx = 0; idx < 32; ++idx) {
-        dp[idx] = a[idx] * dp[idx];     // g
-        c += dp[idx];
-        pre[idx] = c;
+        for (int idx = 0; idx < 32; ++idx) {
+            dp[idx] = a[idx] * dp[idx];     // g
+            c += dp[idx];
+        }
+        const float other = __shfl_xor(c, 32);
+        float run = (lane >= 32) ? Gc + other : Gc;
+#pragma unroll
+        for (int idx = 0; idx < 32; ++idx) {
+            run += dp[idx];
+            dp[idx] = __builtin_fmaf(-beta[idx], run, dp[idx]);
+        }
+        Gc = Gc + c + other;
+    } else {
+        float pre[32];
+#pragma unroll
+        for (int idx = 0; idx < 32; ++idx) {
+            dp[idx] = a[idx] * dp[idx];     // g
+            c += dp[idx];
+            pre[idx] = c;
+        }
+        const float other = __shfl_xor(c, 32);
+        const float F = (lane >= 32) ? Gc + other : Gc;
+#pragma unroll
+        for (int idx = 0; idx < 32; ++idx) dp[idx] = __builtin_fmaf(-beta[idx], pre[idx] + F, dp[idx]);
+        Gc = Gc + c + other;
     }
-    const float other = __shfl_xor(c, 32);
-    const float F = (lane >= 32) ? Gc + other : Gc;
-#pragma unroll
-    for (int idx = 0; idx < 32; ++idx) dp[idx] = __builtin_fmaf(-beta[idx], pre[idx] + F, dp[idx]);
-    Gc = Gc + c + other;
 }
 
 }  // namespace sba

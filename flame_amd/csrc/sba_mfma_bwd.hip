@@ -87,7 +87,7 @@ mask_step(x, key0 + 32 * h, qi, strict);
             stick_weights<true>(x, beta, R, lane);
             dp_tiles<D>(dp, vtile, dof, dr, lane);
             if (row_ok && h == 0) p.gtab[tix] = Gc;
-            logit_grads(x, beta, dp, Gc, lane);
+            logit_grads<false>(x, beta, dp, Gc, lane);
             bf16x8 zf[4];
 #pragma unroll
             for (int c = 0; c < 4; ++c) zf[c] = pack8(&dp[8 * c]);
@@ -135,7 +135,7 @@ __device__ inline void copy_rows_nat(char* tile, const TensorArg& t, int64_t bas
 }
 
 template <int D>
-__global__ __launch_bounds__(kThreads) void mfma_bwd_dkv_kernel(KParams p) {
+__global__ __launch_bounds__(kThreads) void mfma_bwd_dkv_shared_kernel(KParams p) {
     constexpr int kTile = 64 * D * 2;          // K or V tile (64 keys)
     constexpr int kQTile = 128 * D * 2;        // Q or dO tile (128 queries)
     constexpr int kZTile = 128 * 64 * 2;       // weights of one step, [query][key] bf16
@@ -211,7 +211,7 @@ mask_step(x, key0 + 32 * h, qi, strict);
                     dr = Elem<uint16_t>::load(p.d_rem.ptr, (int64_t)job.seq * p.d_rem.sb + (int64_t)head * p.d_rem.sh + job.tok0 + qi);
                 stick_weights<true>(x, beta, R, lane);
                 dp_tiles<D>(dp, vtile, dof, dr, lane);
-                logit_grads(x, beta, dp, Gc, lane);
+                logit_grads<false>(x, beta, dp, Gc, lane);
             } else {
 #pragma unroll
                 for (int idx = 0; idx < 32; ++idx) { x[idx] = 0.f; dp[idx] = 0.f; }
@@ -254,6 +254,192 @@ mask_step(x, key0 + 32 * h, qi, strict);
     }
 }
 
+// ---------------------------------------------------------------- pass 2, head_dim 64
+// Wave-private variant: every wave reduces over its OWN 32 queries of each step, so the
+// sweep has no workgroup barrier at all.  Per step a wave
+//   * copies its 32 rows of Q and dO (prefetched one step ahead) into its LDS slice,
+//   * computes S^T and dP^T for the 64 owned keys, the weights a and dz,
+//   * writes a, dz as bf16 [query][key] rows into its LDS slice and reads them back
+//     transposed (ds_read_b64_tr_b16) as the A operands of
+//         dK[key][d] += dz^T Q,   dV[key][d] += a^T dO        (K dimension = its 32 queries)
+//     with Q, dO read transposed from the same slice as B operands.
+// The four partial dK/dV accumulators of the workgroup are summed through LDS once per
+// 64-key block.
+__device__ inline void wave_rows_load(u32x4 (&r)[4], const TensorArg& t, int64_t base, int row0, int len, int lane) {
+    // 32 rows x 64 bf16 = 256 chunks of 16 bytes; lane takes chunks lane + 64*i
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        int cid = lane + 64 * i;
+        int row = row0 + (cid >> 3), c = cid & 7;
+        u32x4 v = {0u, 0u, 0u, 0u};
+        if (row < len) v = *(const u32x4*)(t.ptr + 2 * (base + (int64_t)row * t.st + c * 8));
+        r[i] = v;
+    }
+}
+__device__ inline void wave_rows_store(char* buf, const u32x4 (&r)[4], int lane) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        int cid = lane + 64 * i;
+        *(u32x4*)(buf + tile_offset<64>(cid >> 3, cid & 7)) = r[i];
+    }
+}
+
+__global__ __launch_bounds__(kThreads) void mfma_bwd_dkv64_kernel(KParams p) {
+    constexpr int D = 64;
+    constexpr int kTile = 64 * D * 2;          // 8 KB: K or V tile (64 keys)
+    constexpr int kSlice = 32 * 64 * 2;        // 4 KB: 32 rows x 64 bf16
+    // K V | per wave: Q dO Zp Zd  (4 x 16 KB)
+    __shared__ __attribute__((aligned(16))) char lds[2 * kTile + 4 * 4 * kSlice];
+    char* ktile = lds;
+    char* vtile = lds + kTile;
+
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int n = lane & 31, h = lane >> 5;
+    char* qbuf = lds + 2 * kTile + wave * 4 * kSlice;
+    char* dobuf = qbuf + kSlice;
+    char* zp = dobuf + kSlice;
+    char* zd = zp + kSlice;
+    const int head = blockIdx.x % p.n_heads;
+    const Job job = decode_job(p, order_job(blockIdx.x / p.n_heads, p.n_jobs, true));
+    const int strict = p.attend_current ? 0 : 1;
+    const int64_t qbase = (int64_t)job.seq * p.q.sb + (int64_t)head * p.q.sh + (int64_t)job.tok0 * p.q.st;
+    const int64_t kbase = (int64_t)job.seq * p.k.sb + (int64_t)head * p.k.sh + (int64_t)job.tok0 * p.k.st;
+    const int64_t vbase = (int64_t)job.seq * p.v.sb + (int64_t)head * p.v.sh + (int64_t)job.tok0 * p.v.st;
+    const int64_t dobase = (int64_t)job.seq * p.d_o.sb + (int64_t)head * p.d_o.sh + (int64_t)job.tok0 * p.d_o.st;
+    const int n_qb = (job.len + kRowBlock - 1) / kRowBlock;
+
+    for (int half = 0; half < 2; ++half) {
+        const int kb = 2 * job.rb + half;
+        const int key0 = kb * kKeyBlock;
+        if (key0 >= job.len) break;            // uniform over the workgroup
+
+        __syncthreads();                       // previous half's reduction is done with the LDS
+        {
+            TileCopy<D> kc, vc;
+            kc.load(p.k, kbase, key0, job.len);
+            vc.load(p.v, vbase, key0, job.len);
+            kc.store(ktile);
+            vc.store(vtile);
+        }
+        __syncthreads();
+
+        f32x16 dkacc[2][2], dvacc[2][2];       // [key half][d block]
+#pragma unroll
+        for (int a = 0; a < 2; ++a)
+#pragma unroll
+            for (int b = 0; b < 2; ++b) { dkacc[a][b] = f32x16{0}; dvacc[a][b] = f32x16{0}; }
+
+        // first query this wave ever needs: rows of the diagonal block at or right of the keys
+        const int qb0 = job.rb;
+        u32x4 qr[4], dor[4];
+        wave_rows_load(qr, p.q, qbase, qb0 * kRowBlock + 32 * wave, job.len, lane);
+        wave_rows_load(dor, p.d_o, dobase, qb0 * kRowBlock + 32 * wave, job.len, lane);
+
+        for (int qb = qb0; qb < n_qb; ++qb) {
+            const int q0w = qb * kRowBlock + 32 * wave;
+            const int qi = q0w + n;
+            const bool row_ok = qi < job.len;
+            // this wave's rows of the step: registers -> LDS slice; prefetch the next step's
+            wave_rows_store(qbuf, qr, lane);
+            wave_rows_store(dobuf, dor, lane);
+            if (qb + 1 < n_qb) {
+                wave_rows_load(qr, p.q, qbase, q0w + kRowBlock, job.len, lane);
+                wave_rows_load(dor, p.d_o, dobase, q0w + kRowBlock, job.len, lane);
+            }
+            if (key0 + strict > q0w + 31 || q0w >= job.len) continue;   // nothing visible / no rows
+
+            bf16x8 qf[D / 16], dof[D / 16];
+#pragma unroll
+            for (int ks = 0; ks < D / 16; ++ks) {
+                qf[ks] = fetch_row_nat<D>(qbuf, n, ks, lane);
+                dof[ks] = fetch_row_nat<D>(dobuf, n, ks, lane);
+            }
+            float x[32], beta[32], dp[32];
+            score_tiles<D>(x, ktile, qf, p.scale2, lane);
+            if (key0 + 63 + strict > q0w) mask_step(x, key0 + 32 * h, qi, strict);
+            const int64_t tix = ((int64_t)head * p.n_kb + kb) * p.tab_tokens + tab_token(p, job, qi);
+            float R = row_ok ? p.rtab[tix] : 1.0f;
+            float Gc = row_ok ? p.gtab[tix] : 0.0f;
+            float dr = 0.f;
+            if (row_ok && p.d_rem.ptr)
+                dr = Elem<uint16_t>::load(p.d_rem.ptr, (int64_t)job.seq * p.d_rem.sb + (int64_t)head * p.d_rem.sh + job.tok0 + qi);
+            stick_weights<true>(x, beta, R, lane);
+            dp_tiles<D>(dp, vtile, dof, dr, lane);
+            logit_grads<true>(x, beta, dp, Gc, lane);
+            // row n of the [query][key] slices: keys 32*h .. 32*h+31
+#pragma unroll
+            for (int c = 0; c < 4; ++c) {
+                *(bf16x8*)(zp + tile_offset<64>(n, 4 * h + c)) = pack8(&x[8 * c]);
+                *(bf16x8*)(zd + tile_offset<64>(n, 4 * h + c)) = pack8(&dp[8 * c]);
+            }
+            // same wave wrote and reads: the compiler's lgkmcnt wait orders it
+#pragma unroll
+            for (int c2 = 0; c2 < 2; ++c2) {
+                bf16x8 bq[2], bdo[2];
+#pragma unroll
+                for (int db = 0; db < 2; ++db) {
+                    bq[db] = fetch_cols_nat<64>(qbuf, 16 * c2, db, lane);
+                    bdo[db] = fetch_cols_nat<64>(dobuf, 16 * c2, db, lane);
+                }
+#pragma unroll
+                for (int kh = 0; kh < 2; ++kh) {
+                    bf16x8 az = fetch_cols_nat<64>(zd, 16 * c2, kh, lane);
+                    bf16x8 ap = fetch_cols_nat<64>(zp, 16 * c2, kh, lane);
+#pragma unroll
+                    for (int db = 0; db < 2; ++db) {
+                        dkacc[kh][db] = mfma(az, bq[db], dkacc[kh][db]);
+                        dvacc[kh][db] = mfma(ap, bdo[db], dvacc[kh][db]);
+                    }
+                }
+            }
+        }
+
+        // ---- sum the four waves' partial tiles through LDS and store.
+        // accumulator layout: lane (n = d within its block, h), register r ->
+        // key 32*kh + 8*(r/4) + 4*h + r%4.  Reduction buffer: [wave][key 64][d 64] fp32 = 16 KB
+        // per wave, reusing the per-wave slices (dK first, then dV).
+        float* red = (float*)(lds + 2 * kTile);
+#pragma unroll
+        for (int which = 0; which < 2; ++which) {
+            __syncthreads();
+#pragma unroll
+            for (int kh = 0; kh < 2; ++kh)
+#pragma unroll
+                for (int db = 0; db < 2; ++db)
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) {
+                        int key = 32 * kh + 8 * (r >> 2) + 4 * h + (r & 3);
+                        float v = which == 0 ? dkacc[kh][db][r] : dvacc[kh][db][r];
+                        red[(wave * 64 + key) * 64 + 32 * db + n] = v;
+                    }
+            __syncthreads();
+            const TensorArg& out = which == 0 ? p.dk : p.dv;
+            const float mul = which == 0 ? p.scale : 1.0f;
+            // 64 x 64 outputs, 256 threads: thread -> (key = tid/4, 16 consecutive d)
+            const int key = threadIdx.x >> 2, d0 = (threadIdx.x & 3) * 16;
+            if (key0 + key < job.len) {
+                const int64_t ob = (int64_t)job.seq * out.sb + (int64_t)head * out.sh + (int64_t)(job.tok0 + key0 + key) * out.st + d0;
+                uint32_t w[8];
+#pragma unroll
+                for (int j = 0; j < 16; j += 2) {
+                    float s0 = 0.f, s1 = 0.f;
+#pragma unroll
+                    for (int wv = 0; wv < 4; ++wv) {
+                        s0 += red[(wv * 64 + key) * 64 + d0 + j];
+                        s1 += red[(wv * 64 + key) * 64 + d0 + j + 1];
+                    }
+                    f32x2 pr = {s0 * mul, s1 * mul};
+                    w[j >> 1] = __builtin_bit_cast(uint32_t, __builtin_convertvector(pr, bf16x2));
+                }
+                u32x4* dst = (u32x4*)(out.ptr + 2 * ob);
+                dst[0] = u32x4{w[0], w[1], w[2], w[3]};
+                dst[1] = u32x4{w[4], w[5], w[6], w[7]};
+            }
+        }
+    }
+}
+
 }  // namespace sba
 
 bool sba_mfma_bwd_available() { return true; }
@@ -264,10 +450,10 @@ int sba_launch_mfma_bwd(const sba::KParams& kp, int phases, hipStream_t s) {
     const bool p1 = phases != 2, p2 = phases != 1;
     if (kp.head_dim == 64) {
         if (p1) hipLaunchKernelGGL((mfma_bwd_dq_kernel<64>), grid, dim3(kThreads), 0, s, kp);
-        if (p2) hipLaunchKernelGGL((mfma_bwd_dkv_kernel<64>), grid, dim3(kThreads), 0, s, kp);
+        if (p2) hipLaunchKernelGGL(mfma_bwd_dkv64_kernel, grid, dim3(kThreads), 0, s, kp);
     } else {
         if (p1) hipLaunchKernelGGL((mfma_bwd_dq_kernel<128>), grid, dim3(kThreads), 0, s, kp);
-        if (p2) hipLaunchKernelGGL((mfma_bwd_dkv_kernel<128>), grid, dim3(kThreads), 0, s, kp);
+        if (p2) hipLaunchKernelGGL((mfma_bwd_dkv_shared_kernel<128>), grid, dim3(kThreads), 0, s, kp);
     }
     return hipGetLastError() == hipSuccess ? SBA_OK : SBA_ERR_LAUNCH;
 }
