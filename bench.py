@@ -151,7 +151,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--workload", default="cfg2", choices=["cfg2", "cfg3", "cfg4", "cfg5"])
+    ap.add_argument("--workload", default="cfg2", choices=["cfg2", "cfg3", "cfg4", "cfg5", "copy"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -165,6 +165,16 @@ def main():
     dev = torch.device("cuda:0")
     if args.workload == "cfg5":
         return bench_model(args, dev)
+    if args.workload == "copy":
+        # plain 256 MiB device copy: the known-size kernel that the FETCH_SIZE / WRITE_SIZE
+        # counters of a profile are scaled by
+        src = torch.empty(256 << 20, dtype=torch.uint8, device=dev)
+        dst = torch.empty_like(src)
+        for _ in range(args.warmup + args.steps):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        print(json.dumps({"workload": "copy", "bytes_read": 256 << 20, "bytes_written": 256 << 20}))
+        return
     desc, (q, k, v, do, cu, max_len), pairs, tokens, D, H = make_workload(args.workload, dev)
     q.requires_grad_(True), k.requires_grad_(True), v.requires_grad_(True)
 
