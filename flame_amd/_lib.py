@@ -105,6 +105,8 @@ def tensor3(t: torch.Tensor) -> SbaTensor:
 
 def usable(t: torch.Tensor) -> torch.Tensor:
     """Kernels need unit stride along D and 16-byte aligned rows; copy otherwise."""
+    if torch.compiler.is_compiling():
+        return t.contiguous()            # no data_ptr() on traced tensors
     ok = t.stride(-1) == 1 and t.data_ptr() % 16 == 0
     if ok:
         per16 = 16 // t.element_size()
@@ -123,3 +125,14 @@ def build_schedule(cu_host: torch.Tensor) -> torch.Tensor:
     got = lib.sba_build_schedule(ptr, n_seq, C.cast(out.data_ptr(), C.POINTER(C.c_int32)), n)
     assert got == n
     return out[:n]
+
+
+def workspace_upper_bound(n_heads: int, seq_len: int, tab_tokens: int, head_dim: int) -> int:
+    """Pure-Python bound on sba_workspace_bytes() (both carry tables plus the generic
+    path's fp32 accumulators), usable while torch.compile traces, where no ctypes call can
+    be made.  Always >= what the library asks for."""
+    def up(x):
+        return (x + 255) & ~255
+    n_kb = (seq_len + 63) // 64
+    dp = 32 if head_dim <= 32 else (64 if head_dim <= 64 else 128)
+    return 2 * up(n_heads * n_kb * tab_tokens * 4) + up(2 * tab_tokens * n_heads * dp * 4)

@@ -9,43 +9,17 @@ from __future__ import annotations
 
 import ctypes as C
 import math
+from typing import Optional
 
 import torch
 
 from .. import _lib
 from . import profiling
+from .utils import custom_op
 
 
-def _launch_fwd(q, k, v, inv_temp, attend_current, need_grad):
-    lib = _lib.load()
+def _params(q, k, v, inv_temp, attend_current):
     B, H, T, D = q.shape
-    o = torch.empty_like(q)          # same strides as q (sb_fwd.py:144 does the same)
-    rem = torch.empty((B, H, T), dtype=q.dtype, device=q.device)
-    p = _lib.SbaParams()
-    p.struct_size = C.sizeof(_lib.SbaParams)
-    p.dtype = _lib.dtype_code(q.dtype)
-    p.n_seq, p.n_heads, p.seq_len, p.total_tokens, p.head_dim = B, H, T, T, D
-    p.attend_current = int(bool(attend_current))
-    p.scale = float(inv_temp)
-    p.save_for_backward = int(need_grad)
-    p.q, p.k, p.v, p.o = _lib.tensor4(q), _lib.tensor4(k), _lib.tensor4(v), _lib.tensor4(o)
-    p.rem = _lib.SbaVector(rem.data_ptr(), rem.stride(0), rem.stride(1))
-    ws = None
-    if need_grad:
-        nbytes = lib.sba_workspace_bytes(C.byref(p))
-        ws = torch.empty(max(nbytes, 16), dtype=torch.uint8, device=q.device)
-        p.workspace, p.workspace_bytes = ws.data_ptr(), nbytes
-    p.stream = torch.cuda.current_stream(q.device).cuda_stream
-    profiling.mark("start")
-    _lib.check(lib.sba_fwd(C.byref(p)), "sba_fwd")
-    profiling.mark("fwd")
-    return o, rem, ws
-
-
-def _launch_bwd(do, drem, q, k, v, ws, inv_temp, attend_current):
-    lib = _lib.load()
-    B, H, T, D = q.shape
-    dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
     p = _lib.SbaParams()
     p.struct_size = C.sizeof(_lib.SbaParams)
     p.dtype = _lib.dtype_code(q.dtype)
@@ -53,13 +27,61 @@ def _launch_bwd(do, drem, q, k, v, ws, inv_temp, attend_current):
     p.attend_current = int(bool(attend_current))
     p.scale = float(inv_temp)
     p.q, p.k, p.v = _lib.tensor4(q), _lib.tensor4(k), _lib.tensor4(v)
-    p.d_o = _lib.tensor4(do)
-    if drem is not None:
-        p.d_rem = _lib.SbaVector(drem.data_ptr(), drem.stride(0), drem.stride(1))
-    p.dq, p.dk, p.dv = _lib.tensor4(dq), _lib.tensor4(dk), _lib.tensor4(dv)
-    p.workspace, p.workspace_bytes = ws.data_ptr(), lib.sba_workspace_bytes(C.byref(p))
     p.stream = torch.cuda.current_stream(q.device).cuda_stream
+    return p
+
+
+def workspace_bytes(q, inv_temp=1.0) -> int:
+    if torch.compiler.is_compiling():
+        B, H, T, D = q.shape
+        return _lib.workspace_upper_bound(H, T, B * T, D)
+    return int(_lib.load().sba_workspace_bytes(C.byref(_params(q, q, q, inv_temp, False))))
+
+
+# Same registered names as the reference (sb_fwd.py:177, sb_bwd.py:207); outputs are
+# allocated by the caller and mutated, as there.
+@custom_op("attn_fwd", mutates_args=("o", "rem", "ws"))
+def _compileable_fwd(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, logit_scale: float,
+                     attend_current: bool, save: bool, o: torch.Tensor, rem: torch.Tensor,
+                     ws: torch.Tensor) -> None:
+    lib = _lib.load()
+    p = _params(q, k, v, logit_scale, attend_current)
+    p.o = _lib.tensor4(o)
+    p.rem = _lib.SbaVector(rem.data_ptr(), rem.stride(0), rem.stride(1))
+    p.save_for_backward = int(save)
+    if save:
+        p.workspace, p.workspace_bytes = ws.data_ptr(), ws.numel()
+    profiling.mark("start")
+    _lib.check(lib.sba_fwd(C.byref(p)), "sba_fwd")
+    profiling.mark("fwd")
+
+
+@custom_op("attn_bwd", mutates_args=("dq", "dk", "dv", "ws"))
+def _compileable_backward(do: torch.Tensor, dr: Optional[torch.Tensor], q: torch.Tensor, k: torch.Tensor,
+                          v: torch.Tensor, ws: torch.Tensor, logit_scale: float, attend_current: bool,
+                          dq: torch.Tensor, dk: torch.Tensor, dv: torch.Tensor) -> None:
+    lib = _lib.load()
+    p = _params(q, k, v, logit_scale, attend_current)
+    p.d_o = _lib.tensor4(do)
+    if dr is not None:
+        p.d_rem = _lib.SbaVector(dr.data_ptr(), dr.stride(0), dr.stride(1))
+    p.dq, p.dk, p.dv = _lib.tensor4(dq), _lib.tensor4(dk), _lib.tensor4(dv)
+    p.workspace, p.workspace_bytes = ws.data_ptr(), ws.numel()
     profiling.launch_bwd(lib, p)
+
+
+def _fwd(q, k, v, logit_scale, attend_current=False, no_grad=False):
+    o = torch.empty_like(q)              # same strides as q (sb_fwd.py:144 does the same)
+    rem = torch.empty(q.shape[:-1], dtype=q.dtype, device=q.device)
+    nbytes = 16 if no_grad else max(workspace_bytes(q), 16)
+    ws = torch.empty(nbytes, dtype=torch.uint8, device=q.device)
+    _compileable_fwd(q, k, v, float(logit_scale), bool(attend_current), not no_grad, o, rem, ws)
+    return o, rem, ws
+
+
+def _bwd(do, dr, q, k, v, ws, logit_scale, attend_current=False):
+    dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+    _compileable_backward(do, dr, q, k, v, ws, float(logit_scale), bool(attend_current), dq, dk, dv)
     return dq, dk, dv
 
 
@@ -75,11 +97,10 @@ class StickBreakingAttention(torch.autograd.Function):
             raise TypeError("q, k, v must share a dtype")
         if not (q.shape == k.shape == v.shape) or q.dim() != 4:
             raise ValueError("q, k, v must all be [B, H, T, D]")
-        need_grad = any(ctx.needs_input_grad[:3])
+        no_grad = not any(ctx.needs_input_grad[:3])
         q, k, v = _lib.usable(q), _lib.usable(k), _lib.usable(v)
-        o, rem, ws = _launch_fwd(q, k, v, inv_temp, attend_current, need_grad)
-        if need_grad:
-            ctx.save_for_backward(q, k, v, ws)
+        o, rem, ws = _fwd(q, k, v, inv_temp, attend_current, no_grad)
+        ctx.save_for_backward(q, k, v, ws)
         ctx.logit_scale = inv_temp
         ctx.attend_current = attend_current
         ctx.set_materialize_grads(False)
@@ -93,7 +114,7 @@ class StickBreakingAttention(torch.autograd.Function):
         do = _lib.usable(do)
         if drem is not None:
             drem = drem.contiguous()
-        dq, dk, dv = _launch_bwd(do, drem, q, k, v, ws, ctx.logit_scale, ctx.attend_current)
+        dq, dk, dv = _bwd(do, drem, q, k, v, ws, ctx.logit_scale, ctx.attend_current)
         return dq, dk, dv, None, None
 
 

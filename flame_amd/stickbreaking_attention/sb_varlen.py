@@ -10,25 +10,27 @@ from __future__ import annotations
 
 import ctypes as C
 import math
-from collections import OrderedDict
+import weakref
+from typing import Optional
 
 import torch
 
 from .. import _lib
 from . import profiling
+from .utils import custom_op
 
-_SCHEDULES: "OrderedDict[tuple, tuple]" = OrderedDict()
-_MAX_CACHED = 16
+# Schedules are cached per cu_seqlens TENSOR OBJECT (identity + version counter), so the 24
+# layers of a model that receive the same tensor share one host sync; a data_ptr-based key
+# would be unsafe because the caching allocator reuses addresses.
+_SCHEDULES: dict = {}
 
 
 def _schedule_for(cu_seqlens: torch.Tensor):
     """(cu int32 on device with leading 0, schedule on device, n_jobs, max_len, total)."""
-    key = (cu_seqlens.data_ptr(), cu_seqlens.numel(), str(cu_seqlens.device), cu_seqlens._version,
-           cu_seqlens.dtype)
+    key = id(cu_seqlens)
     hit = _SCHEDULES.get(key)
-    if hit is not None:
-        _SCHEDULES.move_to_end(key)
-        return hit
+    if hit is not None and hit[0]() is cu_seqlens and hit[1] == cu_seqlens._version:
+        return hit[2]
     cu_host = cu_seqlens.detach().to("cpu", torch.int32)   # one host sync per new packing
     if cu_host.numel() < 2 or int(cu_host[0]) != 0:
         raise ValueError("cu_seqlens must start with 0 and hold at least one document")
@@ -38,27 +40,94 @@ def _schedule_for(cu_seqlens: torch.Tensor):
     sched = _lib.build_schedule(cu_host)
     dev = cu_seqlens.device
     entry = (cu_host.to(dev), sched.to(dev), sched.shape[0], int(lens.max()), int(cu_host[-1]))
-    _SCHEDULES[key] = entry
-    while len(_SCHEDULES) > _MAX_CACHED:
-        _SCHEDULES.popitem(last=False)
+    ref = weakref.ref(cu_seqlens, lambda _r, key=key: _SCHEDULES.pop(key, None))
+    _SCHEDULES[key] = (ref, cu_seqlens._version, entry)
     return entry
 
 
-def _params(q, k, v, sched_entry, inv_temp, attend_current):
-    cu_dev, sched, n_jobs, max_len, total = sched_entry
+def _params(q, k, v, n_docs, max_seqlens, inv_temp, attend_current):
     H, N, D = q.shape
-    if total != N:
-        raise ValueError(f"cu_seqlens ends at {total} but q has {N} tokens")
     p = _lib.SbaParams()
     p.struct_size = C.sizeof(_lib.SbaParams)
     p.dtype = _lib.dtype_code(q.dtype)
-    p.n_seq, p.n_heads, p.seq_len, p.total_tokens, p.head_dim = cu_dev.numel() - 1, H, max_len, N, D
+    p.n_seq, p.n_heads, p.seq_len, p.total_tokens, p.head_dim = n_docs, H, max_seqlens, N, D
     p.attend_current = int(bool(attend_current))
     p.scale = float(inv_temp)
-    p.cu_seqlens, p.schedule, p.n_schedule = cu_dev.data_ptr(), sched.data_ptr(), n_jobs
     p.q, p.k, p.v = _lib.tensor3(q), _lib.tensor3(k), _lib.tensor3(v)
     p.stream = torch.cuda.current_stream(q.device).cuda_stream
     return p
+
+
+def _bind_schedule(p, q, cu_seqlens, max_seqlens):
+    cu_dev, sched, n_jobs, max_len, total = _schedule_for(cu_seqlens)
+    if total != q.shape[1]:
+        raise ValueError(f"cu_seqlens ends at {total} but q has {q.shape[1]} tokens")
+    if max_len > max_seqlens:
+        raise ValueError(f"max_seqlens={max_seqlens} is smaller than the longest document ({max_len})")
+    p.cu_seqlens, p.schedule, p.n_schedule = cu_dev.data_ptr(), sched.data_ptr(), n_jobs
+    return n_jobs
+
+
+def workspace_bytes(q, max_seqlens: int) -> int:
+    if torch.compiler.is_compiling():
+        H, N, D = q.shape
+        return _lib.workspace_upper_bound(H, max_seqlens, N, D)
+    p = _params(q, q, q, 1, max_seqlens, 1.0, False)
+    p.cu_seqlens = 1          # only "packed or not" matters for the size
+    return int(_lib.load().sba_workspace_bytes(C.byref(p)))
+
+
+# Registered names as in the reference (sb_varlen_fwd.py:449, sb_varlen_bwd.py:523).
+@custom_op("varlen_fwd", mutates_args=("o", "rem", "ws"))
+def _compileable_forward(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, cu_seqlens: torch.Tensor,
+                         max_seqlens: int, logit_scale: float, attend_current: bool, save: bool,
+                         o: torch.Tensor, rem: torch.Tensor, ws: torch.Tensor) -> None:
+    lib = _lib.load()
+    p = _params(q, k, v, cu_seqlens.numel() - 1, max_seqlens, logit_scale, attend_current)
+    if _bind_schedule(p, q, cu_seqlens, max_seqlens) == 0:
+        return
+    p.o = _lib.tensor3(o)
+    p.rem = _lib.SbaVector(rem.data_ptr(), 0, rem.stride(0))
+    p.save_for_backward = int(save)
+    if save:
+        p.workspace, p.workspace_bytes = ws.data_ptr(), ws.numel()
+    profiling.mark("start")
+    _lib.check(lib.sba_fwd(C.byref(p)), "sba_fwd")
+    profiling.mark("fwd")
+
+
+@custom_op("varlen_bwd", mutates_args=("dq", "dk", "dv", "ws"))
+def _compileable_backward(do: torch.Tensor, dr: Optional[torch.Tensor], q: torch.Tensor, k: torch.Tensor,
+                          v: torch.Tensor, cu_seqlens: torch.Tensor, max_seqlens: int, ws: torch.Tensor,
+                          logit_scale: float, attend_current: bool, dq: torch.Tensor, dk: torch.Tensor,
+                          dv: torch.Tensor) -> None:
+    lib = _lib.load()
+    p = _params(q, k, v, cu_seqlens.numel() - 1, max_seqlens, logit_scale, attend_current)
+    if _bind_schedule(p, q, cu_seqlens, max_seqlens) == 0:
+        return
+    p.d_o = _lib.tensor3(do)
+    if dr is not None:
+        p.d_rem = _lib.SbaVector(dr.data_ptr(), 0, dr.stride(0))
+    p.dq, p.dk, p.dv = _lib.tensor3(dq), _lib.tensor3(dk), _lib.tensor3(dv)
+    p.workspace, p.workspace_bytes = ws.data_ptr(), ws.numel()
+    profiling.launch_bwd(lib, p)
+
+
+def varlen_fwd(q, k, v, cu_seqlens, max_seqlens, logit_scale, attend_current=False, no_grad=False):
+    o = torch.empty_like(q)
+    rem = torch.empty(q.shape[:-1], dtype=q.dtype, device=q.device)
+    nbytes = 16 if no_grad else max(workspace_bytes(q, max_seqlens), 16)
+    ws = torch.empty(nbytes, dtype=torch.uint8, device=q.device)
+    _compileable_forward(q, k, v, cu_seqlens, int(max_seqlens), float(logit_scale), bool(attend_current),
+                         not no_grad, o, rem, ws)
+    return o, rem, ws
+
+
+def varlen_bwd(do, dr, q, k, v, cu_seqlens, max_seqlens, ws, logit_scale, attend_current=False):
+    dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+    _compileable_backward(do, dr, q, k, v, cu_seqlens, int(max_seqlens), ws, float(logit_scale),
+                          bool(attend_current), dq, dk, dv)
+    return dq, dk, dv
 
 
 class StickBreakingAttention(torch.autograd.Function):
@@ -70,28 +139,10 @@ class StickBreakingAttention(torch.autograd.Function):
                                "there is no CPU path")
         if not (q.shape == k.shape == v.shape) or q.dim() != 3:
             raise ValueError("q, k, v must all be [H, total_tokens, D]")
-        lib = _lib.load()
-        need_grad = any(ctx.needs_input_grad[:3])
+        no_grad = not any(ctx.needs_input_grad[:3])
         q, k, v = _lib.usable(q), _lib.usable(k), _lib.usable(v)
-        entry = _schedule_for(cu_seqlens)
-        H, N, D = q.shape
-        o = torch.empty_like(q)
-        rem = torch.empty((H, N), dtype=q.dtype, device=q.device)
-        ws = None
-        if entry[2] > 0:
-            p = _params(q, k, v, entry, inv_temp, attend_current)
-            p.o = _lib.tensor3(o)
-            p.rem = _lib.SbaVector(rem.data_ptr(), 0, rem.stride(0))
-            p.save_for_backward = int(need_grad)
-            if need_grad:
-                nbytes = lib.sba_workspace_bytes(C.byref(p))
-                ws = torch.empty(max(nbytes, 16), dtype=torch.uint8, device=q.device)
-                p.workspace, p.workspace_bytes = ws.data_ptr(), nbytes
-            profiling.mark("start")
-            _lib.check(lib.sba_fwd(C.byref(p)), "sba_fwd")
-            profiling.mark("fwd")
-        if need_grad:
-            ctx.save_for_backward(q, k, v, ws, cu_seqlens)
+        o, rem, ws = varlen_fwd(q, k, v, cu_seqlens, max_seqlens, inv_temp, attend_current, no_grad)
+        ctx.save_for_backward(q, k, v, ws, cu_seqlens)
         ctx.logit_scale = inv_temp
         ctx.max_seqlens = max_seqlens
         ctx.attend_current = attend_current
@@ -100,22 +151,14 @@ class StickBreakingAttention(torch.autograd.Function):
 
     @staticmethod
     def backward(ctx, do, drem):
-        lib = _lib.load()
         q, k, v, ws, cu_seqlens = ctx.saved_tensors
-        entry = _schedule_for(cu_seqlens)
-        dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
-        if entry[2] > 0:
-            if do is None:
-                do = torch.zeros_like(q)
-            do = _lib.usable(do)
-            p = _params(q, k, v, entry, ctx.logit_scale, ctx.attend_current)
-            p.d_o = _lib.tensor3(do)
-            if drem is not None:
-                drem = drem.contiguous()
-                p.d_rem = _lib.SbaVector(drem.data_ptr(), 0, drem.stride(0))
-            p.dq, p.dk, p.dv = _lib.tensor3(dq), _lib.tensor3(dk), _lib.tensor3(dv)
-            p.workspace, p.workspace_bytes = ws.data_ptr(), lib.sba_workspace_bytes(C.byref(p))
-            profiling.launch_bwd(lib, p)
+        if do is None:
+            do = torch.zeros_like(q)
+        do = _lib.usable(do)
+        if drem is not None:
+            drem = drem.contiguous()
+        dq, dk, dv = varlen_bwd(do, drem, q, k, v, cu_seqlens, ctx.max_seqlens, ws, ctx.logit_scale,
+                                ctx.attend_current)
         return dq, dk, dv, None, None, None, None
 
 

@@ -85,3 +85,13 @@ def test_op_refuses_cpu_tensors():
     q = torch.zeros(1, 1, 4, 8)
     with pytest.raises(RuntimeError, match="GPU only"):
         sb_attn(q, q, q)
+
+
+def test_python_workspace_bound_covers_the_library(lib):
+    for dtype in (_lib.SBA_DTYPE_BF16, _lib.SBA_DTYPE_F32):
+        for (B, H, T, D) in [(1, 16, 4096, 64), (2, 3, 129, 128), (1, 2, 77, 80), (4, 1, 1, 8)]:
+            p = _lib.SbaParams()
+            p.struct_size = C.sizeof(_lib.SbaParams)
+            p.dtype = dtype
+            p.n_seq, p.n_heads, p.seq_len, p.total_tokens, p.head_dim = B, H, T, T, D
+            assert _lib.workspace_upper_bound(H, T, B * T, D) >= lib.sba_workspace_bytes(C.byref(p))

@@ -281,3 +281,34 @@ def test_sba_340m_width_train_step_runs():
     losses = [float(train_step(model, opt, ids, ids, cu, max(lens))[0]) for _ in range(4)]
     print("losses", losses, flush=True)
     assert all(math.isfinite(x) for x in losses) and losses[-1] < losses[0]
+
+
+def test_varlen_rejects_too_small_max_seqlens():
+    _, sb_attn_varlen = _ops()
+    q = randn((2, 300, 64), 1, 0.5, torch.bfloat16).cuda()
+    with pytest.raises(ValueError, match="max_seqlens"):
+        sb_attn_varlen(q, q, q, torch.tensor([0, 100, 300], dtype=torch.int32).cuda(), 150)
+
+
+def test_torch_compile_fullgraph_matches_eager():
+    # the launchers are registered as stickbreaking_attention::{attn_fwd,attn_bwd,varlen_fwd,
+    # varlen_bwd} custom ops (as the reference does, utils.py:20-39), so the op traces
+    sb_attn, sb_attn_varlen = _ops()
+    assert hasattr(torch.ops.stickbreaking_attention, "attn_fwd")
+    assert hasattr(torch.ops.stickbreaking_attention, "varlen_bwd")
+    q, k, v, do = (randn((1, 2, 200, 64), 100 + i, 0.5, torch.bfloat16).cuda() for i in range(4))
+
+    def f(q, k, v):
+        o, rem = sb_attn(q, k, v)
+        return o * 2, rem
+
+    def run(fn):
+        qq, kk, vv = (x.clone().requires_grad_(True) for x in (q, k, v))
+        o, rem = fn(qq, kk, vv)
+        torch.autograd.backward([o], [do])
+        return o, rem, qq.grad, kk.grad, vv.grad
+
+    eager = run(f)
+    compiled = run(torch.compile(f, fullgraph=True))
+    for a, b in zip(eager, compiled):
+        assert torch.equal(a, b)
