@@ -8,7 +8,8 @@
 //           the forward's carry table, forms dz, accumulates dQ in registers, and records
 //           for every (query, key block) the prefix  sum_{j left of the block} g_ij  in a
 //           second table.
-//   pass 2  (key owner): a workgroup owns 128 keys (two 64-key blocks, one after the other),
+//   pass 2  (key owner): a workgroup owns one 64-key block (head_dim 64; two blocks, one
+//           after the other, in the head_dim 128 variant),
 //           sweeps the query blocks at or below the diagonal, recomputes weights and dz of
 //           its tile from the two tables, transposes them through LDS and accumulates
 //           dK = dZ^T Q and dV = P^T dO in registers.
@@ -301,7 +302,11 @@ __global__ __launch_bounds__(kThreads) void mfma_bwd_dkv64_kernel(KParams p) {
     char* zp = dobuf + kSlice;
     char* zd = zp + kSlice;
     const int head = blockIdx.x % p.n_heads;
-    const Job job = decode_job(p, order_job(blockIdx.x / p.n_heads, p.n_jobs, true));
+    // one workgroup per 64-key block: two per scheduled 128-row job, leftmost keys (longest
+    // sweeps) first
+    const int slot = blockIdx.x / p.n_heads;
+    const Job job = decode_job(p, order_job(slot >> 1, p.n_jobs, true));
+    const int half = slot & 1;
     const int strict = p.attend_current ? 0 : 1;
     const int64_t qbase = (int64_t)job.seq * p.q.sb + (int64_t)head * p.q.sh + (int64_t)job.tok0 * p.q.st;
     const int64_t kbase = (int64_t)job.seq * p.k.sb + (int64_t)head * p.k.sh + (int64_t)job.tok0 * p.k.st;
@@ -309,12 +314,11 @@ __global__ __launch_bounds__(kThreads) void mfma_bwd_dkv64_kernel(KParams p) {
     const int64_t dobase = (int64_t)job.seq * p.d_o.sb + (int64_t)head * p.d_o.sh + (int64_t)job.tok0 * p.d_o.st;
     const int n_qb = (job.len + kRowBlock - 1) / kRowBlock;
 
-    for (int half = 0; half < 2; ++half) {
+    {
         const int kb = 2 * job.rb + half;
         const int key0 = kb * kKeyBlock;
-        if (key0 >= job.len) break;            // uniform over the workgroup
+        if (key0 >= job.len) return;           // uniform over the workgroup
 
-        __syncthreads();                       // previous half's reduction is done with the LDS
         {
             TileCopy<D> kc, vc;
             kc.load(p.k, kbase, key0, job.len);
@@ -450,7 +454,7 @@ int sba_launch_mfma_bwd(const sba::KParams& kp, int phases, hipStream_t s) {
     const bool p1 = phases != 2, p2 = phases != 1;
     if (kp.head_dim == 64) {
         if (p1) hipLaunchKernelGGL((mfma_bwd_dq_kernel<64>), grid, dim3(kThreads), 0, s, kp);
-        if (p2) hipLaunchKernelGGL(mfma_bwd_dkv64_kernel, grid, dim3(kThreads), 0, s, kp);
+        if (p2) hipLaunchKernelGGL(mfma_bwd_dkv64_kernel, dim3(2 * grid.x), dim3(kThreads), 0, s, kp);
     } else {
         if (p1) hipLaunchKernelGGL((mfma_bwd_dq_kernel<128>), grid, dim3(kThreads), 0, s, kp);
         if (p2) hipLaunchKernelGGL((mfma_bwd_dkv_shared_kernel<128>), grid, dim3(kThreads), 0, s, kp);

@@ -51,21 +51,24 @@ __global__ __launch_bounds__(kThreads) void mfma_fwd_kernel(KParams p) {
         const char* ktile = lds + buf * 2 * kTile;
         const char* vtile = ktile + kTile;
         const bool more = step > 0;
+        const int key0 = step * kKeyBlock;
+        // whole step right of this wave's last query: nothing visible
+        const bool skip = key0 + strict > q0w + 31;
+        // The carry-table store goes FIRST: vector-memory operations retire in order, so the
+        // wait for the tile loads at the end of the step then also covers this store, long
+        // after it has completed, instead of stalling the next iteration's loads on it.
+        if (!skip && p.save && h == 0 && qi < job.len)
+            p.rtab[((int64_t)head * p.n_kb + step) * p.tab_tokens + tabtok] = R;
         if (more) {
             kc.load(p.k, kbase, (step - 1) * kKeyBlock, job.len);
             vc.load(p.v, vbase, (step - 1) * kKeyBlock, job.len);
         }
-        const int key0 = step * kKeyBlock;
-        // whole step right of this wave's last query: nothing visible
-        const bool skip = key0 + strict > q0w + 31;
         if (!skip) {
             float x[32];
             score_tiles<D>(x, ktile, qf, p.scale2, lane);
             if (key0 + 63 + strict > q0w) {     // diagonal region: mask invisible pairs
 mask_step(x, key0 + 32 * h, qi, strict);
             }
-            if (p.save && h == 0 && qi < job.len)
-                p.rtab[((int64_t)head * p.n_kb + step) * p.tab_tokens + tabtok] = R;
             float dummy[1];
             stick_weights<false>(x, dummy, R, lane);
             bf16x8 pf[4];
