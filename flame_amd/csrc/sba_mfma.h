@@ -50,6 +50,66 @@ template <int D> __device__ inline int tile_offset(int row, int chunk) {   // by
     return row * (D * 2) + ((chunk ^ swz<D>(row)) << 4);
 }
 
+// Lane-dependent byte offsets of the three fetch patterns, computed once per kernel.  The
+// swizzle only looks at row bits 0..3, so moving a fetch by a multiple of 16 rows (another
+// tile t, another 8-key group c, another 16-query group) adds a CONSTANT to the address:
+// every fetch below is "one of these few registers + an immediate".
+template <int D> struct LaneOffsets {
+    int rows[D / 16];          // row fetch: row (lane%32), chunk 2*ks + h          [+ 32*t rows]
+    int cols[2][D / 32];       // transposing fetch, MFMA-order tiles: [a][db]      [+ 32*(c>>1) + 16*(c&1) rows]
+    int nat[2][D / 32];        // transposing fetch, natural-order tiles: [a][cb]   [+ row0 (multiple of 16) rows]
+    __device__ inline void init(int lane) {
+        const int h = lane >> 5, G1 = (lane >> 4) & 1, s = lane & 15;
+#pragma unroll
+        for (int ks = 0; ks < D / 16; ++ks) rows[ks] = tile_offset<D>(lane & 31, 2 * ks + h);
+#pragma unroll
+        for (int a = 0; a < 2; ++a)
+#pragma unroll
+            for (int b = 0; b < D / 32; ++b) {
+                const int chunk = 4 * b + 2 * G1 + ((s & 3) >> 1);
+                cols[a][b] = tile_offset<D>(8 * a + 4 * h + (s >> 2), chunk) + ((s & 1) << 3);
+                nat[a][b] = tile_offset<D>(8 * h + 4 * a + (s >> 2), chunk) + ((s & 1) << 3);
+            }
+    }
+};
+
+__device__ inline s16x4 lds_read_tr(const char* p) {
+    return __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+        (__attribute__((address_space(3))) s16x4*)(uintptr_t)(uint32_t)(uintptr_t)p);
+}
+
+// Same three fetches as fetch_rows / fetch_cols / fetch_cols_nat, from precomputed offsets.
+template <int D> __device__ inline bf16x8 fetch_rows_o(const char* tile, const LaneOffsets<D>& o, int t, int ks) {
+    return *(const bf16x8*)(tile + o.rows[ks] + t * 32 * D * 2);
+}
+template <int D> __device__ inline bf16x8 fetch_cols_o(const char* tile, const LaneOffsets<D>& o, int db, int c) {
+    union { s16x4 v[2]; bf16x8 b; } u;
+    const int add = (32 * (c >> 1) + 16 * (c & 1)) * D * 2;
+    u.v[0] = lds_read_tr(tile + o.cols[0][db] + add);
+    u.v[1] = lds_read_tr(tile + o.cols[1][db] + add);
+    return u.b;
+}
+template <int D> __device__ inline bf16x8 fetch_nat_o(const char* tile, const LaneOffsets<D>& o, int row0, int cb) {
+    union { s16x4 v[2]; bf16x8 b; } u;
+    u.v[0] = lds_read_tr(tile + o.nat[0][cb] + row0 * D * 2);
+    u.v[1] = lds_read_tr(tile + o.nat[1][cb] + row0 * D * 2);
+    return u.b;
+}
+// The same with the two lane offsets already picked (column block chosen at run time:
+// indexing the offset table with a run-time value would push it into scratch memory).
+template <int ROWD> __device__ inline bf16x8 fetch_nat_2(const char* tile, int off0, int off1, int row0) {
+    union { s16x4 v[2]; bf16x8 b; } u;
+    u.v[0] = lds_read_tr(tile + off0 + row0 * ROWD * 2);
+    u.v[1] = lds_read_tr(tile + off1 + row0 * ROWD * 2);
+    return u.b;
+}
+template <int D> __device__ inline int pick_nat(const LaneOffsets<D>& o, int a, int cb) {
+    int v = o.nat[a][0];
+#pragma unroll
+    for (int b = 1; b < D / 32; ++b) v = (cb == b) ? o.nat[a][b] : v;
+    return v;
+}
+
 // Global -> registers -> LDS copy of one 64-row tile (rows row0..row0+63 of a sequence),
 // split so that the global loads of the next tile overlap the arithmetic on this one.
 template <int D> struct TileCopy {
@@ -149,6 +209,18 @@ __device__ inline void score_raw(f32x16 (&raw)[2], const char* ktile, const bf16
     }
 }
 
+template <int D>
+__device__ inline void score_raw_o(f32x16 (&raw)[2], const char* ktile, const LaneOffsets<D>& o,
+                                   const bf16x8 (&qf)[D / 16]) {
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+        f32x16 acc = {0};
+#pragma unroll
+        for (int ks = 0; ks < D / 16; ++ks) acc = mfma(fetch_rows_o<D>(ktile, o, t, ks), qf[ks], acc);
+        raw[t] = acc;
+    }
+}
+
 // base-2 logits from the raw accumulators: x[16*t + r] = scale2 * raw[t][r].
 __device__ inline void scale_scores(float (&x)[32], const f32x16 (&raw)[2], float scale2) {
 #pragma unroll
@@ -162,6 +234,14 @@ __device__ inline void score_tiles(float (&x)[32], const char* ktile, const bf16
                                    float scale2, int lane) {
     f32x16 raw[2];
     score_raw<D>(raw, ktile, qf, lane);
+    scale_scores(x, raw, scale2);
+}
+
+template <int D>
+__device__ inline void score_tiles_o(float (&x)[32], const char* ktile, const LaneOffsets<D>& o,
+                                     const bf16x8 (&qf)[D / 16], float scale2) {
+    f32x16 raw[2];
+    score_raw_o<D>(raw, ktile, o, qf);
     scale_scores(x, raw, scale2);
 }
 
@@ -238,6 +318,21 @@ __device__ inline void dp_tiles(float (&dp)[32], const char* vtile, const bf16x8
         for (int r = 0; r < 16; ++r) acc[r] = -dr;
 #pragma unroll
         for (int ks = 0; ks < D / 16; ++ks) acc = mfma(fetch_rows<D>(vtile, t, ks, lane), dof[ks], acc);
+#pragma unroll
+        for (int r = 0; r < 16; ++r) dp[16 * t + r] = acc[r];
+    }
+}
+
+template <int D>
+__device__ inline void dp_tiles_o(float (&dp)[32], const char* vtile, const LaneOffsets<D>& o,
+                                  const bf16x8 (&dof)[D / 16], float dr) {
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+        f32x16 acc;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[r] = -dr;
+#pragma unroll
+        for (int ks = 0; ks < D / 16; ++ks) acc = mfma(fetch_rows_o<D>(vtile, o, t, ks), dof[ks], acc);
 #pragma unroll
         for (int r = 0; r < 16; ++r) dp[16 * t + r] = acc[r];
     }

@@ -15,6 +15,8 @@ __global__ __launch_bounds__(kThreads) void mfma_fwd_kernel(KParams p) {
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);   // wave-uniform, keep it scalar
     const int n = lane & 31, h = lane >> 5;
+    LaneOffsets<D> lo;
+    lo.init(lane);
     const int head = blockIdx.x % p.n_heads;
     const Job job = decode_job(p, order_job(blockIdx.x / p.n_heads, p.n_jobs, false));
     const int strict = p.attend_current ? 0 : 1;
@@ -65,7 +67,7 @@ __global__ __launch_bounds__(kThreads) void mfma_fwd_kernel(KParams p) {
         }
         if (!skip) {
             float x[32];
-            score_tiles<D>(x, ktile, qf, p.scale2, lane);
+            score_tiles_o<D>(x, ktile, lo, qf, p.scale2);
             if (key0 + 63 + strict > q0w) {     // diagonal region: mask invisible pairs
 mask_step(x, key0 + 32 * h, qi, strict);
             }
@@ -78,7 +80,7 @@ mask_step(x, key0 + 32 * h, qi, strict);
             for (int db = 0; db < D / 32; ++db)
 #pragma unroll
                 for (int c = 0; c < 4; ++c)
-                    oacc[db] = mfma(fetch_cols<D>(vtile, db, c, lane), pf[c], oacc[db]);
+                    oacc[db] = mfma(fetch_cols_o<D>(vtile, lo, db, c), pf[c], oacc[db]);
         }
         if (more) {
             kc.store(lds + (buf ^ 1) * 2 * kTile);
