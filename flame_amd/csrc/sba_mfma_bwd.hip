@@ -135,32 +135,11 @@ mask_step(x, key0 + 32 * h, qi, strict);
 // turns its 32 queries into weights (a, dz), writes them as bf16 [query][key] rows into a
 // tile shared by the workgroup, and after a barrier reduces ONE [32 keys x 32 d] tile of
 // dK and of dV over all 128 queries, so its accumulators are 2 x 16 x D/64 registers and
-// two workgroups fit on a CU.  The Q and dO tiles that the reduction reads (transposed)
-// are DMA'd from global memory straight into LDS at the top of the step, behind the
-// vector arithmetic; the per-lane Q/dO row fragments and the per-query scalars (carry
-// tables, drem) are prefetched into registers one step ahead.
-template <int D>
-__device__ inline void dma_rows_nat(char* tile, const TensorArg& t, int64_t base, int row0, int len, int rows) {
-    // Natural-order tile, `rows` rows x D bf16, swizzled like tile_offset<D>.  Every
-    // instruction moves 64 x 16 bytes into 1 KB of consecutive LDS; the lane picks the global
-    // chunk that belongs at its LDS position.  Rows past the end are clamped (finite
-    // garbage; callers neutralise those rows).
-    constexpr int kCpr = D / 8;                       // 16-byte chunks per row
-    const int lane = threadIdx.x & 63;
-    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const int n_inst = rows * kCpr / 64;
-    for (int i = wave; i < n_inst; i += kThreads / 64) {
-        const int pos = i * 64 + lane;                // LDS chunk position
-        const int r = pos / kCpr, pc = pos % kCpr;
-        const int c = pc ^ swz<D>(r);
-        const int row = min(row0 + r, len - 1);
-        const char* g = t.ptr + 2 * (base + (int64_t)row * t.st + c * 8);
-        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)g,
-                                         (__attribute__((address_space(3))) void*)(uintptr_t)(uint32_t)(uintptr_t)(tile + i * 1024),
-                                         16, 0, 0);
-    }
-}
-
+// two workgroups fit on a CU.  Every Q / dO row is fetched from global memory once, as the
+// per-lane row fragments that the score / dP MFMAs need (Q a step ahead, dO at the top of
+// the step, hidden behind the weights); the same registers are then stored into the shared
+// Q and dO tiles that the reduction reads transposed.  Per-query scalars (carry tables,
+// drem) are prefetched one step ahead.
 template <int D>
 __global__ __launch_bounds__(kThreads, 2) void mfma_bwd_dkv_kernel(KParams p) {
     constexpr int kTile = 64 * D * 2;          // K or V tile (64 keys)
@@ -219,8 +198,10 @@ __global__ __launch_bounds__(kThreads, 2) void mfma_bwd_dkv_kernel(KParams p) {
     const int qb0 = job.rb;
     // prefetched state of the first step
     float Rn = 1.0f, Gn = 0.0f, drn = 0.0f;
+    bf16x8 qfn[D / 16];
     {
         const int qi0 = qb0 * kRowBlock + 32 * wave + n;
+        load_row_frags<D>(qfn, p.q, qbase, qi0, job.len, lane);
         if (qi0 < job.len) {
             const int64_t t = trow + tab_token(p, job, qi0);
             Rn = p.rtab[t]; Gn = p.gtab[t];
@@ -233,17 +214,18 @@ __global__ __launch_bounds__(kThreads, 2) void mfma_bwd_dkv_kernel(KParams p) {
         const int m0 = qb * kRowBlock;
         const int q0w = m0 + 32 * wave;
         const int qi = q0w + n;
-        // (1) start the DMA of this step's Q and dO tiles (every wave passed the barrier that
-        //     ends the previous step's reduction, so the tiles are free)
-        dma_rows_nat<D>(qtile, p.q, qbase, m0, job.len, kRowBlock);
-        dma_rows_nat<D>(dotile, p.d_o, dobase, m0, job.len, kRowBlock);
-        // (2) take over the prefetched per-lane state, prefetch the next step's
+        // (1) this lane's Q row fragments were prefetched during the previous step; its dO
+        //     fragments are requested now and not needed before the weights are done.  Each
+        //     row is fetched from global memory exactly once: the fragments are also what the
+        //     shared Q / dO tiles of the reduction are assembled from.
         bf16x8 qf[D / 16], dof[D / 16];
-        load_row_frags<D>(qf, p.q, qbase, qi, job.len, lane);
+#pragma unroll
+        for (int ks = 0; ks < D / 16; ++ks) qf[ks] = qfn[ks];
         load_row_frags<D>(dof, p.d_o, dobase, qi, job.len, lane);
         float R = Rn, Gc = Gn, dr = drn;
         if (qb + 1 < n_qb) {
             const int qin = qi + kRowBlock;
+            load_row_frags<D>(qfn, p.q, qbase, qin, job.len, lane);
             Rn = 1.0f; Gn = 0.0f; drn = 0.0f;
             if (qin < job.len) {
                 const int64_t t = trow + tab_token(p, job, qin);
@@ -251,6 +233,11 @@ __global__ __launch_bounds__(kThreads, 2) void mfma_bwd_dkv_kernel(KParams p) {
                 if (p.d_rem.ptr) drn = Elem<uint16_t>::load(p.d_rem.ptr, dr_base + qin);
             }
         }
+        // (2) row 32*wave + n of the shared Q tile (every wave passed the barrier that ends the
+        //     previous step's reduction, so the tiles are free)
+#pragma unroll
+        for (int ks = 0; ks < D / 16; ++ks)
+            *(bf16x8*)(qtile + tile_offset<D>(32 * wave + n, 2 * ks + h)) = qf[ks];
         // (3) weights of this wave's 32 queries
         float x[32], dp[32];
         const bool skip = key0 + strict > q0w + 31 || q0w >= job.len;
@@ -259,15 +246,15 @@ __global__ __launch_bounds__(kThreads, 2) void mfma_bwd_dkv_kernel(KParams p) {
             score_tiles_o<D>(x, ktile, lo, qf, p.scale2);
             if (key0 + 63 + strict > q0w) mask_step(x, key0 + 32 * h, qi, strict);
             stick_weights<true>(x, beta, R, lane);
+#pragma unroll
+            for (int ks = 0; ks < D / 16; ++ks)
+                *(bf16x8*)(dotile + tile_offset<D>(32 * wave + n, 2 * ks + h)) = dof[ks];
             dp_tiles_o<D>(dp, vtile, lo, dof, dr);
             logit_grads<true>(x, beta, dp, Gc, lane);
-            if (q0w + 31 >= job.len && qi >= job.len) {
-                // query past the end of the sequence: its DMA'd tile rows are clamped copies,
-                // so its weights must not reach the reduction (dz is already 0 there)
-#pragma unroll
-                for (int idx = 0; idx < 32; ++idx) x[idx] = 0.f;
-            }
         } else {
+#pragma unroll
+            for (int ks = 0; ks < D / 16; ++ks)
+                *(bf16x8*)(dotile + tile_offset<D>(32 * wave + n, 2 * ks + h)) = dof[ks];
 #pragma unroll
             for (int idx = 0; idx < 32; ++idx) { x[idx] = 0.f; dp[idx] = 0.f; }
         }
@@ -276,7 +263,6 @@ __global__ __launch_bounds__(kThreads, 2) void mfma_bwd_dkv_kernel(KParams p) {
             *(bf16x8*)(zp + tile_offset<64>(32 * wave + n, 4 * h + c)) = pack8(&x[8 * c]);
             *(bf16x8*)(zd + tile_offset<64>(32 * wave + n, 4 * h + c)) = pack8(&dp[8 * c]);
         }
-        __builtin_amdgcn_s_waitcnt(0x0f70);    // vmcnt(0): this wave's share of the DMA has landed
         __syncthreads();                       // weights and tiles of all waves visible
         // (4) dK[key][d] += sum_q dz[q][key] Q[q][d];  dV[key][d] += sum_q a[q][key] dO[q][d]
 #pragma unroll
