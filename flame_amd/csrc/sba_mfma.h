@@ -112,30 +112,38 @@ template <int D> __device__ inline int pick_nat(const LaneOffsets<D>& o, int a, 
 
 // Global -> registers -> LDS copy of one 64-row tile (rows row0..row0+63 of a sequence),
 // split so that the global loads of the next tile overlap the arithmetic on this one.
+// A thread moves chunks (row kl, chunk c) and (row kl + 64/kPerThread * i, c): the address
+// is a wave-uniform 64-bit base plus a 32-bit per-thread offset that never changes, so a
+// step costs no vector address arithmetic.
 template <int D> struct TileCopy {
     static constexpr int kChunks = 64 * D / 8;                 // 16-byte chunks per tile
     static constexpr int kPerThread = kChunks / kThreads;      // 2 (D=64) or 4 (D=128)
+    static constexpr int kRowStep = 64 / kPerThread;           // rows between a thread's chunks
     u32x4 regs[kPerThread];
 
-    // rows of the tile in MFMA order when `permute`, natural order otherwise
     __device__ inline void load(const TensorArg& t, int64_t base, int row0, int len) {
+        const int kl = threadIdx.x / (D / 8), c = threadIdx.x % (D / 8);
+        const char* tile_base = t.ptr + 2 * (base + (int64_t)row0 * t.st);          // uniform
+        const uint32_t lane_off = 2u * (uint32_t)(kl * (int)t.st + c * 8);
+        const uint32_t step_off = 2u * (uint32_t)(kRowStep * (int)t.st);
+        if (row0 + 64 <= len) {                                // whole tile inside the sequence
 #pragma unroll
-        for (int r = 0; r < kPerThread; ++r) {
-            int cid = threadIdx.x + r * kThreads;
-            int kl = cid / (D / 8), c = cid % (D / 8);
-            int row = row0 + kl;
-            u32x4 v = {0u, 0u, 0u, 0u};
-            if (row < len) v = *(const u32x4*)(t.ptr + 2 * (base + (int64_t)row * t.st + c * 8));
-            regs[r] = v;
+            for (int r = 0; r < kPerThread; ++r)
+                regs[r] = *(const u32x4*)(tile_base + (size_t)(lane_off + r * step_off));
+        } else {
+#pragma unroll
+            for (int r = 0; r < kPerThread; ++r) {
+                u32x4 v = {0u, 0u, 0u, 0u};
+                if (row0 + kl + r * kRowStep < len) v = *(const u32x4*)(tile_base + (size_t)(lane_off + r * step_off));
+                regs[r] = v;
+            }
         }
     }
     __device__ inline void store(char* tile) const {
+        const int kl = threadIdx.x / (D / 8), c = threadIdx.x % (D / 8);
 #pragma unroll
-        for (int r = 0; r < kPerThread; ++r) {
-            int cid = threadIdx.x + r * kThreads;
-            int kl = cid / (D / 8), c = cid % (D / 8);
-            *(u32x4*)(tile + tile_offset<D>(mfma_row_of_key(kl), c)) = regs[r];
-        }
+        for (int r = 0; r < kPerThread; ++r)
+            *(u32x4*)(tile + tile_offset<D>(mfma_row_of_key(kl + r * kRowStep), c)) = regs[r];
     }
 };
 
@@ -167,16 +175,19 @@ template <int D> __device__ inline bf16x8 fetch_cols(const char* tile, int db, i
 }
 
 // B operand kept in registers for the whole sweep: row `row` of a [rows, D] tensor,
-// columns 16*ks + 8*h .. +7 for every ks.  Rows >= len read as zero.
+// columns 16*ks + 8*h .. +7 for every ks.  Rows >= len read as zero.  One address, one
+// predicate; the ks fragments are at constant offsets from it.
 template <int D>
 __device__ inline void load_row_frags(bf16x8 (&f)[D / 16], const TensorArg& t, int64_t base, int row,
                                       int len, int lane) {
     const int h = lane >> 5;
+    const char* ptr = t.ptr + 2 * (base + (int64_t)row * t.st + 8 * h);
+    if (row < len) {
 #pragma unroll
-    for (int ks = 0; ks < D / 16; ++ks) {
-        u32x4 v = {0u, 0u, 0u, 0u};
-        if (row < len) v = *(const u32x4*)(t.ptr + 2 * (base + (int64_t)row * t.st + 16 * ks + 8 * h));
-        f[ks] = __builtin_bit_cast(bf16x8, v);
+        for (int ks = 0; ks < D / 16; ++ks) f[ks] = __builtin_bit_cast(bf16x8, *(const u32x4*)(ptr + 32 * ks));
+    } else {
+#pragma unroll
+        for (int ks = 0; ks < D / 16; ++ks) f[ks] = bf16x8{0};
     }
 }
 
