@@ -16,9 +16,7 @@
 // LDS tiles hold 64 rows of D bf16.  Row order is "MFMA order": key_local
 // 32*hh + 16*t + 4*g + i lives in row rho = 32*t + 8*g + 4*hh + i, so that the A-operand
 // fetch of tile t reads rows 32*t + lane%32.  16-byte chunks of a row are XOR-swizzled
-// (see swz()) so that both access patterns used here are bank-conflict free:
-//   * row fetches   (ds_read_b128: 16 consecutive rows, one chunk each) and
-//   * transposing fetches (ds_read_b64_tr_b16: 4 consecutive rows x 64 bytes).
+// (see swz()) so that every access pattern used here is bank-conflict free.
 #pragma once
 #include "sba_common.h"
 
@@ -37,13 +35,20 @@ __device__ inline int mfma_row_of_key(int kl) {   // key_local -> LDS row
     return ((kl >> 4) & 1) * 32 + ((kl >> 2) & 3) * 8 + (kl >> 5) * 4 + (kl & 3);
 }
 
+// XOR swizzle of the 16-byte chunk index, a function of row bits 0..3 only.  It has to keep
+// four access patterns conflict-free at once (verified with SQ_LDS_BANK_CONFLICT = 0):
+//   row reads    ds_read_b128  : 16 lanes = 16 consecutive rows, same chunk (64 banks / cycle)
+//   row writes   ds_write_b128 :  8 lanes =  8 consecutive rows, same chunk (32 banks / cycle)
+//   tile stores  ds_write_b128 :  consecutive lanes fill one row
+//   transposing reads ds_read_b64_tr_b16 : 4 consecutive rows x 64 bytes per half-wave
 template <int D> __device__ inline int swz(int row);
-template <> __device__ inline int swz<64>(int row) {   // 8 chunks per row
+template <> __device__ inline int swz<64>(int row) {   // 8 chunks per row, two rows per 64 banks
     int v = (row >> 1) & 7;
-    return ((v & 1) << 2) | (v & 2) | ((v >> 2) & 1);
+    return (((v & 1) << 2) | (v & 2) | ((v >> 2) & 1)) ^ (row & 1);
 }
-template <> __device__ inline int swz<128>(int row) {  // 16 chunks per row
-    return ((row & 3) << 2) | ((row >> 2) & 3);
+template <> __device__ inline int swz<128>(int row) {  // 16 chunks per row, one row per 64 banks
+    const int r0 = row & 1, r1 = (row >> 1) & 1, r2 = (row >> 2) & 1, r3 = (row >> 3) & 1;
+    return (r1 << 3) | (r0 << 2) | ((r1 ^ r3) << 1) | r2;
 }
 
 template <int D> __device__ inline int tile_offset(int row, int chunk) {   // bytes
