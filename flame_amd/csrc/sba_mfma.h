@@ -127,7 +127,8 @@ template <int D> struct TileCopy {
     u32x4 regs[kPerThread];
 
     __device__ inline void load(const TensorArg& t, int64_t base, int row0, int len) {
-        const int kl = threadIdx.x / (D / 8), c = threadIdx.x % (D / 8);
+        const int tid = threadIdx.x & (kThreads - 1);      // 256 threads copy one tile
+        const int kl = tid / (D / 8), c = tid % (D / 8);
         const char* tile_base = t.ptr + 2 * (base + (int64_t)row0 * t.st);          // uniform
         const uint32_t lane_off = 2u * (uint32_t)(kl * (int)t.st + c * 8);
         const uint32_t step_off = 2u * (uint32_t)(kRowStep * (int)t.st);
@@ -145,7 +146,8 @@ template <int D> struct TileCopy {
         }
     }
     __device__ inline void store(char* tile) const {
-        const int kl = threadIdx.x / (D / 8), c = threadIdx.x % (D / 8);
+        const int tid = threadIdx.x & (kThreads - 1);
+        const int kl = tid / (D / 8), c = tid % (D / 8);
 #pragma unroll
         for (int r = 0; r < kPerThread; ++r)
             *(u32x4*)(tile + tile_offset<D>(mfma_row_of_key(kl + r * kRowStep), c)) = regs[r];
@@ -291,6 +293,34 @@ __device__ inline void stick_weights(float (&x)[32], float (&beta)[kNeedBeta ? 3
     R = R * L * other;
 }
 
+// The same in two parts, for kernels in which another wave-group handles the neighbouring
+// step and the carry is only known after an exchange:
+//   part 1: x[idx] <- weights relative to the right edge of THIS lane's 32 keys; returns the
+//           factor that completes them inside the step (1 for the upper half-wave, the upper
+//           half's product for the lower) and, in `total`, the product over all 64 keys;
+//   part 2: x[idx] *= carry * factor.
+template <bool kNeedBeta>
+__device__ inline float stick_weights_local(float (&x)[32], float (&beta)[kNeedBeta ? 32 : 1], float& total,
+                                            int lane) {
+    float L = 1.0f;
+#pragma unroll
+    for (int idx = 31; idx >= 0; --idx) {
+        float e = __builtin_amdgcn_exp2f(x[idx]);
+        float u = __builtin_amdgcn_rcpf(1.0f + e);
+        float b = 1.0f - u;
+        x[idx] = b * L;
+        L *= u;
+        if (kNeedBeta) beta[idx] = b;
+    }
+    const float other = __shfl_xor(L, 32);
+    total = L * other;
+    return (lane >= 32) ? 1.0f : other;
+}
+__device__ inline void scale32(float (&x)[32], float f) {
+#pragma unroll
+    for (int idx = 0; idx < 32; ++idx) x[idx] *= f;
+}
+
 // Sets the logits of invisible (query, key) pairs of a diagonal step to -inf.
 __device__ inline void mask_step(float (&x)[32], int key_first, int qi, int strict) {
     // key_first = first key of this lane's 32; key j visible iff j + strict <= qi
@@ -391,6 +421,29 @@ __device__ inline void logit_grads(const float (&a)[32], const float (&beta)[32]
 #pragma unroll
         for (int idx = 0; idx < 32; ++idx) dp[idx] = __builtin_fmaf(-beta[idx], pre[idx] + F, dp[idx]);
         Gc = Gc + c + other;
+    }
+}
+
+// logit_grads in two parts (see stick_weights_local): part 1 forms g in place of dp and
+// returns this lane's offset inside the step (0 for the lower half-wave, the lower half's
+// sum for the upper) and, in `total`, the step's sum of g; part 2 applies the prefix.
+__device__ inline float logit_grads_local(const float (&a)[32], float (&dp)[32], float& total, int lane) {
+    float c = 0.f;
+#pragma unroll
+    for (int idx = 0; idx < 32; ++idx) {
+        dp[idx] = a[idx] * dp[idx];     // g
+        c += dp[idx];
+    }
+    const float other = __shfl_xor(c, 32);
+    total = c + other;
+    return (lane >= 32) ? other : 0.0f;
+}
+__device__ inline void logit_grads_apply(const float (&beta)[32], float (&dp)[32], float start) {
+    float run = start;
+#pragma unroll
+    for (int idx = 0; idx < 32; ++idx) {
+        run += dp[idx];
+        dp[idx] = __builtin_fmaf(-beta[idx], run, dp[idx]);
     }
 }
 

@@ -109,12 +109,154 @@ mask_step(x, key0 + 32 * h, qi, strict);
     }
 }
 
+// ---------------------------------------------------------------- two steps per iteration
+// Same sweep with 8 waves: wave-group 0 (waves 0-3) and wave-group 1 (waves 4-7) take two
+// CONSECUTIVE 64-key steps of the same 128 queries in every iteration.  All the heavy work of
+// a step (scores, exp/rcp, the in-step product chain, P*V) only needs the step's own keys; what
+// couples neighbouring steps is one number per query, the product of (1 - beta) over the
+// step.  The groups swap those totals through LDS at a barrier, the left group multiplies the
+// right group's total into its carry, and each group accumulates its own partial O, summed once
+// at the end.  The longest dependent chain of a kernel launch (the sweep of the last row-block)
+// is halved, which is what bounds the time when the whole problem is only two waves per SIMD.
+template <int D>
+__global__ __launch_bounds__(2 * kThreads) void mfma_fwd2_kernel(KParams p) {
+    constexpr int kTile = 64 * D * 2;
+    // tile(buf, grp, kv) = lds + ((buf * 2 + grp) * 2 + kv) * kTile
+    __shared__ __attribute__((aligned(16))) char lds[8 * kTile];
+    __shared__ float xch[2][kRowBlock];
+
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int grp = wave >> 2, qs = wave & 3;
+    const int n = lane & 31, h = lane >> 5;
+    LaneOffsets<D> lo;
+    lo.init(lane);
+    const int head = blockIdx.x % p.n_heads;
+    const Job job = decode_job(p, order_job(blockIdx.x / p.n_heads, p.n_jobs, false));
+    const int strict = p.attend_current ? 0 : 1;
+    const int m0 = job.rb * kRowBlock;
+    const int q0w = m0 + 32 * qs;
+    const int qi = q0w + n;
+    const int64_t qbase = (int64_t)job.seq * p.q.sb + (int64_t)head * p.q.sh + (int64_t)job.tok0 * p.q.st;
+    const int64_t kbase = (int64_t)job.seq * p.k.sb + (int64_t)head * p.k.sh + (int64_t)job.tok0 * p.k.st;
+    const int64_t vbase = (int64_t)job.seq * p.v.sb + (int64_t)head * p.v.sh + (int64_t)job.tok0 * p.v.st;
+
+    bf16x8 qf[D / 16];
+    load_row_frags<D>(qf, p.q, qbase, qi, job.len, lane);
+    f32x16 oacc[D / 32];
+#pragma unroll
+    for (int db = 0; db < D / 32; ++db) oacc[db] = f32x16{0};
+    float R = 1.0f;
+
+    const int imax = min(m0 + kRowBlock - 1, job.len - 1);
+    const int kmax = imax - strict;
+    const int n_steps = kmax >= 0 ? kmax / kKeyBlock + 1 : 0;
+    const int n_it = (n_steps + 1) / 2;
+    const int64_t tabtok = tab_token(p, job, qi);
+    char* my_tiles = lds + grp * 2 * kTile;          // + buf * 4 * kTile
+
+    // each group copies its own tiles (256 threads per tile pair)
+    TileCopy<D> kc, vc;
+    {
+        const int s0 = n_steps - 1 - grp;
+        if (s0 >= 0) {
+            kc.load(p.k, kbase, s0 * kKeyBlock, job.len);
+            vc.load(p.v, vbase, s0 * kKeyBlock, job.len);
+            kc.store(my_tiles);
+            vc.store(my_tiles + kTile);
+        }
+    }
+    __syncthreads();
+
+    for (int it = 0, buf = 0; it < n_it; ++it, buf ^= 1) {
+        const int step = n_steps - 1 - 2 * it - grp;          // -1: this group idles in the last iteration
+        const char* ktile = my_tiles + buf * 4 * kTile;
+        const char* vtile = ktile + kTile;
+        const bool more = step - 2 >= 0;
+        if (more) {
+            kc.load(p.k, kbase, (step - 2) * kKeyBlock, job.len);
+            vc.load(p.v, vbase, (step - 2) * kKeyBlock, job.len);
+        }
+        const int key0 = step * kKeyBlock;
+        const bool active = step >= 0 && !(key0 + strict > q0w + 31);
+        float x[32];
+        float total = 1.0f, fac = 1.0f;
+        if (active) {
+            score_tiles_o<D>(x, ktile, lo, qf, p.scale2);
+            if (key0 + 63 + strict > q0w) mask_step(x, key0 + 32 * h, qi, strict);
+            float dummy[1];
+            fac = stick_weights_local<false>(x, dummy, total, lane);
+        }
+        if (h == 0) xch[grp][32 * qs + n] = total;
+        __syncthreads();
+        const float other = xch[grp ^ 1][32 * qs + n];
+        // group 0 holds the right step of the pair: its carry is R; group 1's also contains
+        // group 0's total
+        const float Rmy = grp == 0 ? R : R * other;
+        R = R * total * other;
+        if (active) {
+            if (p.save && h == 0 && qi < job.len)
+                p.rtab[((int64_t)head * p.n_kb + step) * p.tab_tokens + tabtok] = Rmy;
+            scale32(x, fac * Rmy);
+            bf16x8 pf[4];
+#pragma unroll
+            for (int c = 0; c < 4; ++c) pf[c] = pack8(&x[8 * c]);
+#pragma unroll
+            for (int db = 0; db < D / 32; ++db)
+#pragma unroll
+                for (int c = 0; c < 4; ++c)
+                    oacc[db] = mfma(fetch_cols_o<D>(vtile, lo, db, c), pf[c], oacc[db]);
+        }
+        if (more) {
+            kc.store(my_tiles + (buf ^ 1) * 4 * kTile);
+            vc.store(my_tiles + (buf ^ 1) * 4 * kTile + kTile);
+        }
+        __syncthreads();
+    }
+
+    // ---- O = O(group 0) + O(group 1): group 1 parks its accumulators in LDS
+    float* park = (float*)lds;                              // [qs][db][r][lane]
+    if (grp == 1) {
+#pragma unroll
+        for (int db = 0; db < D / 32; ++db)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) park[((qs * (D / 32) + db) * 16 + r) * 64 + lane] = oacc[db][r];
+    }
+    __syncthreads();
+    if (grp == 0 && qi < job.len) {
+        const int64_t obase = (int64_t)job.seq * p.o.sb + (int64_t)head * p.o.sh + (int64_t)(job.tok0 + qi) * p.o.st;
+#pragma unroll
+        for (int db = 0; db < D / 32; ++db) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) oacc[db][r] += park[((qs * (D / 32) + db) * 16 + r) * 64 + lane];
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                f32x2 a = {oacc[db][4 * g], oacc[db][4 * g + 1]};
+                f32x2 b = {oacc[db][4 * g + 2], oacc[db][4 * g + 3]};
+                bf16x2 pa = __builtin_convertvector(a, bf16x2), pb = __builtin_convertvector(b, bf16x2);
+                uint2 w;
+                w.x = __builtin_bit_cast(uint32_t, pa);
+                w.y = __builtin_bit_cast(uint32_t, pb);
+                *(uint2*)(p.o.ptr + 2 * (obase + 32 * db + 8 * g + 4 * h)) = w;
+            }
+        }
+        if (h == 0)
+            Elem<uint16_t>::store(p.rem.ptr, (int64_t)job.seq * p.rem.sb + (int64_t)head * p.rem.sh + job.tok0 + qi, R);
+    }
+}
+
 }  // namespace sba
 
 int sba_launch_mfma_fwd(const sba::KParams& kp, hipStream_t s) {
     using namespace sba;
     dim3 grid((unsigned)kp.n_jobs * kp.n_heads);
-    if (kp.head_dim == 64)
+    // A grid this small cannot give every SIMD more than two waves, and the launch lasts as long
+    // as its longest sweep: take the variant that halves that chain.  Larger grids are bound
+    // by throughput, where the 4-wave kernel (3 waves per SIMD) is ahead.
+    const bool small_grid = grid.x <= 1024;
+    if (kp.head_dim == 64 && small_grid)
+        hipLaunchKernelGGL((mfma_fwd2_kernel<64>), grid, dim3(2 * kThreads), 0, s, kp);
+    else if (kp.head_dim == 64)
         hipLaunchKernelGGL((mfma_fwd_kernel<64>), grid, dim3(kThreads), 0, s, kp);
     else
         hipLaunchKernelGGL((mfma_fwd_kernel<128>), grid, dim3(kThreads), 0, s, kp);

@@ -312,3 +312,17 @@ def test_torch_compile_fullgraph_matches_eager():
     compiled = run(torch.compile(f, fullgraph=True))
     for a, b in zip(eager, compiled):
         assert torch.equal(a, b)
+
+
+def test_small_and_large_grids_take_different_forward_kernels_and_agree():
+    # <= 1024 workgroups: two-step-per-iteration forward; above: one step per iteration.
+    # Same rows computed both ways (a batch of 1 vs the same sequence repeated 40 times).
+    sb_attn, _ = _ops()
+    q, k, v = (randn((1, 4, 1000, 64), 110 + i, 0.5, torch.bfloat16).cuda() for i in range(3))
+    o1, r1 = sb_attn(q, k, v)                                   # 8 row-blocks x 4 heads = 32 workgroups
+    qq, kk, vv = (x.expand(40, -1, -1, -1).contiguous() for x in (q, k, v))
+    o2, r2 = sb_attn(qq, kk, vv)                                # 1280 workgroups
+    assert max_abs(o1.float(), o2[:1].float()) <= 2e-2 and max_abs(r1.float(), r2[:1].float()) <= 1e-2
+    assert torch.equal(o2[0], o2[39]) and torch.equal(r2[0], r2[39])
+    o_ref, rem_ref = O.sb_attn_oracle(q.cpu(), k.cpu(), v.cpu())
+    assert max_abs(o2[39:].float().cpu(), o_ref) <= 2e-2 and max_abs(r2[39:].float().cpu(), rem_ref) <= 2e-2
