@@ -78,6 +78,15 @@ template <int D> struct LaneOffsets {
     }
 };
 
+// Wait for every outstanding global load and store of this wave.  The compiler's wait-count
+// bookkeeping merges control-flow paths pessimistically: a register loaded before a loop, or
+// on a path that skips the instruction consuming it, counts as "perhaps still in flight" in
+// every iteration, and the first read (or reload) of it then waits for ALL memory traffic,
+// the loop's own prefetches included.  An explicit wait in front of such a loop and at the
+// end of each iteration (where everything has long arrived) keeps the loop body free of
+// those waits.
+__device__ inline void wait_global_memory() { __builtin_amdgcn_s_waitcnt(0x0F70); }   // vmcnt(0)
+
 __device__ inline s16x4 lds_read_tr(const char* p) {
     return __builtin_amdgcn_ds_read_tr16_b64_v4i16(
         (__attribute__((address_space(3))) s16x4*)(uintptr_t)(uint32_t)(uintptr_t)p);
@@ -152,6 +161,14 @@ template <int D> struct TileCopy {
         for (int r = 0; r < kPerThread; ++r)
             *(u32x4*)(tile + tile_offset<D>(mfma_row_of_key(kl + r * kRowStep), c)) = regs[r];
     }
+    // rows kept in their natural order (query tiles)
+    __device__ inline void store_nat(char* tile) const {
+        const int tid = threadIdx.x & (kThreads - 1);
+        const int kl = tid / (D / 8), c = tid % (D / 8);
+#pragma unroll
+        for (int r = 0; r < kPerThread; ++r)
+            *(u32x4*)(tile + tile_offset<D>(kl + r * kRowStep, c)) = regs[r];
+    }
 };
 
 // A operand, row fetch: lane (m = lane%32, h = lane/32) gets 8 bf16 of row 32*t + m,
@@ -179,6 +196,30 @@ template <int D> __device__ inline bf16x8 fetch_cols(const char* tile, int db, i
             (__attribute__((address_space(3))) s16x4*)(uintptr_t)(uint32_t)(uintptr_t)p);
     }
     return u.b;
+}
+
+// Epilogue of the key-owner kernels.  An accumulator tile (lane (n, h), register r -> row
+// 8*(r/4) + 4*h + r%4, column n) written straight to global memory is 16 two-byte stores per
+// lane that each touch 64 cache lines; going through a [rows][D] bf16 staging tile in LDS
+// turns a 64-row block into two 16-byte, fully coalesced stores per thread.
+template <int D>
+__device__ inline void stage_acc_tile(char* staging, int row0, int col0, const f32x16& acc, float scale, int lane) {
+    const int n = lane & 31, h = lane >> 5;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+        const int row = row0 + 8 * (r >> 2) + 4 * h + (r & 3);
+        *(uint16_t*)(staging + row * (D * 2) + (col0 + n) * 2) = f32_to_bf16(acc[r] * scale);
+    }
+}
+// 64 staged rows -> rows row0.. of a [rows, D] tensor; `tid` of `n_threads` threads take part.
+template <int D>
+__device__ inline void store_staged_rows(const char* staging, const TensorArg& t, int64_t base, int row0, int len,
+                                         int tid, int n_threads) {
+    for (int c = tid; c < 64 * D / 8; c += n_threads) {
+        const int row = c / (D / 8), cc = c % (D / 8);
+        if (row0 + row < len)
+            *(u32x4*)(t.ptr + 2 * (base + (int64_t)(row0 + row) * t.st + cc * 8)) = *(const u32x4*)(staging + row * (D * 2) + cc * 16);
+    }
 }
 
 // B operand kept in registers for the whole sweep: row `row` of a [rows, D] tensor,

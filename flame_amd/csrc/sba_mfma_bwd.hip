@@ -22,6 +22,7 @@ namespace sba {
 // ---------------------------------------------------------------- pass 1: dQ + prefix table
 template <int D>
 __global__ __launch_bounds__(kThreads) void mfma_bwd_dq_kernel(KParams p) {
+    if (blockIdx.x == 0 && threadIdx.x == 0 && p.counter) *p.counter = 0;   // for the dK/dV kernel that follows
     constexpr int kTile = 64 * D * 2;
     __shared__ __attribute__((aligned(16))) char lds[4 * kTile];   // K0 V0 K1 V1
 
@@ -74,6 +75,7 @@ __global__ __launch_bounds__(kThreads) void mfma_bwd_dq_kernel(KParams p) {
     const int64_t tstride = p.tab_tokens;
     const int64_t tix0 = (int64_t)head * p.n_kb * p.tab_tokens + tabtok;
     float Rnext = (row_ok && n_steps > 0) ? p.rtab[tix0] : 1.0f;
+    wait_global_memory();
     for (int step = 0, buf = 0; step < n_steps; ++step, buf ^= 1) {
         const char* ktile = lds + buf * 2 * kTile;
         const char* vtile = ktile + kTile;
@@ -110,6 +112,7 @@ mask_step(x, key0 + 32 * h, qi, strict);
             kc.store(lds + (buf ^ 1) * 2 * kTile);
             vc.store(lds + (buf ^ 1) * 2 * kTile + kTile);
         }
+        wait_global_memory();                  // nothing in flight across the back edge
         __syncthreads();
     }
 
@@ -197,7 +200,8 @@ __global__ __launch_bounds__(kThreads, 2) void mfma_bwd_dkv_kernel(KParams p) {
 
     const int qb0 = job.rb;
     // prefetched state of the first step
-    float Rn = 1.0f, Gn = 0.0f, drn = 0.0f;
+    float Rn = 1.0f, Gn = 0.0f;
+    uint32_t drn = 0;                          // bf16 bits, widened where used: converting here would wait for the load
     bf16x8 qfn[D / 16];
     {
         const int qi0 = qb0 * kRowBlock + 32 * wave + n;
@@ -205,11 +209,12 @@ __global__ __launch_bounds__(kThreads, 2) void mfma_bwd_dkv_kernel(KParams p) {
         if (qi0 < job.len) {
             const int64_t t = trow + tab_token(p, job, qi0);
             Rn = p.rtab[t]; Gn = p.gtab[t];
-            if (p.d_rem.ptr) drn = Elem<uint16_t>::load(p.d_rem.ptr, dr_base + qi0);
+            if (p.d_rem.ptr) drn = ((const uint16_t*)p.d_rem.ptr)[dr_base + qi0];
         }
     }
     __syncthreads();                           // K, V tiles visible
 
+    wait_global_memory();
     for (int qb = qb0; qb < n_qb; ++qb) {
         const int m0 = qb * kRowBlock;
         const int q0w = m0 + 32 * wave;
@@ -222,15 +227,16 @@ __global__ __launch_bounds__(kThreads, 2) void mfma_bwd_dkv_kernel(KParams p) {
 #pragma unroll
         for (int ks = 0; ks < D / 16; ++ks) qf[ks] = qfn[ks];
         load_row_frags<D>(dof, p.d_o, dobase, qi, job.len, lane);
-        float R = Rn, Gc = Gn, dr = drn;
+        float R = Rn, Gc = Gn;
+        const uint32_t dr_bits = drn;
         if (qb + 1 < n_qb) {
             const int qin = qi + kRowBlock;
             load_row_frags<D>(qfn, p.q, qbase, qin, job.len, lane);
-            Rn = 1.0f; Gn = 0.0f; drn = 0.0f;
+            Rn = 1.0f; Gn = 0.0f; drn = 0;
             if (qin < job.len) {
                 const int64_t t = trow + tab_token(p, job, qin);
                 Rn = p.rtab[t]; Gn = p.gtab[t];
-                if (p.d_rem.ptr) drn = Elem<uint16_t>::load(p.d_rem.ptr, dr_base + qin);
+                if (p.d_rem.ptr) drn = ((const uint16_t*)p.d_rem.ptr)[dr_base + qin];
             }
         }
         // (2) row 32*wave + n of the shared Q tile (every wave passed the barrier that ends the
@@ -249,7 +255,7 @@ __global__ __launch_bounds__(kThreads, 2) void mfma_bwd_dkv_kernel(KParams p) {
 #pragma unroll
             for (int ks = 0; ks < D / 16; ++ks)
                 *(bf16x8*)(dotile + tile_offset<D>(32 * wave + n, 2 * ks + h)) = dof[ks];
-            dp_tiles_o<D>(dp, vtile, lo, dof, dr);
+            dp_tiles_o<D>(dp, vtile, lo, dof, bf16_to_f32((uint16_t)dr_bits));
             logit_grads<true>(x, beta, dp, Gc, lane);
         } else {
 #pragma unroll
@@ -275,28 +281,396 @@ __global__ __launch_bounds__(kThreads, 2) void mfma_bwd_dkv_kernel(KParams p) {
                 dvacc[i] = mfma(ap, fetch_nat_2<D>(dotile, qb0o[i], qb1o[i], 16 * c2), dvacc[i]);
             }
         }
+        wait_global_memory();                  // nothing in flight across the back edge
         __syncthreads();                       // reduction done: tiles may be overwritten
     }
-    // accumulator layout: lane (n = d within the block, h), register r -> key 8*(r/4) + 4*h + r%4
-    // of this wave's 32 keys (the weight tiles are in natural key order)
+    // accumulator rows are keys 32*kh + ..., columns d = 32*(dbw + 2*i) + n (the weight tiles
+    // are in natural key order); the last barrier of the loop has freed the weight tiles
+    char* stage_k = zp;                        // [64 keys][D] bf16 each: kZTile >= kTile
+    char* stage_v = zd;
 #pragma unroll
-    for (int i = 0; i < D / 64; ++i)
+    for (int i = 0; i < D / 64; ++i) {
+        stage_acc_tile<D>(stage_k, 32 * kh, 32 * (dbw + 2 * i), dkacc[i], p.scale, lane);
+        stage_acc_tile<D>(stage_v, 32 * kh, 32 * (dbw + 2 * i), dvacc[i], 1.0f, lane);
+    }
+    __syncthreads();
+    const int64_t dkbase = (int64_t)job.seq * p.dk.sb + (int64_t)head * p.dk.sh + (int64_t)job.tok0 * p.dk.st;
+    const int64_t dvbase = (int64_t)job.seq * p.dv.sb + (int64_t)head * p.dv.sh + (int64_t)job.tok0 * p.dv.st;
+    store_staged_rows<D>(stage_k, p.dk, dkbase, key0, job.len, threadIdx.x, kThreads);
+    store_staged_rows<D>(stage_v, p.dv, dvbase, key0, job.len, threadIdx.x, kThreads);
+}
+
+// ---------------------------------------------------------------- pass 2, head_dim 64
+// dK/dV as ONE resident workgroup per CU that pulls (key block, head) items from a global
+// counter and runs them back to back as a single stream of 128-query steps, with the two
+// halves of a step given to different waves:
+//   waves 0..3 ("producers") turn 32 queries x 64 keys each into weights and logit gradients
+//     and leave them, as bf16 [query][key] rows, in one of two LDS buffers;
+//   waves 4..7 ("consumers") reduce the buffer of the previous step into dK and dV with
+//     MFMAs, and stage what the next step needs (Q / dO tiles, per-query carries, and at an
+//     item boundary the next K / V tiles) from global memory into LDS with coalesced loads.
+// A SIMD holds one wave of each kind, so matrix and memory work run under the producers'
+// vector work, and because the stream never stops at an item boundary nothing of an item's
+// set-up (launch, K/V fetch, first tiles) or tear-down (dK/dV store) is exposed.
+//
+// One iteration s of the stream (barrier B in its middle, A at its end):
+//   producers:  fragments of tile[s&1] -> scores, weights, dP      | B | dz -> Z[s&1]            | A
+//   consumers:  store a staged dK/dV; request step s+1;
+//               reduce Z/tile[(s-1)&1]                            | B | stage a finished dK/dV
+//                                                                       into Z[(s-1)&1];
+//                                                                       deposit step s+1 -> [(s+1)&1] | A
+// B separates the reduction's last read of buffer (s-1)&1 from the stores that reuse it.
+// An item's accumulators are complete after the reduction that follows its last step; they are
+// staged after that iteration's B and written to global memory before the next iteration's B.
+struct KeyItem {
+    Job job;
+    int head, kb, key0, n_steps;
+    bool valid;
+};
+
+__device__ inline KeyItem decode_item(const KParams& p, int idx) {
+    KeyItem r;
+    r.valid = idx >= 0;
+    if (idx < 0) idx = 0;
+    r.head = idx % p.n_heads;
+    const int slot = idx / p.n_heads;          // two 64-key blocks per scheduled 128-row job
+    r.job = decode_job(p, order_job(slot >> 1, p.n_jobs, true));
+    r.kb = 2 * r.job.rb + (slot & 1);
+    r.key0 = r.kb * kKeyBlock;
+    r.n_steps = (r.job.len + kRowBlock - 1) / kRowBlock - r.job.rb;
+    return r;
+}
+
+template <int D>
+__global__ __launch_bounds__(2 * kThreads, 2) void mfma_bwd_dkv_stream_kernel(KParams p) {
+    constexpr int kTile = 64 * D * 2;          // K or V tile (64 keys)
+    constexpr int kQTile = 128 * D * 2;        // Q or dO tile (128 queries)
+    constexpr int kZTile = 128 * 64 * 2;       // weights of one step, [query][key] bf16
+    constexpr int kBuf = 2 * kZTile + 2 * kQTile;
+    constexpr int kCarry = kRowBlock * 16;     // {R, G, d_rem, -} per query
+    __shared__ __attribute__((aligned(1024))) char lds[3 * kTile + 2 * kCarry + 2 * kBuf];
+    __shared__ int slots[4];                   // ring of item indices handed out by the fetcher
+    char* vtiles = lds;                        // V of item j in vtiles + (j&1)*kTile
+    char* ktile = vtiles + 2 * kTile;          // read once per item, into the producers' registers
+    char* carry = ktile + kTile;
+    char* bufs = carry + 2 * kCarry;           // per buffer: zp, zd, qtile, dotile
+
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const bool producer = wave < 4;
+    const int w4 = wave & 3;
+    const int n = lane & 31, h = lane >> 5;
+    const int strict = p.attend_current ? 0 : 1;
+    const int n_items = 2 * p.n_jobs * p.n_heads;
+    const bool fetcher = threadIdx.x == kThreads;
+
+    // Items are taken in list order (longest sweeps first).  A job's second key block can lie
+    // beyond the end of its sequence: such an item runs like any other, its one step finds
+    // nothing to do and nothing is stored, which is cheaper than teaching the pipeline to skip.
+    const int G = gridDim.x, g = blockIdx.x;
+    // items of class c = index % 8 go to the workgroups of XCD c (workgroups are dealt to the
+    // XCDs round-robin): with the head count a multiple of 8 a head's K, V, Q, dO and carries
+    // then stay in one XCD's L2.  Inside a class the workgroups walk the list boustrophedon,
+    // which evens out the sweep lengths (the list is sorted by them).
+    const int W = G >> 3, w = g >> 3, c8 = g & 7;
+    auto static_item = [&](int r) { const int i = 8 * (r * W + ((r & 1) ? W - 1 - w : w)) + c8; return i < n_items ? i : -1; };
+    if (fetcher) {
+        slots[0] = static_item(0);
+        slots[1] = static_item(1);
+    }
+    __syncthreads();
+    KeyItem cur = decode_item(p, __builtin_amdgcn_readfirstlane(slots[0]));
+    if (!cur.valid) return;                    // uniform over the workgroup
+    KeyItem nxt = decode_item(p, __builtin_amdgcn_readfirstlane(slots[1]));
+    int ring = 2;                              // slot that is filled while `cur` runs
+
+    if (producer) {
+        LaneOffsets<D> lo;
+        lo.init(lane);
+        __syncthreads();                       // first item's tiles and carries visible
+        int s = 0;
+        for (int item = 0;; ++item) {
+            const char* vtile = vtiles + (item & 1) * kTile;
+            // the key block of an item never changes: its score operands stay in registers
+            bf16x8 kfr[2][D / 16];
 #pragma unroll
-        for (int r = 0; r < 16; ++r) {
-            int key = key0 + 32 * kh + 8 * (r >> 2) + 4 * h + (r & 3);
-            if (key < job.len) {
-                int d = 32 * (dbw + 2 * i) + n;
-                int64_t kof = (int64_t)job.seq * p.dk.sb + (int64_t)head * p.dk.sh + (int64_t)(job.tok0 + key) * p.dk.st + d;
-                int64_t vof = (int64_t)job.seq * p.dv.sb + (int64_t)head * p.dv.sh + (int64_t)(job.tok0 + key) * p.dv.st + d;
-                Elem<uint16_t>::store(p.dk.ptr, kof, dkacc[i][r] * p.scale);
-                Elem<uint16_t>::store(p.dv.ptr, vof, dvacc[i][r]);
+            for (int t = 0; t < 2; ++t)
+#pragma unroll
+                for (int ks = 0; ks < D / 16; ++ks) kfr[t][ks] = fetch_rows_o<D>(ktile, lo, t, ks);
+            const int key0 = cur.key0;
+            const int len = cur.job.len;
+            for (int it = 0; it < cur.n_steps; ++it, ++s) {
+                char* zp = bufs + (s & 1) * kBuf;
+                char* zd = zp + kZTile;
+                const char* qtile = zd + kZTile;
+                const char* dotile = qtile + kQTile;
+                const int q0w = (cur.job.rb + it) * kRowBlock + 32 * w4;
+                const int qi = q0w + n;
+                const bool skip = key0 + strict > q0w + 31 || q0w >= len;
+                float x[32], beta[32], dp[32];
+                float Gc = 0.f;
+                if (!skip) {
+                    const float4 cv = *(const float4*)(carry + (s & 1) * kCarry + (32 * w4 + n) * 16);
+                    // rows past the end of the sequence hold copies of its last row: a zero carry
+                    // makes their weights and gradients exactly zero
+                    float R = qi < len ? cv.x : 0.f;
+                    Gc = qi < len ? cv.y : 0.f;
+                    bf16x8 qf[D / 16];
+#pragma unroll
+                    for (int ks = 0; ks < D / 16; ++ks) qf[ks] = fetch_rows_o<D>(qtile, lo, w4, ks);
+                    f32x16 raw[2];
+#pragma unroll
+                    for (int t = 0; t < 2; ++t) {
+                        f32x16 acc = {0};
+#pragma unroll
+                        for (int ks = 0; ks < D / 16; ++ks) acc = mfma(kfr[t][ks], qf[ks], acc);
+                        raw[t] = acc;
+                    }
+                    scale_scores(x, raw, p.scale2);
+                    if (key0 + 63 + strict > q0w) mask_step(x, key0 + 32 * h, qi, strict);
+                    stick_weights<true>(x, beta, R, lane);
+                    bf16x8 dof[D / 16];
+#pragma unroll
+                    for (int ks = 0; ks < D / 16; ++ks) dof[ks] = fetch_rows_o<D>(dotile, lo, w4, ks);
+                    dp_tiles_o<D>(dp, vtile, lo, dof, bf16_to_f32((uint16_t)__float_as_uint(cv.z)));
+                }
+                __syncthreads();               // B
+                if (!skip) {
+                    logit_grads<true>(x, beta, dp, Gc, lane);
+                } else {
+#pragma unroll
+                    for (int idx = 0; idx < 32; ++idx) { x[idx] = 0.f; dp[idx] = 0.f; }
+                }
+#pragma unroll
+                for (int c = 0; c < 4; ++c) {
+                    *(bf16x8*)(zp + tile_offset<64>(32 * w4 + n, 4 * h + c)) = pack8(&x[8 * c]);
+                    *(bf16x8*)(zd + tile_offset<64>(32 * w4 + n, 4 * h + c)) = pack8(&dp[8 * c]);
+                }
+                __syncthreads();               // A
             }
+            if (!nxt.valid) break;
+            cur = nxt;
+            nxt = decode_item(p, __builtin_amdgcn_readfirstlane(slots[ring & 3]));
+            ++ring;
         }
+        __syncthreads();                       // B of the draining iteration
+        __syncthreads();                       // A
+    } else {
+        LaneOffsets<D> lo;
+        lo.init(lane);
+        LaneOffsets<64> lz;                    // the weight tiles have 64-key rows whatever D is
+        lz.init(lane);
+        const int ct = threadIdx.x & (kThreads - 1);
+        const int kh = w4 & 1;                 // which 32 keys this wave reduces
+        const int dbw = w4 >> 1;               // and which d-blocks: dbw + 2*i
+        const int za0 = pick_nat<64>(lz, 0, kh), za1 = pick_nat<64>(lz, 1, kh);
+        int qb0o[D / 64], qb1o[D / 64];
+#pragma unroll
+        for (int i = 0; i < D / 64; ++i) { qb0o[i] = pick_nat<D>(lo, 0, dbw + 2 * i); qb1o[i] = pick_nat<D>(lo, 1, dbw + 2 * i); }
+        f32x16 dkacc[D / 64], dvacc[D / 64];
+#pragma unroll
+        for (int i = 0; i < D / 64; ++i) { dkacc[i] = f32x16{0}; dvacc[i] = f32x16{0}; }
+
+        // Staging registers of one step: thread ct holds chunk ct%8 of rows ct/8 + 32*part of the
+        // Q and dO tiles, and (ct < 128) the carries of query ct.  Every request is
+        // unconditional, with rows clamped to the sequence, and every iteration consumes what
+        // it requested: no register is "perhaps still being loaded" on some path, so the
+        // compiler's wait-count bookkeeping stays exact.
+        u32x4 tq[4], td[4];
+        float cR, cG;
+        uint32_t cdr = 0;                      // bf16 bits
+        const int crow = ct >> 3, cch = ct & 7;
+        // The tile requests of a step are issued two at a time between the MFMAs of the
+        // reduction: all CUs stream their tiles from L2 in the same phase of a step, the
+        // memory pipe then accepts about one 1 KB wave load per 80 cycles, and a burst of
+        // eight would stall this wave on a full queue.
+        // Per-item base pointers, worked out once per item: a step's requests then cost a few
+        // vector instructions and no 64-bit scalar arithmetic (a wave issues one instruction
+        // every four or five cycles, scalar ones included, and the consumers' share of a step
+        // is short).
+        struct ItemPtrs {
+            const char *q, *d_o;               // row 0 of the sequence, this head
+            const float *rt, *gt;              // carries of this (head, key block), query 0
+            const uint16_t* dr;                // d_rem of the sequence, query 0 (or null)
+            int row0, len;                     // first query of the item's sweep; sequence length
+        };
+        auto item_ptrs = [&](const KeyItem& t) {
+            ItemPtrs r;
+            r.q = p.q.ptr + 2 * ((int64_t)t.job.seq * p.q.sb + (int64_t)t.head * p.q.sh + (int64_t)t.job.tok0 * p.q.st);
+            r.d_o = p.d_o.ptr + 2 * ((int64_t)t.job.seq * p.d_o.sb + (int64_t)t.head * p.d_o.sh + (int64_t)t.job.tok0 * p.d_o.st);
+            const int64_t tk = ((int64_t)t.head * p.n_kb + t.kb) * p.tab_tokens + tab_token(p, t.job, 0);
+            r.rt = p.rtab + tk;
+            r.gt = p.gtab + tk;
+            r.dr = p.d_rem.ptr ? (const uint16_t*)p.d_rem.ptr + ((int64_t)t.job.seq * p.d_rem.sb + (int64_t)t.head * p.d_rem.sh + t.job.tok0) : nullptr;
+            r.row0 = t.job.rb * kRowBlock;
+            r.len = t.job.len;
+            return r;
+        };
+        const uint32_t q_st2 = 2u * (uint32_t)p.q.st, do_st2 = 2u * (uint32_t)p.d_o.st;
+        auto request_tile = [&](const ItemPtrs& t, int row0, int part) {
+            const uint32_t row = (uint32_t)min(row0 + crow + 32 * part, t.len - 1);
+            tq[part] = *(const u32x4*)(t.q + (size_t)(row * q_st2 + cch * 16));
+            td[part] = *(const u32x4*)(t.d_o + (size_t)(row * do_st2 + cch * 16));
+        };
+        auto request_carry = [&](const ItemPtrs& t, int row0) {
+            const int qi = min(row0 + (ct & (kRowBlock - 1)), t.len - 1);
+            cR = t.rt[qi]; cG = t.gt[qi];
+            if (t.dr) cdr = t.dr[qi];
+        };
+        // K and V tiles of an item go straight from global memory into LDS (no registers, and
+        // nothing for the wait-count bookkeeping to track): every instruction moves 64 x 16 bytes
+        // into 1 KB of consecutive LDS, the lane picks the global chunk that belongs at its LDS
+        // position (rows in MFMA order, chunks swizzled).  Rows past the end are clamped: those
+        // keys are masked for every valid query and their dK/dV rows are not stored.
+        auto request_keys = [&](const KeyItem& t, char* vdst) {
+            const int64_t kbase = (int64_t)t.job.seq * p.k.sb + (int64_t)t.head * p.k.sh + (int64_t)t.job.tok0 * p.k.st;
+            const int64_t vbase = (int64_t)t.job.seq * p.v.sb + (int64_t)t.head * p.v.sh + (int64_t)t.job.tok0 * p.v.st;
+#pragma unroll
+            for (int i2 = 0; i2 < 2; ++i2) {
+                const int inst = w4 + 4 * i2;              // 8 instructions per tile over 4 waves
+                const int pos = inst * 64 + lane;          // LDS chunk position
+                const int r = pos / (D / 8), pc = pos % (D / 8);
+                const int c = pc ^ swz<D>(r);
+                const int kl = (((r >> 2) & 1) << 5) | (((r >> 5) & 1) << 4) | (((r >> 3) & 3) << 2) | (r & 3);
+                const int row = min(t.key0 + kl, t.job.len - 1);
+                __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(p.k.ptr + 2 * (kbase + (int64_t)row * p.k.st + c * 8)),
+                                                 (__attribute__((address_space(3))) void*)(uintptr_t)(uint32_t)(uintptr_t)(ktile + inst * 1024),
+                                                 16, 0, 0);
+                __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(p.v.ptr + 2 * (vbase + (int64_t)row * p.v.st + c * 8)),
+                                                 (__attribute__((address_space(3))) void*)(uintptr_t)(uint32_t)(uintptr_t)(vdst + inst * 1024),
+                                                 16, 0, 0);
+            }
+        };
+        auto deposit = [&](int s) {
+            char* qtile = bufs + (s & 1) * kBuf + 2 * kZTile;
+            char* dotile = qtile + kQTile;
+#pragma unroll
+            for (int part = 0; part < 4; ++part) {
+                *(u32x4*)(qtile + tile_offset<D>(crow + 32 * part, cch)) = tq[part];
+                *(u32x4*)(dotile + tile_offset<D>(crow + 32 * part, cch)) = td[part];
+            }
+            if (ct < kRowBlock)
+                *(float4*)(carry + (s & 1) * kCarry + ct * 16) = float4{cR, cG, __uint_as_float(cdr), 0.f};
+        };
+        auto store_staged = [&](const KeyItem& t, const char* staging) {
+            const int64_t dkbase = (int64_t)t.job.seq * p.dk.sb + (int64_t)t.head * p.dk.sh + (int64_t)t.job.tok0 * p.dk.st;
+            const int64_t dvbase = (int64_t)t.job.seq * p.dv.sb + (int64_t)t.head * p.dv.sh + (int64_t)t.job.tok0 * p.dv.st;
+            store_staged_rows<D>(staging, p.dk, dkbase, t.key0, t.job.len, ct, kThreads);
+            store_staged_rows<D>(staging + kTile, p.dv, dvbase, t.key0, t.job.len, ct, kThreads);
+        };
+        auto stage = [&](char* staging) {
+#pragma unroll
+            for (int i = 0; i < D / 64; ++i) {
+                stage_acc_tile<D>(staging, 32 * kh, 32 * (dbw + 2 * i), dkacc[i], p.scale, lane);
+                stage_acc_tile<D>(staging + kTile, 32 * kh, 32 * (dbw + 2 * i), dvacc[i], 1.0f, lane);
+                dkacc[i] = f32x16{0};
+                dvacc[i] = f32x16{0};
+            }
+        };
+        auto reduce = [&](int s_done, auto&& between) {
+            const char* zp = bufs + (s_done & 1) * kBuf;
+            const char* zd = zp + kZTile;
+            const char* qtile = zd + kZTile;
+            const char* dotile = qtile + kQTile;
+            // dK[key][d] += sum_q dz[q][key] Q[q][d];  dV[key][d] += sum_q a[q][key] dO[q][d]
+#pragma unroll
+            for (int c2 = 0; c2 < 8; ++c2) {
+                if ((c2 & 1) == 0) {
+                    between(c2 >> 1);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+                bf16x8 az = fetch_nat_2<64>(zd, za0, za1, 16 * c2);
+                bf16x8 ap = fetch_nat_2<64>(zp, za0, za1, 16 * c2);
+#pragma unroll
+                for (int i = 0; i < D / 64; ++i) {
+                    dkacc[i] = mfma(az, fetch_nat_2<D>(qtile, qb0o[i], qb1o[i], 16 * c2), dkacc[i]);
+                    dvacc[i] = mfma(ap, fetch_nat_2<D>(dotile, qb0o[i], qb1o[i], 16 * c2), dvacc[i]);
+                }
+            }
+        };
+
+        ItemPtrs cp = item_ptrs(cur), np = item_ptrs(nxt);
+        request_keys(cur, vtiles);
+#pragma unroll
+        for (int part = 0; part < 4; ++part) request_tile(cp, cp.row0, part);
+        request_carry(cp, cp.row0);
+        deposit(0);
+        wait_global_memory();
+        __syncthreads();                       // first item's tiles and carries visible
+
+        int s = 0;
+        bool finish_after_reduce = false;      // the step about to be reduced is its item's last
+        bool store_pending = false;            // a staged dK/dV waits in Z[s&1] to be stored
+        KeyItem fin_stage = cur, fin_store = cur;
+        for (int item = 0;; ++item) {
+            // index of the item after next
+            if (fetcher) slots[ring & 3] = static_item(ring);
+            // the next item's K and V are requested after B of the second-to-last step: K's tile
+            // is free once the producers have taken their fragments (before the item's first B),
+            // V goes to the tile of the other parity
+            const int keys_at = cur.n_steps >= 2 ? cur.n_steps - 2 : 0;
+            for (int it = 0; it < cur.n_steps; ++it, ++s) {
+                const bool last = it + 1 == cur.n_steps;
+                // what the stream's next step needs; at the very end, a harmless repeat
+                const ItemPtrs& rq = (last && nxt.valid) ? np : cp;
+                const int rq_row0 = last ? rq.row0 : cp.row0 + (it + 1) * kRowBlock;
+                if (store_pending) {           // staged in the previous iteration
+                    store_staged(fin_store, bufs + (s & 1) * kBuf);
+                    store_pending = false;
+                }
+                request_carry(rq, rq_row0);
+                if (s > 0) {
+                    reduce(s - 1, [&](int part) { request_tile(rq, rq_row0, part); });
+                } else {
+#pragma unroll
+                    for (int part = 0; part < 4; ++part) request_tile(rq, rq_row0, part);
+                }
+                __syncthreads();               // B: every consumer has finished with buffer (s-1)&1
+                if (it == keys_at && nxt.valid) request_keys(nxt, vtiles + ((item + 1) & 1) * kTile);
+                if (finish_after_reduce) {
+                    stage(bufs + ((s - 1) & 1) * kBuf);
+                    fin_store = fin_stage;
+                    store_pending = true;
+                }
+                deposit(s + 1);
+                finish_after_reduce = last;
+                if (last) fin_stage = cur;
+                wait_global_memory();          // nothing in flight across the back edge
+                __syncthreads();               // A
+            }
+            if (!nxt.valid) break;
+            cur = nxt;
+            nxt = decode_item(p, __builtin_amdgcn_readfirstlane(slots[ring & 3]));
+            ++ring;
+            cp = np;
+            np = item_ptrs(nxt);
+        }
+        // draining iteration: the last step of the last item
+        if (store_pending) store_staged(fin_store, bufs + (s & 1) * kBuf);
+        reduce(s - 1, [&](int) {});
+        __syncthreads();                       // B
+        stage(bufs + ((s - 1) & 1) * kBuf);
+        __syncthreads();                       // A (consumers only need each other's staging)
+        store_staged(fin_stage, bufs + ((s - 1) & 1) * kBuf);
+    }
 }
 
 }  // namespace sba
 
 bool sba_mfma_bwd_available() { return true; }
+
+// compute units of the current device (asked once per device)
+static int sba_cu_count() {
+    static int cached[64] = {0};
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) dev = 0;
+    if (cached[dev] == 0) {
+        int n = 0;
+        if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
+        cached[dev] = n;
+    }
+    return cached[dev];
+}
 
 int sba_launch_mfma_bwd(const sba::KParams& kp, int phases, hipStream_t s) {
     using namespace sba;
@@ -304,7 +678,14 @@ int sba_launch_mfma_bwd(const sba::KParams& kp, int phases, hipStream_t s) {
     const bool p1 = phases != 2, p2 = phases != 1;
     if (kp.head_dim == 64) {
         if (p1) hipLaunchKernelGGL((mfma_bwd_dq_kernel<64>), grid, dim3(kThreads), 0, s, kp);
-        if (p2) hipLaunchKernelGGL((mfma_bwd_dkv_kernel<64>), dim3(2 * grid.x), dim3(kThreads), 0, s, kp);
+        if (p2) {
+            // one resident workgroup per CU; the items are handed out through kp.counter,
+            // which the dQ kernel of the same backward has reset
+            const unsigned n_items = 2 * grid.x;
+            unsigned n_wg = n_items < (unsigned)sba_cu_count() ? n_items : (unsigned)sba_cu_count();
+            n_wg = (n_wg + 7) & ~7u;           // whole XCD rounds (surplus workgroups find no item)
+            hipLaunchKernelGGL((mfma_bwd_dkv_stream_kernel<64>), dim3(n_wg), dim3(2 * kThreads), 0, s, kp);
+        }
     } else {
         if (p1) hipLaunchKernelGGL((mfma_bwd_dq_kernel<128>), grid, dim3(kThreads), 0, s, kp);
         if (p2) hipLaunchKernelGGL((mfma_bwd_dkv_kernel<128>), dim3(2 * grid.x), dim3(kThreads), 0, s, kp);

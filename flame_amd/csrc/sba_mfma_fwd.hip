@@ -49,6 +49,7 @@ __global__ __launch_bounds__(kThreads) void mfma_fwd_kernel(KParams p) {
     }
     __syncthreads();
 
+    wait_global_memory();
     for (int step = n_steps - 1, buf = 0; step >= 0; --step, buf ^= 1) {
         const char* ktile = lds + buf * 2 * kTile;
         const char* vtile = ktile + kTile;
@@ -86,6 +87,7 @@ mask_step(x, key0 + 32 * h, qi, strict);
             kc.store(lds + (buf ^ 1) * 2 * kTile);
             vc.store(lds + (buf ^ 1) * 2 * kTile + kTile);
         }
+        wait_global_memory();                  // nothing in flight across the back edge
         __syncthreads();
     }
 
@@ -168,6 +170,7 @@ __global__ __launch_bounds__(2 * kThreads) void mfma_fwd2_kernel(KParams p) {
     }
     __syncthreads();
 
+    wait_global_memory();
     for (int it = 0, buf = 0; it < n_it; ++it, buf ^= 1) {
         const int step = n_steps - 1 - 2 * it - grp;          // -1: this group idles in the last iteration
         const char* ktile = my_tiles + buf * 4 * kTile;
@@ -211,6 +214,7 @@ __global__ __launch_bounds__(2 * kThreads) void mfma_fwd2_kernel(KParams p) {
             kc.store(my_tiles + (buf ^ 1) * 4 * kTile);
             vc.store(my_tiles + (buf ^ 1) * 4 * kTile + kTile);
         }
+        wait_global_memory();                  // nothing in flight across the back edge
         __syncthreads();
     }
 
