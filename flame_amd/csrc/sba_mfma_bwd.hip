@@ -379,9 +379,11 @@ __global__ __launch_bounds__(2 * kThreads, 2) void mfma_bwd_dkv_stream_kernel(KP
         slots[1] = static_item(1);
     }
     __syncthreads();
-    KeyItem cur = decode_item(p, __builtin_amdgcn_readfirstlane(slots[0]));
+    int cur_idx = __builtin_amdgcn_readfirstlane(slots[0]);
+    int nxt_idx = __builtin_amdgcn_readfirstlane(slots[1]);
+    KeyItem cur = decode_item(p, cur_idx);
     if (!cur.valid) return;                    // uniform over the workgroup
-    KeyItem nxt = decode_item(p, __builtin_amdgcn_readfirstlane(slots[1]));
+    KeyItem nxt = decode_item(p, nxt_idx);
     int ring = 2;                              // slot that is filled while `cur` runs
 
     if (producer) {
@@ -552,7 +554,8 @@ __global__ __launch_bounds__(2 * kThreads, 2) void mfma_bwd_dkv_stream_kernel(KP
             if (ct < kRowBlock)
                 *(float4*)(carry + (s & 1) * kCarry + ct * 16) = float4{cR, cG, __uint_as_float(cdr), 0.f};
         };
-        auto store_staged = [&](const KeyItem& t, const char* staging) {
+        auto store_staged = [&](int idx, const char* staging) {
+            const KeyItem t = decode_item(p, idx);
             const int64_t dkbase = (int64_t)t.job.seq * p.dk.sb + (int64_t)t.head * p.dk.sh + (int64_t)t.job.tok0 * p.dk.st;
             const int64_t dvbase = (int64_t)t.job.seq * p.dv.sb + (int64_t)t.head * p.dv.sh + (int64_t)t.job.tok0 * p.dv.st;
             store_staged_rows<D>(staging, p.dk, dkbase, t.key0, t.job.len, ct, kThreads);
@@ -567,25 +570,37 @@ __global__ __launch_bounds__(2 * kThreads, 2) void mfma_bwd_dkv_stream_kernel(KP
                 dvacc[i] = f32x16{0};
             }
         };
+        // dK[key][d] += sum_q dz[q][key] Q[q][d];  dV[key][d] += sum_q a[q][key] dO[q][d].
+        // The operands of four 16-query groups are fetched as one batch, so that the MFMAs wait
+        // for LDS once per batch rather than once each; `between(b)` (the tile requests) goes
+        // behind the fetches of batch b.
         auto reduce = [&](int s_done, auto&& between) {
             const char* zp = bufs + (s_done & 1) * kBuf;
             const char* zd = zp + kZTile;
             const char* qtile = zd + kZTile;
             const char* dotile = qtile + kQTile;
-            // dK[key][d] += sum_q dz[q][key] Q[q][d];  dV[key][d] += sum_q a[q][key] dO[q][d]
 #pragma unroll
-            for (int c2 = 0; c2 < 8; ++c2) {
-                if ((c2 & 1) == 0) {
-                    between(c2 >> 1);
-                    __builtin_amdgcn_sched_barrier(0);
-                }
-                bf16x8 az = fetch_nat_2<64>(zd, za0, za1, 16 * c2);
-                bf16x8 ap = fetch_nat_2<64>(zp, za0, za1, 16 * c2);
+            for (int b = 0; b < 2; ++b) {
+                bf16x8 az[4], ap[4], bq[4][D / 64], bd[4][D / 64];
 #pragma unroll
-                for (int i = 0; i < D / 64; ++i) {
-                    dkacc[i] = mfma(az, fetch_nat_2<D>(qtile, qb0o[i], qb1o[i], 16 * c2), dkacc[i]);
-                    dvacc[i] = mfma(ap, fetch_nat_2<D>(dotile, qb0o[i], qb1o[i], 16 * c2), dvacc[i]);
+                for (int j = 0; j < 4; ++j) {
+                    const int c2 = 4 * b + j;
+                    az[j] = fetch_nat_2<64>(zd, za0, za1, 16 * c2);
+                    ap[j] = fetch_nat_2<64>(zp, za0, za1, 16 * c2);
+#pragma unroll
+                    for (int i = 0; i < D / 64; ++i) {
+                        bq[j][i] = fetch_nat_2<D>(qtile, qb0o[i], qb1o[i], 16 * c2);
+                        bd[j][i] = fetch_nat_2<D>(dotile, qb0o[i], qb1o[i], 16 * c2);
+                    }
                 }
+                between(b);
+#pragma unroll
+                for (int j = 0; j < 4; ++j)
+#pragma unroll
+                    for (int i = 0; i < D / 64; ++i) {
+                        dkacc[i] = mfma(az[j], bq[j][i], dkacc[i]);
+                        dvacc[i] = mfma(ap[j], bd[j][i], dvacc[i]);
+                    }
             }
         };
 
@@ -601,46 +616,54 @@ __global__ __launch_bounds__(2 * kThreads, 2) void mfma_bwd_dkv_stream_kernel(KP
         int s = 0;
         bool finish_after_reduce = false;      // the step about to be reduced is its item's last
         bool store_pending = false;            // a staged dK/dV waits in Z[s&1] to be stored
-        KeyItem fin_stage = cur, fin_store = cur;
+        int fin_stage = cur_idx, fin_store = cur_idx;
+        // One iteration of the stream; `rq`, `rq_row0` say what the stream's next step needs.
+        auto iteration = [&](const ItemPtrs& rq, int rq_row0, bool last, bool keys_now, int item) {
+            if (store_pending) {               // staged in the previous iteration
+                store_staged(fin_store, bufs + (s & 1) * kBuf);
+                store_pending = false;
+            }
+            request_carry(rq, rq_row0);
+            if (s > 0) {
+                reduce(s - 1, [&](int b) { request_tile(rq, rq_row0, 2 * b); request_tile(rq, rq_row0, 2 * b + 1); });
+            } else {
+#pragma unroll
+                for (int part = 0; part < 4; ++part) request_tile(rq, rq_row0, part);
+            }
+            __syncthreads();                   // B: every consumer has finished with buffer (s-1)&1
+            if (keys_now) request_keys(decode_item(p, nxt_idx), vtiles + ((item + 1) & 1) * kTile);
+            if (finish_after_reduce) {
+                stage(bufs + ((s - 1) & 1) * kBuf);
+                fin_store = fin_stage;
+                store_pending = true;
+            }
+            deposit(s + 1);
+            finish_after_reduce = last;
+            if (last) fin_stage = cur_idx;
+            wait_global_memory();              // nothing in flight across the back edge
+            __syncthreads();                   // A
+            ++s;
+        };
         for (int item = 0;; ++item) {
             // index of the item after next
             if (fetcher) slots[ring & 3] = static_item(ring);
-            // the next item's K and V are requested after B of the second-to-last step: K's tile
+            // The next item's K and V are requested after B of the second-to-last step: K's tile
             // is free once the producers have taken their fragments (before the item's first B),
-            // V goes to the tile of the other parity
-            const int keys_at = cur.n_steps >= 2 ? cur.n_steps - 2 : 0;
-            for (int it = 0; it < cur.n_steps; ++it, ++s) {
-                const bool last = it + 1 == cur.n_steps;
-                // what the stream's next step needs; at the very end, a harmless repeat
-                const ItemPtrs& rq = (last && nxt.valid) ? np : cp;
-                const int rq_row0 = last ? rq.row0 : cp.row0 + (it + 1) * kRowBlock;
-                if (store_pending) {           // staged in the previous iteration
-                    store_staged(fin_store, bufs + (s & 1) * kBuf);
-                    store_pending = false;
-                }
-                request_carry(rq, rq_row0);
-                if (s > 0) {
-                    reduce(s - 1, [&](int part) { request_tile(rq, rq_row0, part); });
-                } else {
-#pragma unroll
-                    for (int part = 0; part < 4; ++part) request_tile(rq, rq_row0, part);
-                }
-                __syncthreads();               // B: every consumer has finished with buffer (s-1)&1
-                if (it == keys_at && nxt.valid) request_keys(nxt, vtiles + ((item + 1) & 1) * kTile);
-                if (finish_after_reduce) {
-                    stage(bufs + ((s - 1) & 1) * kBuf);
-                    fin_store = fin_stage;
-                    store_pending = true;
-                }
-                deposit(s + 1);
-                finish_after_reduce = last;
-                if (last) fin_stage = cur;
-                wait_global_memory();          // nothing in flight across the back edge
-                __syncthreads();               // A
-            }
-            if (!nxt.valid) break;
+            // V goes to the tile of the other parity.
+            const int n_steps = cur.n_steps;
+            const bool has_next = nxt.valid;
+            const int keys_at = n_steps >= 2 ? n_steps - 2 : 0;
+            for (int it = 0; it + 1 < n_steps; ++it)
+                iteration(cp, cp.row0 + (it + 1) * kRowBlock, false, has_next && it == keys_at, item);
+            // the item's last step: the request is the next item's first step, or at the very end
+            // of the stream a harmless repeat
+            if (has_next) iteration(np, np.row0, true, n_steps - 1 == keys_at, item);
+            else iteration(cp, cp.row0, true, false, item);
+            if (!has_next) break;
+            cur_idx = nxt_idx;
             cur = nxt;
-            nxt = decode_item(p, __builtin_amdgcn_readfirstlane(slots[ring & 3]));
+            nxt_idx = __builtin_amdgcn_readfirstlane(slots[ring & 3]);
+            nxt = decode_item(p, nxt_idx);
             ++ring;
             cp = np;
             np = item_ptrs(nxt);
