@@ -15,7 +15,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "csrc", "libsba_mi355x.so")
 
 SBA_DTYPE_F32, SBA_DTYPE_BF16 = 0, 1
-SBA_ABI_VERSION = 1
+SBA_ABI_VERSION = 2
 
 
 class SbaTensor(C.Structure):
@@ -114,14 +114,17 @@ def usable(t: torch.Tensor) -> torch.Tensor:
     return t if ok else t.contiguous()
 
 
+SCHEDULE_INTS = 5      # int32 per job: first_token, doc_len, row_block, doc_index, key_order
+
+
 def build_schedule(cu_host: torch.Tensor) -> torch.Tensor:
-    """Host int32 cu_seqlens (leading 0) -> host int32 [n_jobs, 4] schedule."""
+    """Host int32 cu_seqlens (leading 0) -> host int32 [n_jobs, 5] schedule."""
     lib = load()
     cu = cu_host.to(torch.int32).contiguous()
     n_seq = cu.numel() - 1
     ptr = C.cast(cu.data_ptr(), C.POINTER(C.c_int32))
     n = lib.sba_build_schedule(ptr, n_seq, None, 0)
-    out = torch.empty((max(n, 1), 4), dtype=torch.int32)
+    out = torch.empty((max(n, 1), SCHEDULE_INTS), dtype=torch.int32)
     got = lib.sba_build_schedule(ptr, n_seq, C.cast(out.data_ptr(), C.POINTER(C.c_int32)), n)
     assert got == n
     return out[:n]

@@ -140,11 +140,18 @@ int sba_build_schedule(const int32_t* cu, int n_seq, int32_t* out, int capacity)
     // longest sweeps first; a stable order keeps the schedule deterministic
     std::stable_sort(jobs.begin(), jobs.end(), [](const J& a, const J& b) { return a.rb > b.rb; });
     int n = (int)jobs.size();
-    if (out && capacity >= n)
+    if (out && capacity >= n) {
+        // column 4: the jobs again, ordered for the key-owner kernels, whose sweep from a
+        // job's row-block to the end of its sequence is (blocks of the sequence - rb) long
+        std::vector<int> key_order(n);
+        for (int i = 0; i < n; ++i) key_order[i] = i;
+        auto key_len = [&](int i) { return (jobs[i].len + sba::kRowBlock - 1) / sba::kRowBlock - jobs[i].rb; };
+        std::stable_sort(key_order.begin(), key_order.end(), [&](int a, int b) { return key_len(a) > key_len(b); });
         for (int i = 0; i < n; ++i) {
-            out[4 * i + 0] = jobs[i].tok0; out[4 * i + 1] = jobs[i].len;
-            out[4 * i + 2] = jobs[i].rb;   out[4 * i + 3] = jobs[i].doc;
+            int32_t* o = out + (size_t)sba::kScheduleInts * i;
+            o[0] = jobs[i].tok0; o[1] = jobs[i].len; o[2] = jobs[i].rb; o[3] = jobs[i].doc; o[4] = key_order[i];
         }
+    }
     return n;
 }
 

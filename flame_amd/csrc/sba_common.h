@@ -41,6 +41,8 @@ struct Job { int tok0, len, rb, seq; };
 // the same job and a head stays on one XCD's L2.  Jobs are sorted by decreasing sweep
 // length (longest first); `longest_last` walks the list from its other end (the key-owner
 // pass, whose work grows as the row-block index falls).
+constexpr int kScheduleInts = 5;   // {first_token, doc_len, row_block, doc_index, key_order} per job
+
 __device__ inline int order_job(int slot, int n_jobs, bool longest_last) {
     return longest_last ? n_jobs - 1 - slot : slot;
 }
@@ -56,10 +58,17 @@ __device__ inline Job decode_job(const KParams& p, int job) {
         j.tok0 = 0;
         j.len = p.seq_len;
     } else {
-        const int32_t* s = p.schedule + 4 * (int64_t)job;
+        const int32_t* s = p.schedule + kScheduleInts * (int64_t)job;
         j.tok0 = s[0]; j.len = s[1]; j.rb = s[2]; j.seq = 0;
     }
     return j;
+}
+
+// The key-owner (dK/dV) kernels sweep from a job's row-block to the END of its sequence:
+// their longest sweeps are the FIRST row-blocks of the longest sequences.  i-th job in that
+// order: arithmetic for the dense layout, column 4 of the host-built schedule for the packed.
+__device__ inline int key_order_job(const KParams& p, int i) {
+    return p.cu_seqlens == nullptr ? p.n_jobs - 1 - i : p.schedule[kScheduleInts * (int64_t)i + 4];
 }
 
 // Token index inside the carry tables.

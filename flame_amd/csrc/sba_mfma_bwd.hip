@@ -167,7 +167,7 @@ __global__ __launch_bounds__(kThreads, 2) void mfma_bwd_dkv_kernel(KParams p) {
     lz.init(lane);
     const int head = blockIdx.x % p.n_heads;
     const int slot = blockIdx.x / p.n_heads;   // two 64-key blocks per scheduled 128-row job
-    const Job job = decode_job(p, order_job(slot >> 1, p.n_jobs, true));
+    const Job job = decode_job(p, key_order_job(p, slot >> 1));
     const int kb = 2 * job.rb + (slot & 1);
     const int key0 = kb * kKeyBlock;
     if (key0 >= job.len) return;               // uniform over the workgroup
@@ -334,7 +334,7 @@ __device__ inline KeyItem decode_item(const KParams& p, int idx) {
     if (idx < 0) idx = 0;
     r.head = idx % p.n_heads;
     const int slot = idx / p.n_heads;          // two 64-key blocks per scheduled 128-row job
-    r.job = decode_job(p, order_job(slot >> 1, p.n_jobs, true));
+    r.job = decode_job(p, key_order_job(p, slot >> 1));
     r.kb = 2 * r.job.rb + (slot & 1);
     r.key0 = r.kb * kKeyBlock;
     r.n_steps = (r.job.len + kRowBlock - 1) / kRowBlock - r.job.rb;
@@ -486,38 +486,42 @@ __global__ __launch_bounds__(2 * kThreads, 2) void mfma_bwd_dkv_stream_kernel(KP
         // reduction: all CUs stream their tiles from L2 in the same phase of a step, the
         // memory pipe then accepts about one 1 KB wave load per 80 cycles, and a burst of
         // eight would stall this wave on a full queue.
-        // Per-item base pointers, worked out once per item: a step's requests then cost a few
-        // vector instructions and no 64-bit scalar arithmetic (a wave issues one instruction
-        // every four or five cycles, scalar ones included, and the consumers' share of a step
-        // is short).
+        // Per-item base pointers, worked out once per item and held in VECTOR registers (which
+        // the consumers have to spare): a step's requests then cost a few vector instructions.
+        // Left to itself the compiler keeps such uniform values in scalar registers, runs out
+        // of them, and re-derives the pointers from the kernel arguments in every iteration
+        // (a wave issues one instruction every four or five cycles, scalar ones included, and
+        // the consumers' share of a step is short).
         struct ItemPtrs {
-            const char *q, *d_o;               // row 0 of the sequence, this head
+            const char *q, *d_o;               // row 0 of the sequence, this head, this thread's chunk
             const float *rt, *gt;              // carries of this (head, key block), query 0
-            const uint16_t* dr;                // d_rem of the sequence, query 0 (or null)
+            const uint16_t* dr;                // d_rem of the sequence, query 0
             int row0, len;                     // first query of the item's sweep; sequence length
         };
+        const bool has_dr = p.d_rem.ptr != nullptr;
         auto item_ptrs = [&](const KeyItem& t) {
             ItemPtrs r;
-            r.q = p.q.ptr + 2 * ((int64_t)t.job.seq * p.q.sb + (int64_t)t.head * p.q.sh + (int64_t)t.job.tok0 * p.q.st);
-            r.d_o = p.d_o.ptr + 2 * ((int64_t)t.job.seq * p.d_o.sb + (int64_t)t.head * p.d_o.sh + (int64_t)t.job.tok0 * p.d_o.st);
+            r.q = p.q.ptr + 2 * ((int64_t)t.job.seq * p.q.sb + (int64_t)t.head * p.q.sh + (int64_t)t.job.tok0 * p.q.st) + cch * 16;
+            r.d_o = p.d_o.ptr + 2 * ((int64_t)t.job.seq * p.d_o.sb + (int64_t)t.head * p.d_o.sh + (int64_t)t.job.tok0 * p.d_o.st) + cch * 16;
             const int64_t tk = ((int64_t)t.head * p.n_kb + t.kb) * p.tab_tokens + tab_token(p, t.job, 0);
             r.rt = p.rtab + tk;
             r.gt = p.gtab + tk;
-            r.dr = p.d_rem.ptr ? (const uint16_t*)p.d_rem.ptr + ((int64_t)t.job.seq * p.d_rem.sb + (int64_t)t.head * p.d_rem.sh + t.job.tok0) : nullptr;
+            r.dr = (const uint16_t*)p.d_rem.ptr + ((int64_t)t.job.seq * p.d_rem.sb + (int64_t)t.head * p.d_rem.sh + t.job.tok0);
             r.row0 = t.job.rb * kRowBlock;
             r.len = t.job.len;
+            asm volatile("" : "+v"(r.q), "+v"(r.d_o), "+v"(r.rt), "+v"(r.gt), "+v"(r.dr));
             return r;
         };
         const uint32_t q_st2 = 2u * (uint32_t)p.q.st, do_st2 = 2u * (uint32_t)p.d_o.st;
         auto request_tile = [&](const ItemPtrs& t, int row0, int part) {
             const uint32_t row = (uint32_t)min(row0 + crow + 32 * part, t.len - 1);
-            tq[part] = *(const u32x4*)(t.q + (size_t)(row * q_st2 + cch * 16));
-            td[part] = *(const u32x4*)(t.d_o + (size_t)(row * do_st2 + cch * 16));
+            tq[part] = *(const u32x4*)(t.q + (size_t)row * q_st2);
+            td[part] = *(const u32x4*)(t.d_o + (size_t)row * do_st2);
         };
         auto request_carry = [&](const ItemPtrs& t, int row0) {
             const int qi = min(row0 + (ct & (kRowBlock - 1)), t.len - 1);
             cR = t.rt[qi]; cG = t.gt[qi];
-            if (t.dr) cdr = t.dr[qi];
+            if (has_dr) cdr = t.dr[qi];
         };
         // K and V tiles of an item go straight from global memory into LDS (no registers, and
         // nothing for the wait-count bookkeeping to track): every instruction moves 64 x 16 bytes

@@ -30,7 +30,7 @@ def test_exports_every_declared_symbol(lib):
 
 
 def test_abi_version_and_struct_size(lib):
-    assert lib.sba_abi_version() == 1
+    assert lib.sba_abi_version() == 2
     p = _lib.SbaParams()
     p.struct_size = C.sizeof(_lib.SbaParams) - 8
     assert lib.sba_fwd(C.byref(p)) == -7          # SBA_ERR_ABI, before anything touches a GPU
@@ -66,15 +66,20 @@ def test_workspace_bytes(lib):
 def test_schedule_builder(lib):
     cu = torch.tensor([0, 100, 400, 401, 1000, 1000], dtype=torch.int32)   # last doc empty
     s = _lib.build_schedule(cu)
-    jobs = [tuple(r) for r in s.tolist()]
+    jobs = [tuple(r[:4]) for r in s.tolist()]
     # every (doc, row_block) exactly once, none for the empty document
     expect = {(0, 100, 0, 0), (100, 300, 0, 1), (100, 300, 1, 1), (100, 300, 2, 1), (400, 1, 0, 2)}
     expect |= {(401, 599, rb, 3) for rb in range(5)}
     assert set(jobs) == expect and len(jobs) == len(expect)
     rbs = [j[2] for j in jobs]
     assert rbs == sorted(rbs, reverse=True)       # longest sweeps first
+    # column 4: a permutation of the jobs, longest key-owner sweeps (blocks of the doc - rb) first
+    order = s[:, 4].tolist()
+    assert sorted(order) == list(range(len(jobs)))
+    key_len = [(jobs[i][1] + 127) // 128 - jobs[i][2] for i in order]
+    assert key_len == sorted(key_len, reverse=True) and key_len[0] == 5
     # capacity too small: returns the count needed and writes nothing
-    out = torch.full((2, 4), -1, dtype=torch.int32)
+    out = torch.full((2, 5), -1, dtype=torch.int32)
     n = lib.sba_build_schedule(C.cast(cu.data_ptr(), C.POINTER(C.c_int32)), 5,
                                C.cast(out.data_ptr(), C.POINTER(C.c_int32)), 2)
     assert n == len(expect) and bool((out == -1).all())
