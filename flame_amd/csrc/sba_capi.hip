@@ -42,8 +42,6 @@ size_t table_bytes(const SbaParams* p) {
     return (b + 255) & ~(size_t)255;
 }
 
-constexpr size_t kCounterBytes = 256;   // work counter of the dK/dV stream kernel
-
 size_t generic_acc_bytes(const SbaParams* p) {
     size_t b = (size_t)2 * tab_tokens(p) * p->n_heads * sba_generic_padded_dim(p->head_dim) * sizeof(float);
     return (b + 255) & ~(size_t)255;
@@ -90,8 +88,7 @@ KParams make_kparams(const SbaParams* p) {
     if (ws && use_mfma(p)) {
         kp.rtab = (float*)ws;
         kp.gtab = (float*)(ws + table_bytes(p));
-        kp.counter = (int*)(ws + 2 * table_bytes(p));
-        ws += 2 * table_bytes(p) + kCounterBytes;
+        ws += 2 * table_bytes(p);
     }
     if (ws && !use_mfma_bwd(p)) kp.dkv32 = (float*)ws;
     return kp;
@@ -120,7 +117,7 @@ const char* sba_error_string(int code) {
 size_t sba_workspace_bytes(const SbaParams* p) {
     if (!p || p->n_heads <= 0 || p->seq_len <= 0 || p->head_dim <= 0 || p->head_dim > 128) return 0;
     size_t b = 0;
-    if (use_mfma(p)) b += 2 * table_bytes(p) + kCounterBytes;
+    if (use_mfma(p)) b += 2 * table_bytes(p);
     if (!use_mfma_bwd(p)) b += generic_acc_bytes(p);
     return b;
 }

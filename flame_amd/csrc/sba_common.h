@@ -27,7 +27,6 @@ struct KParams {
     TensorArg q, k, v, o, d_o, dq, dk, dv;
     VectorArg rem, d_rem;
     float* rtab;                   // forward carry table  [H][n_kb][total_tokens] (x n_seq for dense)
-    int* counter;                  // work counter of the dK/dV stream kernel (reset by the dQ kernel)
     float* gtab;                   // backward prefix table, same shape
     float* dkv32;                  // generic path: fp32 dk|dv accumulators
     int n_kb;                      // carry-table columns = ceil(seq_len / kKeyBlock)

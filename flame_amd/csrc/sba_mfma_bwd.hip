@@ -22,7 +22,6 @@ namespace sba {
 // ---------------------------------------------------------------- pass 1: dQ + prefix table
 template <int D>
 __global__ __launch_bounds__(kThreads) void mfma_bwd_dq_kernel(KParams p) {
-    if (blockIdx.x == 0 && threadIdx.x == 0 && p.counter) *p.counter = 0;   // for the dK/dV kernel that follows
     constexpr int kTile = 64 * D * 2;
     __shared__ __attribute__((aligned(16))) char lds[4 * kTile];   // K0 V0 K1 V1
 
@@ -130,6 +129,154 @@ mask_step(x, key0 + 32 * h, qi, strict);
                 w.y = __builtin_bit_cast(uint32_t, pb);
                 *(uint2*)(p.dq.ptr + 2 * (ob + 32 * db + 8 * g + 4 * h)) = w;
             }
+    }
+}
+
+// ---------------------------------------------------------------- pass 1, two steps per iteration
+// Same sweep with 8 waves: wave-group 0 (waves 0-3) and wave-group 1 (waves 4-7) take two
+// CONSECUTIVE 64-key steps of the same 128 queries in every iteration (group 1 the right one).
+// All the heavy work of a step (scores, weights, dP, g = a*dP and its prefix sums inside the
+// step) only needs the step's own keys and the forward's carry table; what couples neighbouring
+// steps is one number per query, the sum of g over the step.  The groups swap those totals
+// through LDS at a barrier, the right group adds the left group's total to its prefix, and each
+// group accumulates its own partial dQ, summed once at the end.  The longest dependent chain
+// of a launch (the sweep of the last row-block) is halved, which is what bounds the time when
+// the whole problem is only two waves per SIMD.
+template <int D>
+__global__ __launch_bounds__(2 * kThreads, 2) void mfma_bwd_dq2_kernel(KParams p) {
+    constexpr int kTile = 64 * D * 2;
+    // tile(buf, grp, kv) = lds + ((buf * 2 + grp) * 2 + kv) * kTile
+    __shared__ __attribute__((aligned(16))) char lds[8 * kTile];
+    __shared__ float xch[2][kRowBlock];
+
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int grp = wave >> 2, qs = wave & 3;
+    const int n = lane & 31, h = lane >> 5;
+    LaneOffsets<D> lo;
+    lo.init(lane);
+    const int head = blockIdx.x % p.n_heads;
+    const Job job = decode_job(p, order_job(blockIdx.x / p.n_heads, p.n_jobs, false));
+    const int strict = p.attend_current ? 0 : 1;
+    const int m0 = job.rb * kRowBlock;
+    const int q0w = m0 + 32 * qs;
+    const int qi = q0w + n;
+    const bool row_ok = qi < job.len;
+    const int64_t qbase = (int64_t)job.seq * p.q.sb + (int64_t)head * p.q.sh + (int64_t)job.tok0 * p.q.st;
+    const int64_t kbase = (int64_t)job.seq * p.k.sb + (int64_t)head * p.k.sh + (int64_t)job.tok0 * p.k.st;
+    const int64_t vbase = (int64_t)job.seq * p.v.sb + (int64_t)head * p.v.sh + (int64_t)job.tok0 * p.v.st;
+    const int64_t dobase = (int64_t)job.seq * p.d_o.sb + (int64_t)head * p.d_o.sh + (int64_t)job.tok0 * p.d_o.st;
+
+    bf16x8 qf[D / 16], dof[D / 16];
+    load_row_frags<D>(qf, p.q, qbase, qi, job.len, lane);
+    load_row_frags<D>(dof, p.d_o, dobase, qi, job.len, lane);
+    float dr = 0.f;
+    if (row_ok && p.d_rem.ptr)
+        dr = Elem<uint16_t>::load(p.d_rem.ptr, (int64_t)job.seq * p.d_rem.sb + (int64_t)head * p.d_rem.sh + job.tok0 + qi);
+
+    f32x16 dqacc[D / 32];
+#pragma unroll
+    for (int db = 0; db < D / 32; ++db) dqacc[db] = f32x16{0};
+    float Gc = 0.f;
+
+    const int imax = min(m0 + kRowBlock - 1, job.len - 1);
+    const int kmax = imax - strict;
+    const int n_steps = kmax >= 0 ? kmax / kKeyBlock + 1 : 0;
+    const int n_it = (n_steps + 1) / 2;
+    const int64_t tabtok = tab_token(p, job, qi);
+    char* my_tiles = lds + grp * 2 * kTile;          // + buf * 4 * kTile
+
+    // each group copies its own tiles (256 threads per tile pair)
+    TileCopy<D> kc, vc;
+    if (grp < n_steps) {
+        kc.load(p.k, kbase, grp * kKeyBlock, job.len);
+        vc.load(p.v, vbase, grp * kKeyBlock, job.len);
+        kc.store(my_tiles);
+        vc.store(my_tiles + kTile);
+    }
+    __syncthreads();
+
+    // the forward's carry for this group's NEXT step is loaded while this one is computed
+    const int64_t tstride = p.tab_tokens;
+    const int64_t tix0 = (int64_t)head * p.n_kb * p.tab_tokens + tabtok;
+    float Rnext = (row_ok && grp < n_steps) ? p.rtab[tix0 + grp * tstride] : 1.0f;
+    wait_global_memory();
+    for (int it = 0, buf = 0; it < n_it; ++it, buf ^= 1) {
+        const int step = 2 * it + grp;                   // == n_steps: this group idles in the last iteration
+        const char* ktile = my_tiles + buf * 4 * kTile;
+        const char* vtile = ktile + kTile;
+        const bool more = step + 2 < n_steps;
+        const int key0 = step * kKeyBlock;
+        const bool active = step < n_steps && !(key0 + strict > q0w + 31);
+        const int64_t tix = tix0 + step * tstride;
+        const float R = Rnext;
+        if (more) {
+            if (row_ok) Rnext = p.rtab[tix + 2 * tstride];
+            kc.load(p.k, kbase, (step + 2) * kKeyBlock, job.len);
+            vc.load(p.v, vbase, (step + 2) * kKeyBlock, job.len);
+        }
+        float x[32], beta[32], dp[32];
+        float total = 0.f, start = 0.f;
+        if (active) {
+            score_tiles_o<D>(x, ktile, lo, qf, p.scale2);
+            if (key0 + 63 + strict > q0w) mask_step(x, key0 + 32 * h, qi, strict);
+            float Rc = R;
+            stick_weights<true>(x, beta, Rc, lane);
+            dp_tiles_o<D>(dp, vtile, lo, dof, dr);
+            start = logit_grads_local(x, dp, total, lane);
+        }
+        if (h == 0) xch[grp][32 * qs + n] = total;
+        __syncthreads();
+        const float other = xch[grp ^ 1][32 * qs + n];
+        // group 1 holds the right step of the pair: its prefix also contains group 0's total
+        const float Gmy = grp == 0 ? Gc : Gc + other;
+        Gc = Gc + total + other;
+        if (active) {
+            if (row_ok && h == 0) p.gtab[tix] = Gmy;
+            logit_grads_apply(beta, dp, Gmy + start);
+            bf16x8 zf[4];
+#pragma unroll
+            for (int c = 0; c < 4; ++c) zf[c] = pack8(&dp[8 * c]);
+#pragma unroll
+            for (int db = 0; db < D / 32; ++db)
+#pragma unroll
+                for (int c = 0; c < 4; ++c)
+                    dqacc[db] = mfma(fetch_cols_o<D>(ktile, lo, db, c), zf[c], dqacc[db]);
+        }
+        if (more) {
+            kc.store(my_tiles + (buf ^ 1) * 4 * kTile);
+            vc.store(my_tiles + (buf ^ 1) * 4 * kTile + kTile);
+        }
+        wait_global_memory();                  // nothing in flight across the back edge
+        __syncthreads();
+    }
+
+    // ---- dQ = dQ(group 0) + dQ(group 1): group 1 parks its accumulators in LDS
+    float* park = (float*)lds;                              // [qs][db][r][lane]
+    if (grp == 1) {
+#pragma unroll
+        for (int db = 0; db < D / 32; ++db)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) park[((qs * (D / 32) + db) * 16 + r) * 64 + lane] = dqacc[db][r];
+    }
+    __syncthreads();
+    if (grp == 0 && row_ok) {
+        const int64_t ob = (int64_t)job.seq * p.dq.sb + (int64_t)head * p.dq.sh + (int64_t)(job.tok0 + qi) * p.dq.st;
+#pragma unroll
+        for (int db = 0; db < D / 32; ++db) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) dqacc[db][r] += park[((qs * (D / 32) + db) * 16 + r) * 64 + lane];
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                f32x2 a = {dqacc[db][4 * g] * p.scale, dqacc[db][4 * g + 1] * p.scale};
+                f32x2 b = {dqacc[db][4 * g + 2] * p.scale, dqacc[db][4 * g + 3] * p.scale};
+                bf16x2 pa = __builtin_convertvector(a, bf16x2), pb = __builtin_convertvector(b, bf16x2);
+                uint2 w;
+                w.x = __builtin_bit_cast(uint32_t, pa);
+                w.y = __builtin_bit_cast(uint32_t, pb);
+                *(uint2*)(p.dq.ptr + 2 * (ob + 32 * db + 8 * g + 4 * h)) = w;
+            }
+        }
     }
 }
 
@@ -301,9 +448,9 @@ __global__ __launch_bounds__(kThreads, 2) void mfma_bwd_dkv_kernel(KParams p) {
 }
 
 // ---------------------------------------------------------------- pass 2, head_dim 64
-// dK/dV as ONE resident workgroup per CU that pulls (key block, head) items from a global
-// counter and runs them back to back as a single stream of 128-query steps, with the two
-// halves of a step given to different waves:
+// dK/dV as ONE resident workgroup per CU that runs its share of the (key block, head) items
+// back to back as a single stream of 128-query steps, with the two halves of a step given to
+// different waves:
 //   waves 0..3 ("producers") turn 32 queries x 64 keys each into weights and logit gradients
 //     and leave them, as bf16 [query][key] rows, in one of two LDS buffers;
 //   waves 4..7 ("consumers") reduce the buffer of the previous step into dK and dV with
@@ -704,13 +851,15 @@ int sba_launch_mfma_bwd(const sba::KParams& kp, int phases, hipStream_t s) {
     dim3 grid((unsigned)kp.n_jobs * kp.n_heads);
     const bool p1 = phases != 2, p2 = phases != 1;
     if (kp.head_dim == 64) {
-        if (p1) hipLaunchKernelGGL((mfma_bwd_dq_kernel<64>), grid, dim3(kThreads), 0, s, kp);
+        // small grids last as long as their longest sweep: take the variant that halves it
+        if (p1 && grid.x <= 1024) hipLaunchKernelGGL((mfma_bwd_dq2_kernel<64>), grid, dim3(2 * kThreads), 0, s, kp);
+        else if (p1) hipLaunchKernelGGL((mfma_bwd_dq_kernel<64>), grid, dim3(kThreads), 0, s, kp);
         if (p2) {
-            // one resident workgroup per CU; the items are handed out through kp.counter,
-            // which the dQ kernel of the same backward has reset
+            // one resident workgroup per CU, in whole rounds of the 8 XCDs (surplus workgroups
+            // find no item)
             const unsigned n_items = 2 * grid.x;
             unsigned n_wg = n_items < (unsigned)sba_cu_count() ? n_items : (unsigned)sba_cu_count();
-            n_wg = (n_wg + 7) & ~7u;           // whole XCD rounds (surplus workgroups find no item)
+            n_wg = (n_wg + 7) & ~7u;
             hipLaunchKernelGGL((mfma_bwd_dkv_stream_kernel<64>), dim3(n_wg), dim3(2 * kThreads), 0, s, kp);
         }
     } else {

@@ -326,3 +326,26 @@ def test_small_and_large_grids_take_different_forward_kernels_and_agree():
     assert torch.equal(o2[0], o2[39]) and torch.equal(r2[0], r2[39])
     o_ref, rem_ref = O.sb_attn_oracle(q.cpu(), k.cpu(), v.cpu())
     assert max_abs(o2[39:].float().cpu(), o_ref) <= 2e-2 and max_abs(r2[39:].float().cpu(), rem_ref) <= 2e-2
+
+
+def test_small_and_large_grids_take_different_backward_kernels_and_agree():
+    # <= 1024 workgroups: two-step-per-iteration dQ kernel; above: one step per iteration.
+    sb_attn, _ = _ops()
+    base = [randn((1, 4, 1000, 64), 120 + i, 0.5, torch.bfloat16).cuda() for i in range(3)]
+    do = randn((1, 4, 1000, 64), 130, 1.0, torch.bfloat16).cuda()
+    drem = randn((1, 4, 1000), 131, 1.0, torch.bfloat16).cuda()
+
+    def grads(rep):
+        q, k, v = (x.expand(rep, -1, -1, -1).contiguous().requires_grad_() for x in base)
+        o, rem = sb_attn(q, k, v)
+        torch.autograd.backward([o, rem], [do.expand(rep, -1, -1, -1).contiguous(), drem.expand(rep, -1, -1).contiguous()])
+        return q.grad, k.grad, v.grad
+
+    small, large = grads(1), grads(40)                      # 32 vs 1280 row-owner workgroups
+    for a, b in zip(small, large):
+        assert torch.equal(b[0], b[39])
+        assert rel_l2(b[:1].float(), a.float()) <= 2e-2
+    q, k, v = (x.cpu() for x in base)
+    ref = O.sb_attn_grads_oracle(q, k, v, do.cpu(), drem.cpu())
+    for a, b, r in zip(small, large, ref[-3:]):
+        assert rel_l2(a.float().cpu(), r) <= 5e-2 and rel_l2(b[39:].float().cpu(), r) <= 5e-2
