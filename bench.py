@@ -18,6 +18,12 @@ if ROOT not in sys.path:
 
 BF16_MFMA_PEAK_TFLOPS = 2516.6     # 256 CU x 2.4 GHz x 4096 FLOP/clk/CU (dense bf16)
 
+# HBM bytes per launch (read + write) from the rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of the
+# cfg2 workload summarised in profiles/sba_cfg2_hbm_traffic.txt (counters cannot be read from
+# inside this process); other workloads report null.
+PROFILED_HBM_BYTES = {("cfg2", "fwd"): int(40.4 * 2**20), ("cfg2", "bwd_dq"): int(56.5 * 2**20),
+                      ("cfg2", "bwd_dkv"): int(65.2 * 2**20)}
+
 
 def _lognormal_lengths(total, seed, median=600.0, sigma=1.0, lo=16, hi=4096):
     import torch
@@ -219,7 +225,8 @@ def main():
         "fwd_tflops": round(4.0 * D * pairs / (kern.get("fwd", float("nan")) * 1e-3) / 1e12, 2),
         "roofline": {"bound": "mfma", "kernel": dom, "achieved": round(achieved, 2),
                      "peak": BF16_MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
-                     "frac": round(achieved / BF16_MFMA_PEAK_TFLOPS, 4), "traffic": None},
+                     "frac": round(achieved / BF16_MFMA_PEAK_TFLOPS, 4),
+                     "traffic": PROFILED_HBM_BYTES.get((args.workload, dom))},
     }
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(args.workload)
