@@ -460,13 +460,19 @@ __global__ __launch_bounds__(kThreads, 2) void mfma_bwd_dkv_kernel(KParams p) {
 // vector work, and because the stream never stops at an item boundary nothing of an item's
 // set-up (launch, K/V fetch, first tiles) or tear-down (dK/dV store) is exposed.
 //
-// One iteration s of the stream (barrier B in its middle, A at its end):
-//   producers:  fragments of tile[s&1] -> scores, weights, dP      | B | dz -> Z[s&1]            | A
+// One iteration s of the stream (workgroup barrier A at its end; B is a barrier of the four
+// consumer waves only, a running count in LDS, so that the producers - the critical path -
+// never wait in the middle of a step):
+//   producers:  fragments of tile[s&1] -> scores, weights, dP, dz -> Z[s&1]                    | A
 //   consumers:  store a staged dK/dV; request step s+1;
 //               reduce Z/tile[(s-1)&1]                            | B | stage a finished dK/dV
 //                                                                       into Z[(s-1)&1];
 //                                                                       deposit step s+1 -> [(s+1)&1] | A
-// B separates the reduction's last read of buffer (s-1)&1 from the stores that reuse it.
+// B separates the reduction's last read of buffer (s-1)&1 from the stores that reuse it.  Two
+// rarer hand-overs: a staged dK/dV occupies the Z buffer that the producers write in the next
+// iteration, so that iteration has one more workgroup barrier (X) after the consumers' store;
+// and the K tile is refilled only after a second LDS count says that every producer holds
+// the current item's K fragments.
 // An item's accumulators are complete after the reduction that follows its last step; they are
 // staged after that iteration's B and written to global memory before the next iteration's B.
 struct KeyItem {
@@ -496,7 +502,8 @@ __global__ __launch_bounds__(2 * kThreads, 2) void mfma_bwd_dkv_stream_kernel(KP
     constexpr int kBuf = 2 * kZTile + 2 * kQTile;
     constexpr int kCarry = kRowBlock * 16;     // {R, G, d_rem, -} per query
     __shared__ __attribute__((aligned(1024))) char lds[3 * kTile + 2 * kCarry + 2 * kBuf];
-    __shared__ int slots[4];                   // ring of item indices handed out by the fetcher
+    __shared__ int consumers_done;             // consumer waves that have finished a reduction, running total
+    __shared__ int producers_took_k;           // producer waves that hold an item's K fragments, running total
     char* vtiles = lds;                        // V of item j in vtiles + (j&1)*kTile
     char* ktile = vtiles + 2 * kTile;          // read once per item, into the producers' registers
     char* carry = ktile + kTile;
@@ -509,7 +516,6 @@ __global__ __launch_bounds__(2 * kThreads, 2) void mfma_bwd_dkv_stream_kernel(KP
     const int n = lane & 31, h = lane >> 5;
     const int strict = p.attend_current ? 0 : 1;
     const int n_items = 2 * p.n_jobs * p.n_heads;
-    const bool fetcher = threadIdx.x == kThreads;
 
     // Items are taken in list order (longest sweeps first).  A job's second key block can lie
     // beyond the end of its sequence: such an item runs like any other, its one step finds
@@ -521,23 +527,20 @@ __global__ __launch_bounds__(2 * kThreads, 2) void mfma_bwd_dkv_stream_kernel(KP
     // which evens out the sweep lengths (the list is sorted by them).
     const int W = G >> 3, w = g >> 3, c8 = g & 7;
     auto static_item = [&](int r) { const int i = 8 * (r * W + ((r & 1) ? W - 1 - w : w)) + c8; return i < n_items ? i : -1; };
-    if (fetcher) {
-        slots[0] = static_item(0);
-        slots[1] = static_item(1);
-    }
-    __syncthreads();
-    int cur_idx = __builtin_amdgcn_readfirstlane(slots[0]);
-    int nxt_idx = __builtin_amdgcn_readfirstlane(slots[1]);
+    int cur_idx = static_item(0);
+    int nxt_idx = static_item(1);
     KeyItem cur = decode_item(p, cur_idx);
     if (!cur.valid) return;                    // uniform over the workgroup
     KeyItem nxt = decode_item(p, nxt_idx);
-    int ring = 2;                              // slot that is filled while `cur` runs
+    int ring = 2;                              // round of the item after `nxt`
+    if (threadIdx.x == 0) { consumers_done = 0; producers_took_k = 0; }
 
     if (producer) {
         LaneOffsets<D> lo;
         lo.init(lane);
         __syncthreads();                       // first item's tiles and carries visible
         int s = 0;
+        bool staged_prev = false;              // the consumers staged a dK/dV in the previous iteration
         for (int item = 0;; ++item) {
             const char* vtile = vtiles + (item & 1) * kTile;
             // the key block of an item never changes: its score operands stay in registers
@@ -546,9 +549,16 @@ __global__ __launch_bounds__(2 * kThreads, 2) void mfma_bwd_dkv_stream_kernel(KP
             for (int t = 0; t < 2; ++t)
 #pragma unroll
                 for (int ks = 0; ks < D / 16; ++ks) kfr[t][ks] = fetch_rows_o<D>(ktile, lo, t, ks);
+            // tell the consumers that the K tile may be refilled
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+            if (lane == 0) __hip_atomic_fetch_add(&producers_took_k, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
             const int key0 = cur.key0;
             const int len = cur.job.len;
             for (int it = 0; it < cur.n_steps; ++it, ++s) {
+                // A dK/dV staged in the previous iteration sits in the Z buffer this iteration
+                // writes: wait (barrier X) until the consumers have stored it.
+                const bool x_now = staged_prev;
+                staged_prev = it == 0 && item > 0;
                 char* zp = bufs + (s & 1) * kBuf;
                 char* zd = zp + kZTile;
                 const char* qtile = zd + kZTile;
@@ -583,7 +593,7 @@ __global__ __launch_bounds__(2 * kThreads, 2) void mfma_bwd_dkv_stream_kernel(KP
                     for (int ks = 0; ks < D / 16; ++ks) dof[ks] = fetch_rows_o<D>(dotile, lo, w4, ks);
                     dp_tiles_o<D>(dp, vtile, lo, dof, bf16_to_f32((uint16_t)__float_as_uint(cv.z)));
                 }
-                __syncthreads();               // B
+                if (x_now) __syncthreads();    // X
                 if (!skip) {
                     logit_grads<true>(x, beta, dp, Gc, lane);
                 } else {
@@ -599,11 +609,10 @@ __global__ __launch_bounds__(2 * kThreads, 2) void mfma_bwd_dkv_stream_kernel(KP
             }
             if (!nxt.valid) break;
             cur = nxt;
-            nxt = decode_item(p, __builtin_amdgcn_readfirstlane(slots[ring & 3]));
+            nxt = decode_item(p, static_item(ring));
             ++ring;
         }
-        __syncthreads();                       // B of the draining iteration
-        __syncthreads();                       // A
+        __syncthreads();                       // A of the draining iteration
     } else {
         LaneOffsets<D> lo;
         lo.init(lane);
@@ -768,11 +777,24 @@ __global__ __launch_bounds__(2 * kThreads, 2) void mfma_bwd_dkv_stream_kernel(KP
         bool finish_after_reduce = false;      // the step about to be reduced is its item's last
         bool store_pending = false;            // a staged dK/dV waits in Z[s&1] to be stored
         int fin_stage = cur_idx, fin_store = cur_idx;
+        // B, a barrier of the four consumer waves only (the producers have no part in what it
+        // protects and must not be held up by it): a running count in LDS, bumped by each wave
+        // after its reduction, and a short spin.  All four waves are resident, so it terminates.
+        int sync_target = 0;
+        auto consumer_sync = [&]() {
+            sync_target += 4;
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+            if (lane == 0) __hip_atomic_fetch_add(&consumers_done, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+            while (__hip_atomic_load(&consumers_done, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) < sync_target)
+                __builtin_amdgcn_s_sleep(1);
+            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+        };
         // One iteration of the stream; `rq`, `rq_row0` say what the stream's next step needs.
         auto iteration = [&](const ItemPtrs& rq, int rq_row0, bool last, bool keys_now, int item) {
             if (store_pending) {               // staged in the previous iteration
                 store_staged(fin_store, bufs + (s & 1) * kBuf);
                 store_pending = false;
+                __syncthreads();               // X: the producers may overwrite the staging
             }
             request_carry(rq, rq_row0);
             if (s > 0) {
@@ -781,8 +803,14 @@ __global__ __launch_bounds__(2 * kThreads, 2) void mfma_bwd_dkv_stream_kernel(KP
 #pragma unroll
                 for (int part = 0; part < 4; ++part) request_tile(rq, rq_row0, part);
             }
-            __syncthreads();                   // B: every consumer has finished with buffer (s-1)&1
-            if (keys_now) request_keys(decode_item(p, nxt_idx), vtiles + ((item + 1) & 1) * kTile);
+            consumer_sync();                   // B: every consumer has finished with buffer (s-1)&1
+            if (keys_now) {
+                // the K tile is free once every producer holds this item's fragments
+                while (__hip_atomic_load(&producers_took_k, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) < 4 * (item + 1))
+                    __builtin_amdgcn_s_sleep(1);
+                __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+                request_keys(decode_item(p, nxt_idx), vtiles + ((item + 1) & 1) * kTile);
+            }
             if (finish_after_reduce) {
                 stage(bufs + ((s - 1) & 1) * kBuf);
                 fin_store = fin_stage;
@@ -796,8 +824,6 @@ __global__ __launch_bounds__(2 * kThreads, 2) void mfma_bwd_dkv_stream_kernel(KP
             ++s;
         };
         for (int item = 0;; ++item) {
-            // index of the item after next
-            if (fetcher) slots[ring & 3] = static_item(ring);
             // The next item's K and V are requested after B of the second-to-last step: K's tile
             // is free once the producers have taken their fragments (before the item's first B),
             // V goes to the tile of the other parity.
@@ -813,7 +839,7 @@ __global__ __launch_bounds__(2 * kThreads, 2) void mfma_bwd_dkv_stream_kernel(KP
             if (!has_next) break;
             cur_idx = nxt_idx;
             cur = nxt;
-            nxt_idx = __builtin_amdgcn_readfirstlane(slots[ring & 3]);
+            nxt_idx = static_item(ring);
             nxt = decode_item(p, nxt_idx);
             ++ring;
             cp = np;
@@ -822,7 +848,7 @@ __global__ __launch_bounds__(2 * kThreads, 2) void mfma_bwd_dkv_stream_kernel(KP
         // draining iteration: the last step of the last item
         if (store_pending) store_staged(fin_store, bufs + (s & 1) * kBuf);
         reduce(s - 1, [&](int) {});
-        __syncthreads();                       // B
+        consumer_sync();                       // B
         stage(bufs + ((s - 1) & 1) * kBuf);
         __syncthreads();                       // A (consumers only need each other's staging)
         store_staged(fin_stage, bufs + ((s - 1) & 1) * kBuf);
