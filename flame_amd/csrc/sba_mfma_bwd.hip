@@ -619,15 +619,18 @@ __global__ __launch_bounds__(2 * kThreads, 2) void mfma_bwd_dkv_stream_kernel(KP
         LaneOffsets<64> lz;                    // the weight tiles have 64-key rows whatever D is
         lz.init(lane);
         const int ct = threadIdx.x & (kThreads - 1);
-        const int kh = w4 & 1;                 // which 32 keys this wave reduces
-        const int dbw = w4 >> 1;               // and which d-blocks: dbw + 2*i
-        const int za0 = pick_nat<64>(lz, 0, kh), za1 = pick_nat<64>(lz, 1, kh);
-        int qb0o[D / 64], qb1o[D / 64];
+        // Wave w4 reduces ONE of the two outputs (even: dK from dz and Q, odd: dV from a and dO),
+        // all 64 keys of it and one 32-wide d-block: the two key halves share the Q / dO operand,
+        // three operand fetches per two MFMAs instead of four.
+        static_assert(D == 64, "the consumers' tiling assumes two 32-wide d-blocks");
+        const bool is_dv = w4 & 1;
+        const int dbw = w4 >> 1;
+        int za[2][2];
 #pragma unroll
-        for (int i = 0; i < D / 64; ++i) { qb0o[i] = pick_nat<D>(lo, 0, dbw + 2 * i); qb1o[i] = pick_nat<D>(lo, 1, dbw + 2 * i); }
-        f32x16 dkacc[D / 64], dvacc[D / 64];
-#pragma unroll
-        for (int i = 0; i < D / 64; ++i) { dkacc[i] = f32x16{0}; dvacc[i] = f32x16{0}; }
+        for (int kh = 0; kh < 2; ++kh) { za[kh][0] = pick_nat<64>(lz, 0, kh); za[kh][1] = pick_nat<64>(lz, 1, kh); }
+        const int qb0o = pick_nat<D>(lo, 0, dbw), qb1o = pick_nat<D>(lo, 1, dbw);
+        f32x16 acc[2];                         // key halves
+        acc[0] = f32x16{0}; acc[1] = f32x16{0};
 
         // Staging registers of one step: thread ct holds chunk ct%8 of rows ct/8 + 32*part of the
         // Q and dO tiles, and (ct < 128) the carries of query ct.  Every request is
@@ -723,44 +726,34 @@ __global__ __launch_bounds__(2 * kThreads, 2) void mfma_bwd_dkv_stream_kernel(KP
         };
         auto stage = [&](char* staging) {
 #pragma unroll
-            for (int i = 0; i < D / 64; ++i) {
-                stage_acc_tile<D>(staging, 32 * kh, 32 * (dbw + 2 * i), dkacc[i], p.scale, lane);
-                stage_acc_tile<D>(staging + kTile, 32 * kh, 32 * (dbw + 2 * i), dvacc[i], 1.0f, lane);
-                dkacc[i] = f32x16{0};
-                dvacc[i] = f32x16{0};
+            for (int kh = 0; kh < 2; ++kh) {
+                stage_acc_tile<D>(staging + (is_dv ? kTile : 0), 32 * kh, 32 * dbw, acc[kh], is_dv ? 1.0f : p.scale, lane);
+                acc[kh] = f32x16{0};
             }
         };
-        // dK[key][d] += sum_q dz[q][key] Q[q][d];  dV[key][d] += sum_q a[q][key] dO[q][d].
+        // dK[key][d] += sum_q dz[q][key] Q[q][d]  or  dV[key][d] += sum_q a[q][key] dO[q][d].
         // The operands of four 16-query groups are fetched as one batch, so that the MFMAs wait
         // for LDS once per batch rather than once each; `between(b)` (the tile requests) goes
         // behind the fetches of batch b.
         auto reduce = [&](int s_done, auto&& between) {
-            const char* zp = bufs + (s_done & 1) * kBuf;
-            const char* zd = zp + kZTile;
-            const char* qtile = zd + kZTile;
-            const char* dotile = qtile + kQTile;
+            const char* zt = bufs + (s_done & 1) * kBuf + (is_dv ? 0 : kZTile);            // a or dz
+            const char* xt = bufs + (s_done & 1) * kBuf + 2 * kZTile + (is_dv ? kQTile : 0); // dO or Q
 #pragma unroll
             for (int b = 0; b < 2; ++b) {
-                bf16x8 az[4], ap[4], bq[4][D / 64], bd[4][D / 64];
+                bf16x8 aw[4][2], bx[4];
 #pragma unroll
                 for (int j = 0; j < 4; ++j) {
                     const int c2 = 4 * b + j;
-                    az[j] = fetch_nat_2<64>(zd, za0, za1, 16 * c2);
-                    ap[j] = fetch_nat_2<64>(zp, za0, za1, 16 * c2);
-#pragma unroll
-                    for (int i = 0; i < D / 64; ++i) {
-                        bq[j][i] = fetch_nat_2<D>(qtile, qb0o[i], qb1o[i], 16 * c2);
-                        bd[j][i] = fetch_nat_2<D>(dotile, qb0o[i], qb1o[i], 16 * c2);
-                    }
+                    aw[j][0] = fetch_nat_2<64>(zt, za[0][0], za[0][1], 16 * c2);
+                    aw[j][1] = fetch_nat_2<64>(zt, za[1][0], za[1][1], 16 * c2);
+                    bx[j] = fetch_nat_2<D>(xt, qb0o, qb1o, 16 * c2);
                 }
                 between(b);
 #pragma unroll
-                for (int j = 0; j < 4; ++j)
-#pragma unroll
-                    for (int i = 0; i < D / 64; ++i) {
-                        dkacc[i] = mfma(az[j], bq[j][i], dkacc[i]);
-                        dvacc[i] = mfma(ap[j], bd[j][i], dvacc[i]);
-                    }
+                for (int j = 0; j < 4; ++j) {
+                    acc[0] = mfma(aw[j][0], bx[j], acc[0]);
+                    acc[1] = mfma(aw[j][1], bx[j], acc[1]);
+                }
             }
         };
 
