@@ -321,10 +321,12 @@ __device__ inline void stick_weights(float (&x)[32], float (&beta)[kNeedBeta ? 3
     for (int idx = 31; idx >= 0; --idx) {
         float e = __builtin_amdgcn_exp2f(x[idx]);
         float u = __builtin_amdgcn_rcpf(1.0f + e);
-        float b = 1.0f - u;
-        x[idx] = b * L;
-        L *= u;
-        if (kNeedBeta) beta[idx] = b;
+        // beta * L = L - u * L, and u * L is the next value of the chain anyway: one instruction
+        // less than forming beta first (the rounding error, one ulp of L, is the same)
+        const float Ln = L * u;
+        x[idx] = L - Ln;
+        L = Ln;
+        if (kNeedBeta) beta[idx] = 1.0f - u;
     }
     const float other = __shfl_xor(L, 32);
     // upper half-wave holds the right 32 keys: its chain starts from R itself
@@ -348,10 +350,12 @@ __device__ inline float stick_weights_local(float (&x)[32], float (&beta)[kNeedB
     for (int idx = 31; idx >= 0; --idx) {
         float e = __builtin_amdgcn_exp2f(x[idx]);
         float u = __builtin_amdgcn_rcpf(1.0f + e);
-        float b = 1.0f - u;
-        x[idx] = b * L;
-        L *= u;
-        if (kNeedBeta) beta[idx] = b;
+        // beta * L = L - u * L, and u * L is the next value of the chain anyway: one instruction
+        // less than forming beta first (the rounding error, one ulp of L, is the same)
+        const float Ln = L * u;
+        x[idx] = L - Ln;
+        L = Ln;
+        if (kNeedBeta) beta[idx] = 1.0f - u;
     }
     const float other = __shfl_xor(L, 32);
     total = L * other;
