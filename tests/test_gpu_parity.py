@@ -147,6 +147,15 @@ def test_varlen_lognormal_pack_8192():
     _check_varlen(4, 64, lens, torch.bfloat16, seed=13)
 
 
+def test_varlen_many_short_documents_stream_many_items_per_workgroup():
+    # 2 x jobs x H = about 2500 (key block, head) items for the 256 resident dK/dV workgroups: ten
+    # rounds each, most items a single step long (a finished dK/dV is staged and stored every
+    # iteration), many second key blocks lying beyond the end of their document
+    g = torch.Generator().manual_seed(21)
+    lens = [int(x) for x in torch.randint(1, 201, (60,), generator=g)] + [64, 65, 128, 129, 256]
+    _check_varlen(16, 64, lens, torch.bfloat16, seed=22)
+
+
 def test_varlen_equals_dense_per_document():
     sb_attn, sb_attn_varlen = _ops()
     H, D, lens = 3, 64, [130, 64, 257]
