@@ -543,12 +543,15 @@ __global__ __launch_bounds__(2 * kThreads, 2) void mfma_bwd_dkv_stream_kernel(KP
         bool staged_prev = false;              // the consumers staged a dK/dV in the previous iteration
         for (int item = 0;; ++item) {
             const char* vtile = vtiles + (item & 1) * kTile;
-            // the key block of an item never changes: its score operands stay in registers
-            bf16x8 kfr[2][D / 16];
+            // the key block of an item never changes: its score and dP operands stay in registers
+            bf16x8 kfr[2][D / 16], vfr[2][D / 16];
 #pragma unroll
             for (int t = 0; t < 2; ++t)
 #pragma unroll
-                for (int ks = 0; ks < D / 16; ++ks) kfr[t][ks] = fetch_rows_o<D>(ktile, lo, t, ks);
+                for (int ks = 0; ks < D / 16; ++ks) {
+                    kfr[t][ks] = fetch_rows_o<D>(ktile, lo, t, ks);
+                    vfr[t][ks] = fetch_rows_o<D>(vtile, lo, t, ks);
+                }
             // tell the consumers that the K tile may be refilled
             __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
             if (lane == 0) __hip_atomic_fetch_add(&producers_took_k, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
@@ -574,9 +577,12 @@ __global__ __launch_bounds__(2 * kThreads, 2) void mfma_bwd_dkv_stream_kernel(KP
                     // makes their weights and gradients exactly zero
                     float R = qi < len ? cv.x : 0.f;
                     Gc = qi < len ? cv.y : 0.f;
-                    bf16x8 qf[D / 16];
+                    bf16x8 qf[D / 16], dof[D / 16];
 #pragma unroll
-                    for (int ks = 0; ks < D / 16; ++ks) qf[ks] = fetch_rows_o<D>(qtile, lo, w4, ks);
+                    for (int ks = 0; ks < D / 16; ++ks) {
+                        qf[ks] = fetch_rows_o<D>(qtile, lo, w4, ks);
+                        dof[ks] = fetch_rows_o<D>(dotile, lo, w4, ks);
+                    }
                     f32x16 raw[2];
 #pragma unroll
                     for (int t = 0; t < 2; ++t) {
@@ -587,11 +593,29 @@ __global__ __launch_bounds__(2 * kThreads, 2) void mfma_bwd_dkv_stream_kernel(KP
                     }
                     scale_scores(x, raw, p.scale2);
                     if (key0 + 63 + strict > q0w) mask_step(x, key0 + 32 * h, qi, strict);
-                    stick_weights<true>(x, beta, R, lane);
-                    bf16x8 dof[D / 16];
+                    // dP = dO V^T - d_rem does not depend on the weights: its eight MFMAs are spread
+                    // under the weights' vector arithmetic.  (Only instructions of ONE wave overlap
+                    // this way: a SIMD does not issue another wave's vector instructions while a
+                    // wave's back-to-back MFMAs wait for the matrix pipe.)
+                    const float dr = bf16_to_f32((uint16_t)__float_as_uint(cv.z));
+                    f32x16 dacc[2];
 #pragma unroll
-                    for (int ks = 0; ks < D / 16; ++ks) dof[ks] = fetch_rows_o<D>(dotile, lo, w4, ks);
-                    dp_tiles_o<D>(dp, vtile, lo, dof, bf16_to_f32((uint16_t)__float_as_uint(cv.z)));
+                    for (int t = 0; t < 2; ++t) {
+#pragma unroll
+                        for (int r = 0; r < 16; ++r) dacc[t][r] = -dr;
+#pragma unroll
+                        for (int ks = 0; ks < D / 16; ++ks) dacc[t] = mfma(vfr[t][ks], dof[ks], dacc[t]);
+                    }
+                    stick_weights<true>(x, beta, R, lane);
+#pragma unroll
+                    for (int i = 0; i < 2 * (D / 16); ++i) {
+                        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);     // one MFMA
+                        __builtin_amdgcn_sched_group_barrier(0x002, 36, 0);    // 36 vector instructions
+                    }
+#pragma unroll
+                    for (int t = 0; t < 2; ++t)
+#pragma unroll
+                        for (int r = 0; r < 16; ++r) dp[16 * t + r] = dacc[t][r];
                 }
                 if (x_now) __syncthreads();    // X
                 if (!skip) {
