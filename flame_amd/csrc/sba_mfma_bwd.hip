@@ -95,8 +95,21 @@ __global__ __launch_bounds__(kThreads) void mfma_bwd_dq_kernel(KParams p) {
             if (key0 + 63 + strict > q0w) {
 mask_step(x, key0 + 32 * h, qi, strict);
             }
-            stick_weights<true>(x, beta, R, lane);
-            dp_tiles_o<D>(dp, vtile, lo, dof, dr);
+            if (D == 128) {
+                // dP does not depend on the weights: its 16 MFMAs are spread under their vector
+                // arithmetic (measured: a gain at head_dim 128, none at 64)
+                dp_tiles_o<D>(dp, vtile, lo, dof, dr);
+                stick_weights<true>(x, beta, R, lane);
+#pragma unroll
+                for (int i = 0; i < 2 * (D / 16); ++i) {
+                    __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);     // one LDS read (the MFMA's A operand)
+                    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);     // one MFMA
+                    __builtin_amdgcn_sched_group_barrier(0x002, 8, 0);     // eight vector instructions
+                }
+            } else {
+                stick_weights<true>(x, beta, R, lane);
+                dp_tiles_o<D>(dp, vtile, lo, dof, dr);
+            }
             logit_grads<false>(x, beta, dp, Gc, lane);
             bf16x8 zf[4];
 #pragma unroll
