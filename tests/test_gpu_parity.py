@@ -358,3 +358,75 @@ def test_small_and_large_grids_take_different_backward_kernels_and_agree():
     ref = O.sb_attn_grads_oracle(q, k, v, do.cpu(), drem.cpu())
     for a, b, r in zip(small, large, ref[-3:]):
         assert rel_l2(a.float().cpu(), r) <= 5e-2 and rel_l2(b[39:].float().cpu(), r) <= 5e-2
+
+
+def _full_size_properties(fwd_bwd, v_shape_like, check_docs=None):
+    """Size-independent properties of a forward+backward at a full BASELINE size (no O(T^2)
+    oracle needed): the backward is linear in the upstream gradients and bit-reproducible,
+    and every result is finite."""
+    do1, do2, dr1, dr2 = v_shape_like
+    g1 = fwd_bwd(do1, dr1)
+    g1b = fwd_bwd(do1, dr1)
+    assert all(torch.equal(a, b) for a, b in zip(g1, g1b))          # no atomics: same bits
+    g2 = fwd_bwd(do2, dr2)
+    g12 = fwd_bwd((do1.float() + do2.float()).to(do1.dtype), (dr1.float() + dr2.float()).to(dr1.dtype))
+    for a, b, c in zip(g1, g2, g12):
+        assert torch.isfinite(c).all()
+        # bf16 rounding of the summed upstream gradient and of each result: a few 2^-8 relative
+        assert rel_l2(c.float(), a.float() + b.float()) <= 2e-2
+
+
+def test_config3_size_packed_invariants():
+    # full size of BASELINE config 3: 65536 packed tokens, H=16, d=64, bf16, log-normal documents
+    _, sb_attn_varlen = _ops()
+    H, N, D = 16, 65536, 64
+    lens = lognormal_lengths(N, seed=0)
+    cu = cu_from_lengths(lens).cuda()
+    q, k = (randn((H, N, D), 140 + i, 0.5, torch.bfloat16).cuda() for i in range(2))
+    ones = torch.ones(H, N, D, dtype=torch.bfloat16, device="cuda")
+    o, rem = sb_attn_varlen(q, k, ones, cu, max(lens))
+    assert (o.float() + rem.float()[..., None] - 1).abs().max() <= 2e-2          # row mass
+    starts = cu[:-1].long()
+    assert rem[:, starts].float().min() == 1 and o[:, starts].abs().max() == 0   # first token of every document
+    # block-diagonal: one document cut out and run alone gives the same rows
+    d = max(range(len(lens)), key=lambda i: lens[i])
+    a, b = int(cu[d]), int(cu[d + 1])
+    o_d, rem_d = sb_attn_varlen(q[:, a:b].contiguous(), k[:, a:b].contiguous(), ones[:, a:b].contiguous(),
+                                torch.tensor([0, b - a], dtype=torch.int32, device="cuda"), b - a)
+    assert torch.equal(o_d, o[:, a:b]) and torch.equal(rem_d, rem[:, a:b])
+    v = randn((H, N, D), 142, 0.5, torch.bfloat16).cuda()
+    ups = [randn((H, N, D), 143 + i, 1.0, torch.bfloat16).cuda() for i in range(2)] + \
+          [randn((H, N), 145 + i, 1.0, torch.bfloat16).cuda() for i in range(2)]
+
+    def fwd_bwd(do, drem):
+        qq, kk, vv = (x.clone().requires_grad_(True) for x in (q, k, v))
+        oo, rr = sb_attn_varlen(qq, kk, vv, cu, max(lens))
+        torch.autograd.backward([oo, rr], [do, drem])
+        return qq.grad, kk.grad, vv.grad
+
+    _full_size_properties(fwd_bwd, ups)
+
+
+def test_config4_size_invariants():
+    # full size of BASELINE config 4: B=1, H=16, T=16384, d=128, bf16
+    sb_attn, _ = _ops()
+    B, H, T, D = 1, 16, 16384, 128
+    q, k = (randn((B, H, T, D), 150 + i, 0.5, torch.bfloat16).cuda() for i in range(2))
+    ones = torch.ones(B, H, T, D, dtype=torch.bfloat16, device="cuda")
+    o, rem = sb_attn(q, k, ones)
+    assert (o.float() + rem.float()[..., None] - 1).abs().max() <= 2e-2
+    assert rem[:, :, 0].float().min() == 1 and o[:, :, 0].abs().max() == 0
+    # causality: the first 1000 rows do not depend on what follows them
+    o_p, rem_p = sb_attn(q[:, :, :1000].contiguous(), k[:, :, :1000].contiguous(), ones[:, :, :1000].contiguous())
+    assert max_abs(o_p.float(), o[:, :, :1000].float()) <= 1e-2 and max_abs(rem_p.float(), rem[:, :, :1000].float()) <= 1e-2
+    v = randn((B, H, T, D), 152, 1.0, torch.bfloat16).cuda()
+    ups = [randn((B, H, T, D), 153 + i, 1.0, torch.bfloat16).cuda() for i in range(2)] + \
+          [randn((B, H, T), 155 + i, 1.0, torch.bfloat16).cuda() for i in range(2)]
+
+    def fwd_bwd(do, drem):
+        qq, kk, vv = (x.clone().requires_grad_(True) for x in (q, k, v))
+        oo, rr = sb_attn(qq, kk, vv)
+        torch.autograd.backward([oo, rr], [do, drem])
+        return qq.grad, kk.grad, vv.grad
+
+    _full_size_properties(fwd_bwd, ups)
