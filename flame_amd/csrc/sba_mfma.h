@@ -206,9 +206,14 @@ template <int D>
 __device__ inline void stage_acc_tile(char* staging, int row0, int col0, const f32x16& acc, float scale, int lane) {
     const int n = lane & 31, h = lane >> 5;
 #pragma unroll
-    for (int r = 0; r < 16; ++r) {
+    for (int r = 0; r < 16; r += 2) {
+        // registers r, r+1 are two consecutive rows of the same column: one packed conversion
+        // (round to nearest even in hardware), two 2-byte stores
         const int row = row0 + 8 * (r >> 2) + 4 * h + (r & 3);
-        *(uint16_t*)(staging + row * (D * 2) + (col0 + n) * 2) = f32_to_bf16(acc[r] * scale);
+        const f32x2 v = {acc[r] * scale, acc[r + 1] * scale};
+        const uint32_t w = __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2));
+        *(uint16_t*)(staging + row * (D * 2) + (col0 + n) * 2) = (uint16_t)w;
+        *(uint16_t*)(staging + (row + 1) * (D * 2) + (col0 + n) * 2) = (uint16_t)(w >> 16);
     }
 }
 // 64 staged rows -> rows row0.. of a [rows, D] tensor; `tid` of `n_threads` threads take part.
