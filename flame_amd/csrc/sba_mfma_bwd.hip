@@ -669,15 +669,18 @@ __global__ __launch_bounds__(2 * kThreads, 2) void mfma_bwd_dkv_stream_kernel(KP
         f32x16 acc[2];                         // key halves
         acc[0] = f32x16{0}; acc[1] = f32x16{0};
 
-        // Staging registers of one step: thread ct holds chunk ct%8 of rows ct/8 + 32*part of the
-        // Q and dO tiles, and (ct < 128) the carries of query ct.  Every request is
-        // unconditional, with rows clamped to the sequence, and every iteration consumes what
-        // it requested: no register is "perhaps still being loaded" on some path, so the
-        // compiler's wait-count bookkeeping stays exact.
-        u32x4 tq[4], td[4];
+        // Staging registers of one step.  A consumer wave stages exactly the part of the step's
+        // tiles that its own reduction reads - the 32-wide d-block `dbw` of Q (dK waves) or of dO
+        // (dV waves), all 128 rows: lane l holds the 16-byte chunk l%4 of rows l/4 + 16*part - so
+        // refilling a tile buffer needs no barrier among the consumers (the producers, who read
+        // whole rows, are kept apart from it by A).  Threads ct < 128 also stage the carries of
+        // query ct.  Every request is unconditional, with rows clamped to the sequence, and every
+        // iteration consumes what it requested: no register is "perhaps still being loaded" on
+        // some path, so the compiler's wait-count bookkeeping stays exact.
+        u32x4 tx[8];
         float cR, cG;
         uint32_t cdr = 0;                      // bf16 bits
-        const int crow = ct >> 3, cch = ct & 7;
+        const int crow = lane >> 2, cch = 4 * dbw + (lane & 3);
         // The tile requests of a step are issued two at a time between the MFMAs of the
         // reduction: all CUs stream their tiles from L2 in the same phase of a step, the
         // memory pipe then accepts about one 1 KB wave load per 80 cycles, and a burst of
@@ -689,7 +692,7 @@ __global__ __launch_bounds__(2 * kThreads, 2) void mfma_bwd_dkv_stream_kernel(KP
         // (a wave issues one instruction every four or five cycles, scalar ones included, and
         // the consumers' share of a step is short).
         struct ItemPtrs {
-            const char *q, *d_o;               // row 0 of the sequence, this head, this thread's chunk
+            const char* x;                     // Q or dO: row 0 of the sequence, this head, this thread's chunk
             const float *rt, *gt;              // carries of this (head, key block), query 0
             const uint16_t* dr;                // d_rem of the sequence, query 0
             int row0, len;                     // first query of the item's sweep; sequence length
@@ -697,22 +700,24 @@ __global__ __launch_bounds__(2 * kThreads, 2) void mfma_bwd_dkv_stream_kernel(KP
         const bool has_dr = p.d_rem.ptr != nullptr;
         auto item_ptrs = [&](const KeyItem& t) {
             ItemPtrs r;
-            r.q = p.q.ptr + 2 * ((int64_t)t.job.seq * p.q.sb + (int64_t)t.head * p.q.sh + (int64_t)t.job.tok0 * p.q.st) + cch * 16;
-            r.d_o = p.d_o.ptr + 2 * ((int64_t)t.job.seq * p.d_o.sb + (int64_t)t.head * p.d_o.sh + (int64_t)t.job.tok0 * p.d_o.st) + cch * 16;
+            const TensorArg& xt = is_dv ? p.d_o : p.q;
+            r.x = xt.ptr + 2 * ((int64_t)t.job.seq * xt.sb + (int64_t)t.head * xt.sh + (int64_t)t.job.tok0 * xt.st) + cch * 16;
             const int64_t tk = ((int64_t)t.head * p.n_kb + t.kb) * p.tab_tokens + tab_token(p, t.job, 0);
             r.rt = p.rtab + tk;
             r.gt = p.gtab + tk;
             r.dr = (const uint16_t*)p.d_rem.ptr + ((int64_t)t.job.seq * p.d_rem.sb + (int64_t)t.head * p.d_rem.sh + t.job.tok0);
             r.row0 = t.job.rb * kRowBlock;
             r.len = t.job.len;
-            asm volatile("" : "+v"(r.q), "+v"(r.d_o), "+v"(r.rt), "+v"(r.gt), "+v"(r.dr));
+            asm volatile("" : "+v"(r.x), "+v"(r.rt), "+v"(r.gt), "+v"(r.dr));
             return r;
         };
-        const uint32_t q_st2 = 2u * (uint32_t)p.q.st, do_st2 = 2u * (uint32_t)p.d_o.st;
-        auto request_tile = [&](const ItemPtrs& t, int row0, int part) {
-            const uint32_t row = (uint32_t)min(row0 + crow + 32 * part, t.len - 1);
-            tq[part] = *(const u32x4*)(t.q + (size_t)row * q_st2);
-            td[part] = *(const u32x4*)(t.d_o + (size_t)row * do_st2);
+        const uint32_t x_st2 = 2u * (uint32_t)(is_dv ? p.d_o.st : p.q.st);
+        auto request_tile = [&](const ItemPtrs& t, int row0, int part) {       // part 0..3: two loads each
+#pragma unroll
+            for (int i = 2 * part; i < 2 * part + 2; ++i) {
+                const uint32_t row = (uint32_t)min(row0 + crow + 16 * i, t.len - 1);
+                tx[i] = *(const u32x4*)(t.x + (size_t)row * x_st2);
+            }
         };
         auto request_carry = [&](const ItemPtrs& t, int row0) {
             const int qi = min(row0 + (ct & (kRowBlock - 1)), t.len - 1);
@@ -744,13 +749,9 @@ __global__ __launch_bounds__(2 * kThreads, 2) void mfma_bwd_dkv_stream_kernel(KP
             }
         };
         auto deposit = [&](int s) {
-            char* qtile = bufs + (s & 1) * kBuf + 2 * kZTile;
-            char* dotile = qtile + kQTile;
+            char* xtile = bufs + (s & 1) * kBuf + 2 * kZTile + (is_dv ? kQTile : 0);
 #pragma unroll
-            for (int part = 0; part < 4; ++part) {
-                *(u32x4*)(qtile + tile_offset<D>(crow + 32 * part, cch)) = tq[part];
-                *(u32x4*)(dotile + tile_offset<D>(crow + 32 * part, cch)) = td[part];
-            }
+            for (int i = 0; i < 8; ++i) *(u32x4*)(xtile + tile_offset<D>(crow + 16 * i, cch)) = tx[i];
             if (ct < kRowBlock)
                 *(float4*)(carry + (s & 1) * kCarry + ct * 16) = float4{cR, cG, __uint_as_float(cdr), 0.f};
         };
@@ -808,8 +809,8 @@ __global__ __launch_bounds__(2 * kThreads, 2) void mfma_bwd_dkv_stream_kernel(KP
         bool store_pending = false;            // a staged dK/dV waits in Z[s&1] to be stored
         int fin_stage = cur_idx, fin_store = cur_idx;
         // B, a barrier of the four consumer waves only (the producers have no part in what it
-        // protects and must not be held up by it): a running count in LDS, bumped by each wave
-        // after its reduction, and a short spin.  All four waves are resident, so it terminates.
+        // protects and must not be held up by it): a running count in LDS, bumped by each wave,
+        // and a short spin.  All four waves are resident, so it terminates.
         int sync_target = 0;
         auto consumer_sync = [&]() {
             sync_target += 4;
@@ -833,7 +834,9 @@ __global__ __launch_bounds__(2 * kThreads, 2) void mfma_bwd_dkv_stream_kernel(KP
 #pragma unroll
                 for (int part = 0; part < 4; ++part) request_tile(rq, rq_row0, part);
             }
-            consumer_sync();                   // B: every consumer has finished with buffer (s-1)&1
+            // B, only where a finished dK/dV is staged into the Z buffer just reduced: every
+            // consumer must be through with it
+            if (finish_after_reduce) consumer_sync();
             if (keys_now) {
                 // the K tile is free once every producer holds this item's fragments
                 while (__hip_atomic_load(&producers_took_k, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) < 4 * (item + 1))
