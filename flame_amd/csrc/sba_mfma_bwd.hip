@@ -473,16 +473,16 @@ __global__ __launch_bounds__(kThreads, 2) void mfma_bwd_dkv_kernel(KParams p) {
 // vector work, and because the stream never stops at an item boundary nothing of an item's
 // set-up (launch, K/V fetch, first tiles) or tear-down (dK/dV store) is exposed.
 //
-// One iteration s of the stream (workgroup barrier A at its end; B is a barrier of the four
-// consumer waves only, a running count in LDS, so that the producers - the critical path -
-// never wait in the middle of a step):
+// One iteration s of the stream (workgroup barrier A at its end):
 //   producers:  fragments of tile[s&1] -> scores, weights, dP, dz -> Z[s&1]                    | A
 //   consumers:  store a staged dK/dV; request step s+1;
-//               reduce Z/tile[(s-1)&1]                            | B | stage a finished dK/dV
-//                                                                       into Z[(s-1)&1];
-//                                                                       deposit step s+1 -> [(s+1)&1] | A
-// B separates the reduction's last read of buffer (s-1)&1 from the stores that reuse it.  Two
-// rarer hand-overs: a staged dK/dV occupies the Z buffer that the producers write in the next
+//               reduce Z/tile[(s-1)&1]; [B] stage a finished dK/dV into Z[(s-1)&1];
+//               deposit step s+1 -> tile[(s+1)&1]                                              | A
+// A consumer wave deposits exactly the part of the tiles that its own reduction reads, so the
+// refill of buffer (s+1)&1 = (s-1)&1 only has to follow that wave's own reads.  B, needed only
+// where a finished dK/dV is staged into the Z buffer that all four consumers have just read, is
+// a barrier of the consumer waves alone (a running count in LDS): the producers - the critical
+// path - never wait in the middle of a step.  Two rarer hand-overs: a staged dK/dV occupies the Z buffer that the producers write in the next
 // iteration, so that iteration has one more workgroup barrier (X) after the consumers' store;
 // and the K tile is refilled only after a second LDS count says that every producer holds
 // the current item's K fragments.
