@@ -15,7 +15,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "csrc", "libsba_mi355x.so")
 
 SBA_DTYPE_F32, SBA_DTYPE_BF16 = 0, 1
-SBA_ABI_VERSION = 2
+SBA_ABI_VERSION = 3
 
 
 class SbaTensor(C.Structure):
@@ -114,11 +114,11 @@ def usable(t: torch.Tensor) -> torch.Tensor:
     return t if ok else t.contiguous()
 
 
-SCHEDULE_INTS = 5      # int32 per job: first_token, doc_len, row_block, doc_index, key_order
+SCHEDULE_INTS = 8      # int32 per row: {first_token, doc_len, row_block, doc_index} of job i, then of the i-th job in key-owner order
 
 
 def build_schedule(cu_host: torch.Tensor) -> torch.Tensor:
-    """Host int32 cu_seqlens (leading 0) -> host int32 [n_jobs, 5] schedule."""
+    """Host int32 cu_seqlens (leading 0) -> host int32 [n_jobs, 8] schedule."""
     lib = load()
     cu = cu_host.to(torch.int32).contiguous()
     n_seq = cu.numel() - 1

@@ -138,15 +138,17 @@ int sba_build_schedule(const int32_t* cu, int n_seq, int32_t* out, int capacity)
     std::stable_sort(jobs.begin(), jobs.end(), [](const J& a, const J& b) { return a.rb > b.rb; });
     int n = (int)jobs.size();
     if (out && capacity >= n) {
-        // column 4: the jobs again, ordered for the key-owner kernels, whose sweep from a
-        // job's row-block to the end of its sequence is (blocks of the sequence - rb) long
+        // second half of row i: the job that comes i-th for the key-owner kernels, whose sweep
+        // from a job's row-block to the end of its sequence is (blocks of the sequence - rb) long
         std::vector<int> key_order(n);
         for (int i = 0; i < n; ++i) key_order[i] = i;
         auto key_len = [&](int i) { return (jobs[i].len + sba::kRowBlock - 1) / sba::kRowBlock - jobs[i].rb; };
         std::stable_sort(key_order.begin(), key_order.end(), [&](int a, int b) { return key_len(a) > key_len(b); });
         for (int i = 0; i < n; ++i) {
             int32_t* o = out + (size_t)sba::kScheduleInts * i;
-            o[0] = jobs[i].tok0; o[1] = jobs[i].len; o[2] = jobs[i].rb; o[3] = jobs[i].doc; o[4] = key_order[i];
+            const J& k = jobs[key_order[i]];
+            o[0] = jobs[i].tok0; o[1] = jobs[i].len; o[2] = jobs[i].rb; o[3] = jobs[i].doc;
+            o[4] = k.tok0; o[5] = k.len; o[6] = k.rb; o[7] = k.doc;
         }
     }
     return n;

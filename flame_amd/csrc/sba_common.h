@@ -40,34 +40,52 @@ struct Job { int tok0, len, rb, seq; };
 // the same job and a head stays on one XCD's L2.  Jobs are sorted by decreasing sweep
 // length (longest first); `longest_last` walks the list from its other end (the key-owner
 // pass, whose work grows as the row-block index falls).
-constexpr int kScheduleInts = 5;   // {first_token, doc_len, row_block, doc_index, key_order} per job
-
 __device__ inline int order_job(int slot, int n_jobs, bool longest_last) {
     return longest_last ? n_jobs - 1 - slot : slot;
 }
 
 // Dense jobs are generated arithmetically (row-blocks in decreasing order); packed jobs
-// come from the host-built schedule, which has the same order.
-__device__ inline Job decode_job(const KParams& p, int job) {
+// come from the host-built schedule, which has the same order.  Row i of the schedule:
+// {first_token, doc_len, row_block, doc_index} of the i-th job, then the same four of the job
+// that comes i-th for the key-owner kernels.
+constexpr int kScheduleInts = 8;
+
+// The schedule is read-only for the kernels and indexed with wave-uniform values: read it
+// through the constant address space, so that the loads are scalar (one per wave, and no wait
+// for the vector-memory traffic in flight).
+typedef const __attribute__((address_space(4))) int32_t* ScheduleRow;
+__device__ inline ScheduleRow schedule_row(const KParams& p, int i, int offset) {
+    return (ScheduleRow)(uintptr_t)(p.schedule + kScheduleInts * (int64_t)i + offset);
+}
+
+__device__ inline Job dense_job(const KParams& p, int job) {
     Job j;
-    if (p.cu_seqlens == nullptr) {
-        int n_rb = (p.seq_len + kRowBlock - 1) / kRowBlock;
-        j.rb = n_rb - 1 - job / p.n_seq;
-        j.seq = job % p.n_seq;
-        j.tok0 = 0;
-        j.len = p.seq_len;
-    } else {
-        const int32_t* s = p.schedule + kScheduleInts * (int64_t)job;
-        j.tok0 = s[0]; j.len = s[1]; j.rb = s[2]; j.seq = 0;
-    }
+    int n_rb = (p.seq_len + kRowBlock - 1) / kRowBlock;
+    j.rb = n_rb - 1 - job / p.n_seq;
+    j.seq = job % p.n_seq;
+    j.tok0 = 0;
+    j.len = p.seq_len;
+    return j;
+}
+
+__device__ inline Job decode_job(const KParams& p, int job) {
+    if (p.cu_seqlens == nullptr) return dense_job(p, job);
+    const ScheduleRow s = schedule_row(p, job, 0);
+    Job j;
+    j.tok0 = s[0]; j.len = s[1]; j.rb = s[2]; j.seq = 0;
     return j;
 }
 
 // The key-owner (dK/dV) kernels sweep from a job's row-block to the END of its sequence:
 // their longest sweeps are the FIRST row-blocks of the longest sequences.  i-th job in that
-// order: arithmetic for the dense layout, column 4 of the host-built schedule for the packed.
-__device__ inline int key_order_job(const KParams& p, int i) {
-    return p.cu_seqlens == nullptr ? p.n_jobs - 1 - i : p.schedule[kScheduleInts * (int64_t)i + 4];
+// order: arithmetic for the dense layout, the second half of row i of the host-built schedule
+// for the packed.
+__device__ inline Job decode_key_job(const KParams& p, int i) {
+    if (p.cu_seqlens == nullptr) return dense_job(p, p.n_jobs - 1 - i);
+    const ScheduleRow s = schedule_row(p, i, 4);
+    Job j;
+    j.tok0 = s[0]; j.len = s[1]; j.rb = s[2]; j.seq = 0;
+    return j;
 }
 
 // Token index inside the carry tables.

@@ -327,7 +327,7 @@ __global__ __launch_bounds__(kThreads, 2) void mfma_bwd_dkv_kernel(KParams p) {
     lz.init(lane);
     const int head = blockIdx.x % p.n_heads;
     const int slot = blockIdx.x / p.n_heads;   // two 64-key blocks per scheduled 128-row job
-    const Job job = decode_job(p, key_order_job(p, slot >> 1));
+    const Job job = decode_key_job(p, slot >> 1);
     const int kb = 2 * job.rb + (slot & 1);
     const int key0 = kb * kKeyBlock;
     if (key0 >= job.len) return;               // uniform over the workgroup
@@ -500,7 +500,7 @@ __device__ inline KeyItem decode_item(const KParams& p, int idx) {
     if (idx < 0) idx = 0;
     r.head = idx % p.n_heads;
     const int slot = idx / p.n_heads;          // two 64-key blocks per scheduled 128-row job
-    r.job = decode_job(p, key_order_job(p, slot >> 1));
+    r.job = decode_key_job(p, slot >> 1);
     r.kb = 2 * r.job.rb + (slot & 1);
     r.key0 = r.kb * kKeyBlock;
     r.n_steps = (r.job.len + kRowBlock - 1) / kRowBlock - r.job.rb;

@@ -34,8 +34,8 @@
 extern "C" {
 #endif
 
-#define SBA_ABI_VERSION 2
-#define SBA_SCHEDULE_INTS 5   /* int32 per scheduled job, see sba_build_schedule() */
+#define SBA_ABI_VERSION 3
+#define SBA_SCHEDULE_INTS 8   /* int32 per scheduled job, see sba_build_schedule() */
 
 enum { SBA_DTYPE_F32 = 0, SBA_DTYPE_BF16 = 1 };
 
@@ -113,11 +113,11 @@ size_t sba_workspace_bytes(const SbaParams* p);
 
 /*
  * Row-block schedule for the packed layout, built on the host from host cu_seqlens
- * (n_seq+1 entries, leading 0).  Writes up to `capacity` jobs of SBA_SCHEDULE_INTS (5)
- * int32 each {first_token, doc_len, row_block, doc_index, key_order} into `out` (host
- * memory), longest row-blocks first, and returns the number of jobs; key_order[i] is the
- * index of the job that comes i-th for the dK/dV kernel, whose sweeps run from a row-block
- * to the END of its document (or the number needed when
+ * (n_seq+1 entries, leading 0).  Writes up to `capacity` rows of SBA_SCHEDULE_INTS (8)
+ * int32 each into `out` (host memory) and returns the number of jobs: ints 0-3 of row i are
+ * {first_token, doc_len, row_block, doc_index} of the i-th job, longest row-blocks first;
+ * ints 4-7 are the same four of the job that comes i-th for the dK/dV kernel, whose sweeps
+ * run from a row-block to the END of its document (or the number needed when
  * `out` is NULL or capacity is too small).  The caller copies it to the device and passes
  * it as SbaParams.schedule.  Replaces the reference's 3-D launch grid
  * (n_docs, ceil(H/2), ceil(max_len/64)+1) and its long/short head pairing

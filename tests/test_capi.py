@@ -30,7 +30,7 @@ def test_exports_every_declared_symbol(lib):
 
 
 def test_abi_version_and_struct_size(lib):
-    assert lib.sba_abi_version() == 2
+    assert lib.sba_abi_version() == 3
     p = _lib.SbaParams()
     p.struct_size = C.sizeof(_lib.SbaParams) - 8
     assert lib.sba_fwd(C.byref(p)) == -7          # SBA_ERR_ABI, before anything touches a GPU
@@ -73,13 +73,13 @@ def test_schedule_builder(lib):
     assert set(jobs) == expect and len(jobs) == len(expect)
     rbs = [j[2] for j in jobs]
     assert rbs == sorted(rbs, reverse=True)       # longest sweeps first
-    # column 4: a permutation of the jobs, longest key-owner sweeps (blocks of the doc - rb) first
-    order = s[:, 4].tolist()
-    assert sorted(order) == list(range(len(jobs)))
-    key_len = [(jobs[i][1] + 127) // 128 - jobs[i][2] for i in order]
+    # ints 4-7: the same jobs again, longest key-owner sweeps (blocks of the doc - rb) first
+    key_jobs = [tuple(r[4:8]) for r in s.tolist()]
+    assert sorted(key_jobs) == sorted(jobs)
+    key_len = [(j[1] + 127) // 128 - j[2] for j in key_jobs]
     assert key_len == sorted(key_len, reverse=True) and key_len[0] == 5
     # capacity too small: returns the count needed and writes nothing
-    out = torch.full((2, 5), -1, dtype=torch.int32)
+    out = torch.full((2, 8), -1, dtype=torch.int32)
     n = lib.sba_build_schedule(C.cast(cu.data_ptr(), C.POINTER(C.c_int32)), 5,
                                C.cast(out.data_ptr(), C.POINTER(C.c_int32)), 2)
     assert n == len(expect) and bool((out == -1).all())
