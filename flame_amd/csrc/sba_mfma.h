@@ -171,6 +171,56 @@ template <int D> struct TileCopy {
     }
 };
 
+// Global -> LDS copy of one 64-row tile that bypasses the registers: every instruction moves
+// 64 x 16 bytes into 1 KB of consecutive LDS, and the lane picks the global chunk that belongs
+// at its LDS position (rows in MFMA order, chunks swizzled).  Four waves copy a tile; wave w4
+// issues instructions w4, w4 + 4, ...  The per-lane byte offsets inside a tile never change, so
+// a step costs no vector address arithmetic.  Rows past the end of the sequence are clamped to
+// its last row instead of zero-filled: those keys are masked for every valid query.
+template <int D> struct TileDma {
+    static constexpr int kPerWave = 64 * D * 2 / 1024 / 4;    // 2 (D=64) or 4 (D=128)
+    uint32_t off[kPerWave];
+    int w4, lane;
+
+    __device__ static inline void where(int inst, int lane, int& kl, int& c) {
+        const int pos = inst * 64 + lane;                  // LDS chunk position
+        const int r = pos / (D / 8), pc = pos % (D / 8);
+        c = pc ^ swz<D>(r);
+        kl = (((r >> 2) & 1) << 5) | (((r >> 5) & 1) << 4) | (((r >> 3) & 3) << 2) | (r & 3);
+    }
+    __device__ inline void init(int lane_, int w4_, int64_t st) {
+        lane = lane_; w4 = w4_;
+#pragma unroll
+        for (int i = 0; i < kPerWave; ++i) {
+            int kl, c;
+            where(w4 + 4 * i, lane, kl, c);
+            off[i] = 2u * (uint32_t)(kl * (int)st + c * 8);
+        }
+    }
+    __device__ inline void issue(const TensorArg& t, int64_t base, int row0, int len, char* tile) const {
+        const char* tile_base = t.ptr + 2 * (base + (int64_t)row0 * t.st);          // uniform
+        if (row0 + 64 <= len) {
+#pragma unroll
+            for (int i = 0; i < kPerWave; ++i)
+                __builtin_amdgcn_global_load_lds(
+                    (const __attribute__((address_space(1))) void*)(tile_base + (size_t)off[i]),
+                    (__attribute__((address_space(3))) void*)(uintptr_t)(uint32_t)(uintptr_t)(tile + (w4 + 4 * i) * 1024),
+                    16, 0, 0);
+        } else {
+#pragma unroll
+            for (int i = 0; i < kPerWave; ++i) {
+                int kl, c;
+                where(w4 + 4 * i, lane, kl, c);
+                kl = min(kl, len - 1 - row0);
+                __builtin_amdgcn_global_load_lds(
+                    (const __attribute__((address_space(1))) void*)(tile_base + 2 * ((int64_t)kl * t.st + c * 8)),
+                    (__attribute__((address_space(3))) void*)(uintptr_t)(uint32_t)(uintptr_t)(tile + (w4 + 4 * i) * 1024),
+                    16, 0, 0);
+            }
+        }
+    }
+};
+
 // A operand, row fetch: lane (m = lane%32, h = lane/32) gets 8 bf16 of row 32*t + m,
 // columns 16*ks + 8*h .. +7.
 template <int D> __device__ inline bf16x8 fetch_rows(const char* tile, int t, int ks, int lane) {

@@ -40,16 +40,16 @@ __global__ __launch_bounds__(kThreads) void mfma_fwd_kernel(KParams p) {
     const int n_steps = kmax >= 0 ? kmax / kKeyBlock + 1 : 0;
     const int64_t tabtok = tab_token(p, job, qi);
 
-    TileCopy<D> kc, vc;
+    TileDma<D> kc, vc;
+    kc.init(lane, wave, p.k.st);
+    vc.init(lane, wave, p.v.st);
     if (n_steps > 0) {
-        kc.load(p.k, kbase, (n_steps - 1) * kKeyBlock, job.len);
-        vc.load(p.v, vbase, (n_steps - 1) * kKeyBlock, job.len);
-        kc.store(lds);
-        vc.store(lds + kTile);
+        kc.issue(p.k, kbase, (n_steps - 1) * kKeyBlock, job.len, lds);
+        vc.issue(p.v, vbase, (n_steps - 1) * kKeyBlock, job.len, lds + kTile);
     }
+    wait_global_memory();
     __syncthreads();
 
-    wait_global_memory();
     for (int step = n_steps - 1, buf = 0; step >= 0; --step, buf ^= 1) {
         const char* ktile = lds + buf * 2 * kTile;
         const char* vtile = ktile + kTile;
@@ -62,9 +62,9 @@ __global__ __launch_bounds__(kThreads) void mfma_fwd_kernel(KParams p) {
         // after it has completed, instead of stalling the next iteration's loads on it.
         if (!skip && p.save && h == 0 && qi < job.len)
             p.rtab[((int64_t)head * p.n_kb + step) * p.tab_tokens + tabtok] = R;
-        if (more) {
-            kc.load(p.k, kbase, (step - 1) * kKeyBlock, job.len);
-            vc.load(p.v, vbase, (step - 1) * kKeyBlock, job.len);
+        if (more) {       // next tiles, straight into the other buffer (free since the last barrier)
+            kc.issue(p.k, kbase, (step - 1) * kKeyBlock, job.len, lds + (buf ^ 1) * 2 * kTile);
+            vc.issue(p.v, vbase, (step - 1) * kKeyBlock, job.len, lds + (buf ^ 1) * 2 * kTile + kTile);
         }
         if (!skip) {
             float x[32];
@@ -83,11 +83,7 @@ mask_step(x, key0 + 32 * h, qi, strict);
                 for (int c = 0; c < 4; ++c)
                     oacc[db] = mfma(fetch_cols_o<D>(vtile, lo, db, c), pf[c], oacc[db]);
         }
-        if (more) {
-            kc.store(lds + (buf ^ 1) * 2 * kTile);
-            vc.store(lds + (buf ^ 1) * 2 * kTile + kTile);
-        }
-        wait_global_memory();                  // nothing in flight across the back edge
+        wait_global_memory();                  // the next tiles have landed
         __syncthreads();
     }
 
@@ -158,27 +154,27 @@ __global__ __launch_bounds__(2 * kThreads) void mfma_fwd2_kernel(KParams p) {
     char* my_tiles = lds + grp * 2 * kTile;          // + buf * 4 * kTile
 
     // each group copies its own tiles (256 threads per tile pair)
-    TileCopy<D> kc, vc;
+    TileDma<D> kc, vc;
+    kc.init(lane, qs, p.k.st);
+    vc.init(lane, qs, p.v.st);
     {
         const int s0 = n_steps - 1 - grp;
         if (s0 >= 0) {
-            kc.load(p.k, kbase, s0 * kKeyBlock, job.len);
-            vc.load(p.v, vbase, s0 * kKeyBlock, job.len);
-            kc.store(my_tiles);
-            vc.store(my_tiles + kTile);
+            kc.issue(p.k, kbase, s0 * kKeyBlock, job.len, my_tiles);
+            vc.issue(p.v, vbase, s0 * kKeyBlock, job.len, my_tiles + kTile);
         }
     }
+    wait_global_memory();
     __syncthreads();
 
-    wait_global_memory();
     for (int it = 0, buf = 0; it < n_it; ++it, buf ^= 1) {
         const int step = n_steps - 1 - 2 * it - grp;          // -1: this group idles in the last iteration
         const char* ktile = my_tiles + buf * 4 * kTile;
         const char* vtile = ktile + kTile;
         const bool more = step - 2 >= 0;
-        if (more) {
-            kc.load(p.k, kbase, (step - 2) * kKeyBlock, job.len);
-            vc.load(p.v, vbase, (step - 2) * kKeyBlock, job.len);
+        if (more) {       // next tiles, straight into the other buffer (free since the last barrier)
+            kc.issue(p.k, kbase, (step - 2) * kKeyBlock, job.len, my_tiles + (buf ^ 1) * 4 * kTile);
+            vc.issue(p.v, vbase, (step - 2) * kKeyBlock, job.len, my_tiles + (buf ^ 1) * 4 * kTile + kTile);
         }
         const int key0 = step * kKeyBlock;
         const bool active = step >= 0 && !(key0 + strict > q0w + 31);
@@ -210,11 +206,7 @@ __global__ __launch_bounds__(2 * kThreads) void mfma_fwd2_kernel(KParams p) {
                 for (int c = 0; c < 4; ++c)
                     oacc[db] = mfma(fetch_cols_o<D>(vtile, lo, db, c), pf[c], oacc[db]);
         }
-        if (more) {
-            kc.store(my_tiles + (buf ^ 1) * 4 * kTile);
-            vc.store(my_tiles + (buf ^ 1) * 4 * kTile + kTile);
-        }
-        wait_global_memory();                  // nothing in flight across the back edge
+        wait_global_memory();                  // the next tiles have landed
         __syncthreads();
     }
 
