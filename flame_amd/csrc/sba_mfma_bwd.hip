@@ -59,14 +59,13 @@ __global__ __launch_bounds__(kThreads) void mfma_bwd_dq_kernel(KParams p) {
     const int n_steps = kmax >= 0 ? kmax / kKeyBlock + 1 : 0;
     const int64_t tabtok = tab_token(p, job, qi);
 
-    TileCopy<D> kc, vc;
+    TileDma<D> kc, vc;
+    kc.init(lane, wave, p.k.st);
+    vc.init(lane, wave, p.v.st);
     if (n_steps > 0) {
-        kc.load(p.k, kbase, 0, job.len);
-        vc.load(p.v, vbase, 0, job.len);
-        kc.store(lds);
-        vc.store(lds + kTile);
+        kc.issue(p.k, kbase, 0, job.len, lds);
+        vc.issue(p.v, vbase, 0, job.len, lds + kTile);
     }
-    __syncthreads();
 
     // carry-table traffic is kept off the critical path: the value of the NEXT step is loaded
     // while this one is computed, and this step's prefix is stored before the tile loads are
@@ -75,6 +74,7 @@ __global__ __launch_bounds__(kThreads) void mfma_bwd_dq_kernel(KParams p) {
     const int64_t tix0 = (int64_t)head * p.n_kb * p.tab_tokens + tabtok;
     float Rnext = (row_ok && n_steps > 0) ? p.rtab[tix0] : 1.0f;
     wait_global_memory();
+    __syncthreads();
     for (int step = 0, buf = 0; step < n_steps; ++step, buf ^= 1) {
         const char* ktile = lds + buf * 2 * kTile;
         const char* vtile = ktile + kTile;
@@ -86,8 +86,9 @@ __global__ __launch_bounds__(kThreads) void mfma_bwd_dq_kernel(KParams p) {
         float R = Rnext;
         if (more) {
             if (row_ok) Rnext = p.rtab[tix + tstride];
-            kc.load(p.k, kbase, (step + 1) * kKeyBlock, job.len);
-            vc.load(p.v, vbase, (step + 1) * kKeyBlock, job.len);
+            // next tiles, straight into the other buffer (free since the last barrier)
+            kc.issue(p.k, kbase, (step + 1) * kKeyBlock, job.len, lds + (buf ^ 1) * 2 * kTile);
+            vc.issue(p.v, vbase, (step + 1) * kKeyBlock, job.len, lds + (buf ^ 1) * 2 * kTile + kTile);
         }
         if (!skip) {
             float x[32], beta[32], dp[32];
@@ -120,11 +121,7 @@ mask_step(x, key0 + 32 * h, qi, strict);
                 for (int c = 0; c < 4; ++c)
                     dqacc[db] = mfma(fetch_cols_o<D>(ktile, lo, db, c), zf[c], dqacc[db]);
         }
-        if (more) {
-            kc.store(lds + (buf ^ 1) * 2 * kTile);
-            vc.store(lds + (buf ^ 1) * 2 * kTile + kTile);
-        }
-        wait_global_memory();                  // nothing in flight across the back edge
+        wait_global_memory();                  // the next tiles have landed
         __syncthreads();
     }
 
@@ -200,20 +197,20 @@ __global__ __launch_bounds__(2 * kThreads, 2) void mfma_bwd_dq2_kernel(KParams p
     char* my_tiles = lds + grp * 2 * kTile;          // + buf * 4 * kTile
 
     // each group copies its own tiles (256 threads per tile pair)
-    TileCopy<D> kc, vc;
+    TileDma<D> kc, vc;
+    kc.init(lane, qs, p.k.st);
+    vc.init(lane, qs, p.v.st);
     if (grp < n_steps) {
-        kc.load(p.k, kbase, grp * kKeyBlock, job.len);
-        vc.load(p.v, vbase, grp * kKeyBlock, job.len);
-        kc.store(my_tiles);
-        vc.store(my_tiles + kTile);
+        kc.issue(p.k, kbase, grp * kKeyBlock, job.len, my_tiles);
+        vc.issue(p.v, vbase, grp * kKeyBlock, job.len, my_tiles + kTile);
     }
-    __syncthreads();
 
     // the forward's carry for this group's NEXT step is loaded while this one is computed
     const int64_t tstride = p.tab_tokens;
     const int64_t tix0 = (int64_t)head * p.n_kb * p.tab_tokens + tabtok;
     float Rnext = (row_ok && grp < n_steps) ? p.rtab[tix0 + grp * tstride] : 1.0f;
     wait_global_memory();
+    __syncthreads();
     for (int it = 0, buf = 0; it < n_it; ++it, buf ^= 1) {
         const int step = 2 * it + grp;                   // == n_steps: this group idles in the last iteration
         const char* ktile = my_tiles + buf * 4 * kTile;
@@ -225,8 +222,9 @@ __global__ __launch_bounds__(2 * kThreads, 2) void mfma_bwd_dq2_kernel(KParams p
         const float R = Rnext;
         if (more) {
             if (row_ok) Rnext = p.rtab[tix + 2 * tstride];
-            kc.load(p.k, kbase, (step + 2) * kKeyBlock, job.len);
-            vc.load(p.v, vbase, (step + 2) * kKeyBlock, job.len);
+            // next tiles, straight into the other buffer (free since the last barrier)
+            kc.issue(p.k, kbase, (step + 2) * kKeyBlock, job.len, my_tiles + (buf ^ 1) * 4 * kTile);
+            vc.issue(p.v, vbase, (step + 2) * kKeyBlock, job.len, my_tiles + (buf ^ 1) * 4 * kTile + kTile);
         }
         float x[32], beta[32], dp[32];
         float total = 0.f, start = 0.f;
@@ -256,11 +254,7 @@ __global__ __launch_bounds__(2 * kThreads, 2) void mfma_bwd_dq2_kernel(KParams p
                 for (int c = 0; c < 4; ++c)
                     dqacc[db] = mfma(fetch_cols_o<D>(ktile, lo, db, c), zf[c], dqacc[db]);
         }
-        if (more) {
-            kc.store(my_tiles + (buf ^ 1) * 4 * kTile);
-            vc.store(my_tiles + (buf ^ 1) * 4 * kTile + kTile);
-        }
-        wait_global_memory();                  // nothing in flight across the back edge
+        wait_global_memory();                  // the next tiles have landed
         __syncthreads();
     }
 
