@@ -2,6 +2,7 @@
 #pragma once
 #include <hip/hip_runtime.h>
 #include <stdint.h>
+#include <stdlib.h>
 #include "../../include/sba_mi355x.h"
 
 namespace sba {
@@ -112,6 +113,16 @@ template <> struct Elem<uint16_t> {   // bf16 bits
 };
 
 }  // namespace sba
+
+// Grids of at most this many workgroups take the two-steps-per-iteration kernels (head_dim 64).
+// SBA_TWO_STEP_MAX_GRID overrides it for experiments; read once per process.
+inline unsigned sba_two_step_max_grid() {
+    static const unsigned v = [] {
+        const char* e = getenv("SBA_TWO_STEP_MAX_GRID");
+        return e ? (unsigned)atoi(e) : 512u;
+    }();
+    return v;
+}
 
 // Launchers implemented in the kernel translation units.
 int sba_generic_padded_dim(int D);

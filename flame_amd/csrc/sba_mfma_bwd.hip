@@ -905,7 +905,7 @@ int sba_launch_mfma_bwd(const sba::KParams& kp, int phases, hipStream_t s) {
     const bool p1 = phases != 2, p2 = phases != 1;
     if (kp.head_dim == 64) {
         // small grids last as long as their longest sweep: take the variant that halves it
-        if (p1 && grid.x <= 512) hipLaunchKernelGGL((mfma_bwd_dq2_kernel<64>), grid, dim3(2 * kThreads), 0, s, kp);
+        if (p1 && grid.x <= sba_two_step_max_grid()) hipLaunchKernelGGL((mfma_bwd_dq2_kernel<64>), grid, dim3(2 * kThreads), 0, s, kp);
         else if (p1) hipLaunchKernelGGL((mfma_bwd_dq_kernel<64>), grid, dim3(kThreads), 0, s, kp);
         if (p2) {
             // one resident workgroup per CU, in whole rounds of the 8 XCDs (surplus workgroups

@@ -250,7 +250,7 @@ int sba_launch_mfma_fwd(const sba::KParams& kp, hipStream_t s) {
     // as its longest sweep: take the variant that halves that chain.  Larger grids are bound
     // by throughput, where the 4-wave kernel (3 waves per SIMD) is ahead (measured: already at
     // 640 workgroups).
-    const bool small_grid = grid.x <= 512;
+    const bool small_grid = grid.x <= sba_two_step_max_grid();
     if (kp.head_dim == 64 && small_grid)
         hipLaunchKernelGGL((mfma_fwd2_kernel<64>), grid, dim3(2 * kThreads), 0, s, kp);
     else if (kp.head_dim == 64)
