@@ -131,11 +131,11 @@ def build_schedule(cu_host: torch.Tensor) -> torch.Tensor:
 
 
 def workspace_upper_bound(n_heads: int, seq_len: int, tab_tokens: int, head_dim: int) -> int:
-    """Pure-Python bound on sba_workspace_bytes() (both carry tables plus the generic
+    """Pure-Python bound on sba_workspace_bytes() (the four carry tables plus the generic
     path's fp32 accumulators), usable while torch.compile traces, where no ctypes call can
     be made.  Always >= what the library asks for."""
     def up(x):
         return (x + 255) & ~255
     n_kb = (seq_len + 63) // 64
     dp = 32 if head_dim <= 32 else (64 if head_dim <= 64 else 128)
-    return 2 * up(n_heads * n_kb * tab_tokens * 4) + up(2 * tab_tokens * n_heads * dp * 4)
+    return 4 * up(n_heads * n_kb * tab_tokens * 4) + up(2 * tab_tokens * n_heads * dp * 4)

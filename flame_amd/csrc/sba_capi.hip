@@ -88,7 +88,9 @@ KParams make_kparams(const SbaParams* p) {
     if (ws && use_mfma(p)) {
         kp.rtab = (float*)ws;
         kp.gtab = (float*)(ws + table_bytes(p));
-        ws += 2 * table_bytes(p);
+        kp.rmid = (float*)(ws + 2 * table_bytes(p));
+        kp.gmid = (float*)(ws + 3 * table_bytes(p));
+        ws += 4 * table_bytes(p);
     }
     if (ws && !use_mfma_bwd(p)) kp.dkv32 = (float*)ws;
     return kp;
@@ -117,7 +119,7 @@ const char* sba_error_string(int code) {
 size_t sba_workspace_bytes(const SbaParams* p) {
     if (!p || p->n_heads <= 0 || p->seq_len <= 0 || p->head_dim <= 0 || p->head_dim > 128) return 0;
     size_t b = 0;
-    if (use_mfma(p)) b += 2 * table_bytes(p);
+    if (use_mfma(p)) b += 4 * table_bytes(p);
     if (!use_mfma_bwd(p)) b += generic_acc_bytes(p);
     return b;
 }

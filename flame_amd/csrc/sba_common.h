@@ -29,6 +29,8 @@ struct KParams {
     VectorArg rem, d_rem;
     float* rtab;                   // forward carry table  [H][n_kb][total_tokens] (x n_seq for dense)
     float* gtab;                   // backward prefix table, same shape
+    float* rmid;                   // the same two carries in the MIDDLE of each 64-key block (entering
+    float* gmid;                   //   its left / right 32 keys), written by the dQ pass
     float* dkv32;                  // generic path: fp32 dk|dv accumulators
     int n_kb;                      // carry-table columns = ceil(seq_len / kKeyBlock)
     int64_t tab_tokens;            // tokens per head in the tables (n_seq*T dense, sumT packed)

@@ -177,7 +177,7 @@ template <int D> struct TileCopy {
 // issues instructions w4, w4 + 4, ...  The per-lane byte offsets inside a tile never change, so
 // a step costs no vector address arithmetic.  Rows past the end of the sequence are clamped to
 // its last row instead of zero-filled: those keys are masked for every valid query.
-template <int D> struct TileDma {
+template <int D, bool kNatural = false> struct TileDma {      // kNatural: rows kept in their order (query tiles)
     static constexpr int kPerWave = 64 * D * 2 / 1024 / 4;    // 2 (D=64) or 4 (D=128)
     uint32_t off[kPerWave];
     int w4, lane;
@@ -186,7 +186,7 @@ template <int D> struct TileDma {
         const int pos = inst * 64 + lane;                  // LDS chunk position
         const int r = pos / (D / 8), pc = pos % (D / 8);
         c = pc ^ swz<D>(r);
-        kl = (((r >> 2) & 1) << 5) | (((r >> 5) & 1) << 4) | (((r >> 3) & 3) << 2) | (r & 3);
+        kl = kNatural ? r : (((r >> 2) & 1) << 5) | (((r >> 5) & 1) << 4) | (((r >> 3) & 3) << 2) | (r & 3);
     }
     __device__ inline void init(int lane_, int w4_, int64_t st) {
         lane = lane_; w4 = w4_;
@@ -370,7 +370,8 @@ __device__ inline void score_tiles_o(float (&x)[32], const char* ktile, const La
 // Outputs: x[idx] = A (attention weight); beta[idx] when kNeedBeta; R updated to the carry
 // for the next (left) step.
 template <bool kNeedBeta>
-__device__ inline void stick_weights(float (&x)[32], float (&beta)[kNeedBeta ? 32 : 1], float& R, int lane) {
+__device__ inline void stick_weights(float (&x)[32], float (&beta)[kNeedBeta ? 32 : 1], float& R, int lane,
+                                     float* lane_carry = nullptr) {
     float L = 1.0f;
 #pragma unroll
     for (int idx = 31; idx >= 0; --idx) {
@@ -386,6 +387,7 @@ __device__ inline void stick_weights(float (&x)[32], float (&beta)[kNeedBeta ? 3
     const float other = __shfl_xor(L, 32);
     // upper half-wave holds the right 32 keys: its chain starts from R itself
     const float F = (lane >= 32) ? R : R * other;
+    if (lane_carry) *lane_carry = F;      // the carry entering this lane's 32 keys
 #pragma unroll
     for (int idx = 0; idx < 32; ++idx) x[idx] *= F;
     R = R * L * other;
@@ -492,7 +494,7 @@ __device__ inline void dp_tiles_o(float (&dp)[32], const char* vtile, const Lane
 // not keeping the 32 prefix values alive (two passes: sum, then running prefix).
 template <bool kLowReg>
 __device__ inline void logit_grads(const float (&a)[32], const float (&beta)[32], float (&dp)[32], float& Gc,
-                                   int lane) {
+                                   int lane, float* lane_prefix = nullptr) {
     float c = 0.f;
     if (kLowReg) {
 #pragma unroll
@@ -502,6 +504,7 @@ __device__ inline void logit_grads(const float (&a)[32], const float (&beta)[32]
         }
         const float other = __shfl_xor(c, 32);
         float run = (lane >= 32) ? Gc + other : Gc;
+        if (lane_prefix) *lane_prefix = run;     // the prefix entering this lane's 32 keys
 #pragma unroll
         for (int idx = 0; idx < 32; ++idx) {
             run += dp[idx];
@@ -518,6 +521,7 @@ __device__ inline void logit_grads(const float (&a)[32], const float (&beta)[32]
         }
         const float other = __shfl_xor(c, 32);
         const float F = (lane >= 32) ? Gc + other : Gc;
+        if (lane_prefix) *lane_prefix = F;       // the prefix entering this lane's 32 keys
 #pragma unroll
         for (int idx = 0; idx < 32; ++idx) dp[idx] = __builtin_fmaf(-beta[idx], pre[idx] + F, dp[idx]);
         Gc = Gc + c + other;

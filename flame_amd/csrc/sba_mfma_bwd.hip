@@ -15,6 +15,7 @@
 //
 // Every element of the score matrix is therefore evaluated twice in the backward (once per
 // pass); in exchange nothing is reduced through memory.
+#include <string.h>
 #include "sba_mfma.h"
 
 namespace sba {
@@ -73,6 +74,9 @@ __global__ __launch_bounds__(kThreads) void mfma_bwd_dq_kernel(KParams p) {
     const int64_t tstride = p.tab_tokens;
     const int64_t tix0 = (int64_t)head * p.n_kb * p.tab_tokens + tabtok;
     float Rnext = (row_ok && n_steps > 0) ? p.rtab[tix0] : 1.0f;
+    float* mid_table = h == 0 ? p.rmid : p.gmid;
+    float mid = 0.f;
+    bool mid_pending = false;
     wait_global_memory();
     __syncthreads();
     for (int step = 0, buf = 0; step < n_steps; ++step, buf ^= 1) {
@@ -82,6 +86,8 @@ __global__ __launch_bounds__(kThreads) void mfma_bwd_dq_kernel(KParams p) {
         const int key0 = step * kKeyBlock;
         const bool skip = key0 + strict > q0w + 31;
         const int64_t tix = tix0 + step * tstride;
+        if (mid_pending && row_ok && p.rmid) mid_table[tix - tstride] = mid;
+        mid_pending = false;
         if (!skip && row_ok && h == 0) p.gtab[tix] = Gc;
         float R = Rnext;
         if (more) {
@@ -92,6 +98,7 @@ __global__ __launch_bounds__(kThreads) void mfma_bwd_dq_kernel(KParams p) {
         }
         if (!skip) {
             float x[32], beta[32], dp[32];
+            float Rlane, Glane;
             score_tiles_o<D>(x, ktile, lo, qf, p.scale2);
             if (key0 + 63 + strict > q0w) {
 mask_step(x, key0 + 32 * h, qi, strict);
@@ -100,7 +107,7 @@ mask_step(x, key0 + 32 * h, qi, strict);
                 // dP does not depend on the weights: its 16 MFMAs are spread under their vector
                 // arithmetic (measured: a gain at head_dim 128, none at 64)
                 dp_tiles_o<D>(dp, vtile, lo, dof, dr);
-                stick_weights<true>(x, beta, R, lane);
+                stick_weights<true>(x, beta, R, lane, &Rlane);
 #pragma unroll
                 for (int i = 0; i < 2 * (D / 16); ++i) {
                     __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);     // one LDS read (the MFMA's A operand)
@@ -108,10 +115,15 @@ mask_step(x, key0 + 32 * h, qi, strict);
                     __builtin_amdgcn_sched_group_barrier(0x002, 8, 0);     // eight vector instructions
                 }
             } else {
-                stick_weights<true>(x, beta, R, lane);
+                stick_weights<true>(x, beta, R, lane, &Rlane);
                 dp_tiles_o<D>(dp, vtile, lo, dof, dr);
             }
-            logit_grads<false>(x, beta, dp, Gc, lane);
+            logit_grads<false>(x, beta, dp, Gc, lane, &Glane);
+            // carries in the middle of the block, for the key-owner pass whose waves own 32 keys:
+            // the left half-wave holds the product entering the left 32 keys, the right half-wave
+            // the prefix entering the right 32 (stored at the top of the next iteration)
+            mid = h == 0 ? Rlane : Glane;
+            mid_pending = true;
             bf16x8 zf[4];
 #pragma unroll
             for (int c = 0; c < 4; ++c) zf[c] = pack8(&dp[8 * c]);
@@ -124,6 +136,7 @@ mask_step(x, key0 + 32 * h, qi, strict);
         wait_global_memory();                  // the next tiles have landed
         __syncthreads();
     }
+    if (mid_pending && row_ok && p.rmid) mid_table[tix0 + (n_steps - 1) * tstride] = mid;
 
     if (row_ok) {
         const int64_t ob = (int64_t)job.seq * p.dq.sb + (int64_t)head * p.dq.sh + (int64_t)(job.tok0 + qi) * p.dq.st;
@@ -209,6 +222,9 @@ __global__ __launch_bounds__(2 * kThreads, 2) void mfma_bwd_dq2_kernel(KParams p
     const int64_t tstride = p.tab_tokens;
     const int64_t tix0 = (int64_t)head * p.n_kb * p.tab_tokens + tabtok;
     float Rnext = (row_ok && grp < n_steps) ? p.rtab[tix0 + grp * tstride] : 1.0f;
+    float* mid_table = h == 0 ? p.rmid : p.gmid;
+    float mid = 0.f;
+    bool mid_pending = false;
     wait_global_memory();
     __syncthreads();
     for (int it = 0, buf = 0; it < n_it; ++it, buf ^= 1) {
@@ -219,6 +235,8 @@ __global__ __launch_bounds__(2 * kThreads, 2) void mfma_bwd_dq2_kernel(KParams p
         const int key0 = step * kKeyBlock;
         const bool active = step < n_steps && !(key0 + strict > q0w + 31);
         const int64_t tix = tix0 + step * tstride;
+        if (mid_pending && row_ok && p.rmid) mid_table[tix - 2 * tstride] = mid;
+        mid_pending = false;
         const float R = Rnext;
         if (more) {
             if (row_ok) Rnext = p.rtab[tix + 2 * tstride];
@@ -227,12 +245,12 @@ __global__ __launch_bounds__(2 * kThreads, 2) void mfma_bwd_dq2_kernel(KParams p
             vc.issue(p.v, vbase, (step + 2) * kKeyBlock, job.len, my_tiles + (buf ^ 1) * 4 * kTile + kTile);
         }
         float x[32], beta[32], dp[32];
-        float total = 0.f, start = 0.f;
+        float total = 0.f, start = 0.f, Rlane = 1.f;
         if (active) {
             score_tiles_o<D>(x, ktile, lo, qf, p.scale2);
             if (key0 + 63 + strict > q0w) mask_step(x, key0 + 32 * h, qi, strict);
             float Rc = R;
-            stick_weights<true>(x, beta, Rc, lane);
+            stick_weights<true>(x, beta, Rc, lane, &Rlane);
             dp_tiles_o<D>(dp, vtile, lo, dof, dr);
             start = logit_grads_local(x, dp, total, lane);
         }
@@ -244,6 +262,9 @@ __global__ __launch_bounds__(2 * kThreads, 2) void mfma_bwd_dq2_kernel(KParams p
         Gc = Gc + total + other;
         if (active) {
             if (row_ok && h == 0) p.gtab[tix] = Gmy;
+            // carries in the middle of the block (see the one-step kernel)
+            mid = h == 0 ? Rlane : Gmy + start;
+            mid_pending = true;
             logit_grads_apply(beta, dp, Gmy + start);
             bf16x8 zf[4];
 #pragma unroll
@@ -257,6 +278,8 @@ __global__ __launch_bounds__(2 * kThreads, 2) void mfma_bwd_dq2_kernel(KParams p
         wait_global_memory();                  // the next tiles have landed
         __syncthreads();
     }
+
+    if (mid_pending && row_ok && p.rmid) mid_table[tix0 + (2 * (n_it - 1) + grp) * tstride] = mid;
 
     // ---- dQ = dQ(group 0) + dQ(group 1): group 1 parks its accumulators in LDS
     float* park = (float*)lds;                              // [qs][db][r][lane]
@@ -882,6 +905,209 @@ __global__ __launch_bounds__(2 * kThreads, 2) void mfma_bwd_dkv_stream_kernel(KP
     }
 }
 
+// ---------------------------------------------------------------- pass 2, every wave on its own keys
+// One workgroup per (128-key block, head); wave w owns the 32 keys 32w..32w+31 of the block for
+// the whole sweep, K and V fragments in registers, and accumulates its [32 keys x D] slices of
+// dK and dV itself: nothing is exchanged between waves, and the only workgroup barrier is the
+// one that publishes the next 64-query Q / dO tiles (global -> LDS DMA, double-buffered).
+// A step covers 64 queries as two [32 keys x 32 queries] score tiles; lane (n, h) holds the 16
+// consecutive keys 16h..16h+15 of one query per tile.  The carries that enter the wave's 32 keys
+// come from the tables of the forward and of the dQ pass: the block-edge ones for the half of
+// a 64-key block that touches the edge, the mid-block ones for the other half.  Weights and
+// logit gradients go as bf16 [query][32 a | 32 dz] rows into a tile private to the wave and
+// come back transposed as the A operands of  dV += A^T dO  and  dK += dZ^T Q.
+__device__ inline void own_tile_weights(float (&x)[16], float (&beta)[16], float Rin, int lane) {
+    float L = 1.0f;
+#pragma unroll
+    for (int idx = 15; idx >= 0; --idx) {
+        const float e = __builtin_amdgcn_exp2f(x[idx]);
+        const float u = __builtin_amdgcn_rcpf(1.0f + e);
+        const float Ln = L * u;
+        x[idx] = L - Ln;
+        L = Ln;
+        beta[idx] = 1.0f - u;
+    }
+    const float other = __shfl_xor(L, 32);
+    const float F = (lane >= 32) ? Rin : Rin * other;       // upper half-wave: the right 16 keys
+#pragma unroll
+    for (int idx = 0; idx < 16; ++idx) x[idx] *= F;
+}
+__device__ inline void own_tile_grads(const float (&a)[16], const float (&beta)[16], float (&dp)[16], float Gin,
+                                      int lane) {
+    float c = 0.f, pre[16];
+#pragma unroll
+    for (int idx = 0; idx < 16; ++idx) {
+        dp[idx] = a[idx] * dp[idx];     // g
+        c += dp[idx];
+        pre[idx] = c;
+    }
+    const float other = __shfl_xor(c, 32);
+    const float F = (lane >= 32) ? Gin + other : Gin;
+#pragma unroll
+    for (int idx = 0; idx < 16; ++idx) dp[idx] = __builtin_fmaf(-beta[idx], pre[idx] + F, dp[idx]);
+}
+
+template <int D>
+__global__ __launch_bounds__(kThreads, D == 64 ? 2 : 1) void mfma_bwd_dkv_own_kernel(KParams p) {
+    constexpr int kQTile = 64 * D * 2;           // Q or dO tile of one step (64 queries)
+    constexpr int kZTile = 64 * 64 * 2;          // per wave: [64 queries][32 a | 32 dz] bf16
+    constexpr int kStep = 64;
+    __shared__ __attribute__((aligned(16))) char lds[4 * kQTile + 4 * kZTile];   // Q0 dO0 Q1 dO1 | one Z tile per wave
+
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int n = lane & 31, h = lane >> 5;
+    LaneOffsets<D> lo;
+    lo.init(lane);
+    LaneOffsets<64> lz;
+    lz.init(lane);
+    const int head = blockIdx.x % p.n_heads;
+    const Job job = decode_key_job(p, blockIdx.x / p.n_heads);
+    const int strict = p.attend_current ? 0 : 1;
+    const int q_begin = job.rb * kRowBlock;            // first key of the block = first query that may see it
+    const int kb0 = q_begin + 32 * wave;               // first key of this wave
+    char* ztile = lds + 4 * kQTile + wave * kZTile;
+
+    const int64_t qbase = (int64_t)job.seq * p.q.sb + (int64_t)head * p.q.sh + (int64_t)job.tok0 * p.q.st;
+    const int64_t kbase = (int64_t)job.seq * p.k.sb + (int64_t)head * p.k.sh + (int64_t)job.tok0 * p.k.st;
+    const int64_t vbase = (int64_t)job.seq * p.v.sb + (int64_t)head * p.v.sh + (int64_t)job.tok0 * p.v.st;
+    const int64_t dobase = (int64_t)job.seq * p.d_o.sb + (int64_t)head * p.d_o.sh + (int64_t)job.tok0 * p.d_o.st;
+
+    // A operands of the score tiles: MFMA row m holds key 16*((m>>2)&1) + 4*(m>>3) + (m&3) of
+    // the wave, so that the accumulator registers of a lane are 16 consecutive keys
+    bf16x8 kfr[D / 16], vfr[D / 16];
+    {
+        const int m = lane & 31;
+        const int key = kb0 + 16 * ((m >> 2) & 1) + 4 * (m >> 3) + (m & 3);
+        load_row_frags<D>(kfr, p.k, kbase, key, job.len, lane);
+        load_row_frags<D>(vfr, p.v, vbase, key, job.len, lane);
+    }
+
+    f32x16 dkacc[D / 32], dvacc[D / 32];
+#pragma unroll
+    for (int db = 0; db < D / 32; ++db) { dkacc[db] = f32x16{0}; dvacc[db] = f32x16{0}; }
+
+    const int n_steps = q_begin < job.len ? (job.len - q_begin + kStep - 1) / kStep : 0;
+
+    TileDma<D, true> qc, dc;
+    qc.init(lane, wave, p.q.st);
+    dc.init(lane, wave, p.d_o.st);
+    if (n_steps > 0) {
+        qc.issue(p.q, qbase, q_begin, job.len, lds);
+        dc.issue(p.d_o, dobase, q_begin, job.len, lds + kQTile);
+    }
+
+    // carries of a (query, this wave's 32 keys) pair: the right half of a 64-key block takes the
+    // forward's block-edge carry and the mid-block prefix, the left half the other two
+    const int kb64 = min((q_begin + 32 * wave) / kKeyBlock, p.n_kb - 1);   // (waves past the end have no work)
+    const float* rsrc = ((wave & 1) ? p.rtab : p.rmid) + ((int64_t)head * p.n_kb + kb64) * p.tab_tokens;
+    const float* gsrc = ((wave & 1) ? p.gmid : p.gtab) + ((int64_t)head * p.n_kb + kb64) * p.tab_tokens;
+    const char* drsrc = p.d_rem.ptr ? p.d_rem.ptr + 2 * ((int64_t)job.seq * p.d_rem.sb + (int64_t)head * p.d_rem.sh + job.tok0) : nullptr;
+    float Rn[2] = {1.f, 1.f}, Gn[2] = {0.f, 0.f};
+    uint32_t drn[2] = {0u, 0u};
+    auto request_carries = [&](int q0) {
+#pragma unroll
+        for (int t = 0; t < 2; ++t) {
+            const int qi = min(q0 + 32 * t + n, job.len - 1);
+            const int64_t tok = tab_token(p, job, qi);
+            Rn[t] = rsrc[tok];
+            Gn[t] = gsrc[tok];
+            if (drsrc) drn[t] = ((const uint16_t*)drsrc)[qi];
+        }
+    };
+    if (n_steps > 0) request_carries(q_begin);
+    wait_global_memory();
+    __syncthreads();
+
+    for (int step = 0, buf = 0; step < n_steps; ++step, buf ^= 1) {
+        const char* qtile = lds + buf * 2 * kQTile;
+        const char* dotile = qtile + kQTile;
+        const int q0 = q_begin + step * kStep;
+        const bool more = step + 1 < n_steps;
+        float Rin[2], Gin[2], dr[2];
+#pragma unroll
+        for (int t = 0; t < 2; ++t) { Rin[t] = Rn[t]; Gin[t] = Gn[t]; dr[t] = bf16_to_f32((uint16_t)drn[t]); }
+        if (more) {       // next tiles, straight into the other buffer (free since the last barrier)
+            qc.issue(p.q, qbase, q0 + kStep, job.len, lds + (buf ^ 1) * 2 * kQTile);
+            dc.issue(p.d_o, dobase, q0 + kStep, job.len, lds + (buf ^ 1) * 2 * kQTile + kQTile);
+            request_carries(q0 + kStep);
+        }
+        // whole step left of this wave's first key: nothing visible
+        const bool skip = kb0 + strict > q0 + kStep - 1 || kb0 >= job.len;
+        if (!skip) {
+#pragma unroll
+            for (int t = 0; t < 2; ++t) {
+                const int qt0 = q0 + 32 * t;
+                const int qi = qt0 + n;
+                // visible keys among this lane's 16 (queries past the end see none)
+                const int nvis = qi < job.len ? qi - strict - (kb0 + 16 * h) + 1 : 0;
+                const bool sees_wave = qi < job.len && qi - strict - kb0 + 1 > 0;
+                const float Rt = sees_wave ? Rin[t] : 1.0f;      // table entries of invisible pairs are not written
+                const float Gt = sees_wave ? Gin[t] : 0.0f;
+                float x[16], beta[16], dp[16];
+                {
+                    f32x16 acc = {0};
+#pragma unroll
+                    for (int ks = 0; ks < D / 16; ++ks)
+                        acc = mfma(kfr[ks], fetch_row_nat<D>(qtile, 32 * t + n, ks, lane), acc);
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) x[r] = acc[r] * p.scale2;
+                }
+                if (kb0 + 31 + strict > qt0 || qt0 + 31 >= job.len) {     // diagonal or ragged tile
+#pragma unroll
+                    for (int idx = 0; idx < 16; ++idx)
+                        if (idx >= nvis) x[idx] = -INFINITY;
+                }
+                own_tile_weights(x, beta, Rt, lane);
+                {
+                    f32x16 acc;
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) acc[r] = -dr[t];
+#pragma unroll
+                    for (int ks = 0; ks < D / 16; ++ks)
+                        acc = mfma(vfr[ks], fetch_row_nat<D>(dotile, 32 * t + n, ks, lane), acc);
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) dp[r] = acc[r];
+                }
+                // a -> columns 16h.. of row (32t + n), dz -> columns 32 + 16h..
+                *(bf16x8*)(ztile + tile_offset<64>(32 * t + n, 2 * h)) = pack8(&x[0]);
+                *(bf16x8*)(ztile + tile_offset<64>(32 * t + n, 2 * h + 1)) = pack8(&x[8]);
+                own_tile_grads(x, beta, dp, Gt, lane);
+                *(bf16x8*)(ztile + tile_offset<64>(32 * t + n, 4 + 2 * h)) = pack8(&dp[0]);
+                *(bf16x8*)(ztile + tile_offset<64>(32 * t + n, 4 + 2 * h + 1)) = pack8(&dp[8]);
+            }
+            // dV += A^T dO, dK += dZ^T Q over the 64 queries of the step
+#pragma unroll
+            for (int kk = 0; kk < 4; ++kk) {
+                const bf16x8 af = fetch_nat_o<64>(ztile, lz, 16 * kk, 0);
+                const bf16x8 zf = fetch_nat_o<64>(ztile, lz, 16 * kk, 1);
+#pragma unroll
+                for (int db = 0; db < D / 32; ++db) {
+                    dvacc[db] = mfma(af, fetch_nat_o<D>(dotile, lo, 16 * kk, db), dvacc[db]);
+                    dkacc[db] = mfma(zf, fetch_nat_o<D>(qtile, lo, 16 * kk, db), dkacc[db]);
+                }
+            }
+        }
+        wait_global_memory();                  // the next tiles and carries have landed
+        __syncthreads();
+    }
+
+    // ---- rows kb0.. of dK (scaled) and dV, through the wave's own tile as coalesced 16-byte stores
+#pragma unroll
+    for (int which = 0; which < 2; ++which) {
+        const TensorArg& out = which == 0 ? p.dk : p.dv;
+        const int64_t ob = (int64_t)job.seq * out.sb + (int64_t)head * out.sh + (int64_t)job.tok0 * out.st;
+#pragma unroll
+        for (int db = 0; db < D / 32; ++db)
+            stage_acc_tile<D>(ztile, 0, 32 * db, which == 0 ? dkacc[db] : dvacc[db], which == 0 ? p.scale : 1.0f, lane);
+        for (int c = lane; c < 32 * D / 8; c += 64) {
+            const int row = c / (D / 8), cc = c % (D / 8);
+            if (kb0 + row < job.len)
+                *(u32x4*)(out.ptr + 2 * (ob + (int64_t)(kb0 + row) * out.st + cc * 8)) = *(const u32x4*)(ztile + row * (D * 2) + cc * 16);
+        }
+    }
+}
+
 }  // namespace sba
 
 bool sba_mfma_bwd_available() { return true; }
@@ -899,25 +1125,46 @@ static int sba_cu_count() {
     return cached[dev];
 }
 
-int sba_launch_mfma_bwd(const sba::KParams& kp, int phases, hipStream_t s) {
+// SBA_DKV_KERNEL=own / =other overrides the choice between the key-owner kernels (tests run
+// both on the same inputs).
+static bool own_keys_kernel(bool by_size) {
+    const char* e = getenv("SBA_DKV_KERNEL");
+    if (e && !strcmp(e, "own")) return true;
+    if (e && !strcmp(e, "other")) return false;
+    return by_size;
+}
+
+int sba_launch_mfma_bwd(const sba::KParams& kp_in, int phases, hipStream_t s) {
     using namespace sba;
+    KParams kp = kp_in;
     dim3 grid((unsigned)kp.n_jobs * kp.n_heads);
     const bool p1 = phases != 2, p2 = phases != 1;
+    // Key-owner pass.  head_dim 64: from about three workgroups per CU on, the kernel whose waves
+    // own their keys outright is ahead; below, the resident producer/consumer stream, which splits
+    // the work into twice as many items and balances them itself.  head_dim 128: the own-keys
+    // kernel once every CU has more than one workgroup (128-key blocks); below, the kernel with
+    // 64-key blocks, which has twice as many workgroups.
+    const unsigned cus = (unsigned)sba_cu_count();
+    const bool own = own_keys_kernel(kp.head_dim == 64 ? grid.x >= 3u * cus : grid.x > cus);
+    if (!own) kp.rmid = kp.gmid = nullptr;     // only the own-keys kernel reads the mid-block carries: dQ skips them
     if (kp.head_dim == 64) {
         // small grids last as long as their longest sweep: take the variant that halves it
         if (p1 && grid.x <= sba_two_step_max_grid()) hipLaunchKernelGGL((mfma_bwd_dq2_kernel<64>), grid, dim3(2 * kThreads), 0, s, kp);
         else if (p1) hipLaunchKernelGGL((mfma_bwd_dq_kernel<64>), grid, dim3(kThreads), 0, s, kp);
-        if (p2) {
+        if (p2 && own) {
+            hipLaunchKernelGGL((mfma_bwd_dkv_own_kernel<64>), grid, dim3(kThreads), 0, s, kp);
+        } else if (p2) {
             // one resident workgroup per CU, in whole rounds of the 8 XCDs (surplus workgroups
             // find no item)
             const unsigned n_items = 2 * grid.x;
-            unsigned n_wg = n_items < (unsigned)sba_cu_count() ? n_items : (unsigned)sba_cu_count();
+            unsigned n_wg = n_items < cus ? n_items : cus;
             n_wg = (n_wg + 7) & ~7u;
             hipLaunchKernelGGL((mfma_bwd_dkv_stream_kernel<64>), dim3(n_wg), dim3(2 * kThreads), 0, s, kp);
         }
     } else {
         if (p1) hipLaunchKernelGGL((mfma_bwd_dq_kernel<128>), grid, dim3(kThreads), 0, s, kp);
-        if (p2) hipLaunchKernelGGL((mfma_bwd_dkv_kernel<128>), dim3(2 * grid.x), dim3(kThreads), 0, s, kp);
+        if (p2 && own) hipLaunchKernelGGL((mfma_bwd_dkv_own_kernel<128>), grid, dim3(kThreads), 0, s, kp);
+        else if (p2) hipLaunchKernelGGL((mfma_bwd_dkv_kernel<128>), dim3(2 * grid.x), dim3(kThreads), 0, s, kp);
     }
     return hipGetLastError() == hipSuccess ? SBA_OK : SBA_ERR_LAUNCH;
 }

@@ -324,7 +324,7 @@ def test_torch_compile_fullgraph_matches_eager():
 
 
 def test_small_and_large_grids_take_different_forward_kernels_and_agree():
-    # <= 1024 workgroups: two-step-per-iteration forward; above: one step per iteration.
+    # <= 512 workgroups: two-step-per-iteration forward; above: one step per iteration.
     # Same rows computed both ways (a batch of 1 vs the same sequence repeated 40 times).
     sb_attn, _ = _ops()
     q, k, v = (randn((1, 4, 1000, 64), 110 + i, 0.5, torch.bfloat16).cuda() for i in range(3))
@@ -337,11 +337,14 @@ def test_small_and_large_grids_take_different_forward_kernels_and_agree():
     assert max_abs(o2[39:].float().cpu(), o_ref) <= 2e-2 and max_abs(r2[39:].float().cpu(), rem_ref) <= 2e-2
 
 
-def test_small_and_large_grids_take_different_backward_kernels_and_agree():
-    # <= 1024 workgroups: two-step-per-iteration dQ kernel; above: one step per iteration.
+@pytest.mark.parametrize("D", [64, 128])
+def test_small_and_large_grids_take_different_backward_kernels_and_agree(D):
+    # <= 512 workgroups: two-step-per-iteration dQ kernel (d = 64); above: one step per iteration.
+    # Key-owner pass: the resident stream (d = 64) or the 64-key-block kernel (d = 128) on the
+    # small grid, the kernel whose waves own their keys on the large one.
     sb_attn, _ = _ops()
-    base = [randn((1, 4, 1000, 64), 120 + i, 0.5, torch.bfloat16).cuda() for i in range(3)]
-    do = randn((1, 4, 1000, 64), 130, 1.0, torch.bfloat16).cuda()
+    base = [randn((1, 4, 1000, D), 120 + i, 0.5, torch.bfloat16).cuda() for i in range(3)]
+    do = randn((1, 4, 1000, D), 130, 1.0, torch.bfloat16).cuda()
     drem = randn((1, 4, 1000), 131, 1.0, torch.bfloat16).cuda()
 
     def grads(rep):
@@ -432,11 +435,15 @@ def test_config4_size_invariants():
     _full_size_properties(fwd_bwd, ups)
 
 
-def test_randomized_packed_batches_mfma_vs_generic_backward():
+@pytest.mark.parametrize("dkv_kernel,D", [("", 64), ("own", 64), ("other", 64), ("own", 128), ("other", 128)])
+def test_randomized_packed_batches_mfma_vs_generic_backward(dkv_kernel, D, monkeypatch):
     # Seeded random packed batches (document counts, lengths around the 64/128 block edges,
     # head counts that are and are not multiples of 8, both masks): the MFMA kernels against the
     # generic vector-ALU kernels, an independent implementation, forward and all three gradients.
+    # Either key-owner kernel is forced in turn (the library picks between them by grid size).
     _, sb_attn_varlen = _ops()
+    if dkv_kernel:
+        monkeypatch.setenv("SBA_DKV_KERNEL", dkv_kernel)
     g = torch.Generator().manual_seed(1234)
     edges = [1, 2, 31, 32, 33, 63, 64, 65, 127, 128, 129, 191, 192, 193, 255, 256, 257, 384, 500, 777, 1025]
     for case in range(12):
@@ -446,9 +453,9 @@ def test_randomized_packed_batches_mfma_vs_generic_backward():
         attend_current = bool(case % 2)
         N = sum(lens)
         cu = cu_from_lengths(lens).cuda()
-        q, k, v, do = (randn((H, N, 64), 1000 + 10 * case + i, 0.5 if i < 3 else 1.0, torch.bfloat16).cuda() for i in range(4))
+        q, k, v, do = (randn((H, N, D), 1000 + 10 * case + i, 0.5 if i < 3 else 1.0, torch.bfloat16).cuda() for i in range(4))
         drem = randn((H, N), 1000 + 10 * case + 5, 1.0, torch.bfloat16).cuda()
-        print(f"case {case}: H={H} docs={n_docs} N={N} attend_current={attend_current}", flush=True)
+        print(f"case {case}: D={D} dkv={dkv_kernel!r} H={H} docs={n_docs} N={N} attend_current={attend_current}", flush=True)
 
         def run():
             qq, kk, vv = (x.clone().requires_grad_(True) for x in (q, k, v))
