@@ -180,7 +180,8 @@ template <int D> struct TileCopy {
 template <int D, bool kNatural = false> struct TileDma {      // kNatural: rows kept in their order (query tiles)
     static constexpr int kPerWave = 64 * D * 2 / 1024 / 4;    // 2 (D=64) or 4 (D=128)
     uint32_t off[kPerWave];
-    int w4, lane;
+    const char* origin;        // row 0 of the (sequence, head) slice: uniform
+    int st, w4, lane;          // row stride in elements
 
     __device__ static inline void where(int inst, int lane, int& kl, int& c) {
         const int pos = inst * 64 + lane;                  // LDS chunk position
@@ -188,17 +189,21 @@ template <int D, bool kNatural = false> struct TileDma {      // kNatural: rows 
         c = pc ^ swz<D>(r);
         kl = kNatural ? r : (((r >> 2) & 1) << 5) | (((r >> 5) & 1) << 4) | (((r >> 3) & 3) << 2) | (r & 3);
     }
-    __device__ inline void init(int lane_, int w4_, int64_t st) {
+    // Only the slice origin and the row stride are kept: holding on to the whole tensor
+    // descriptor costs scalar registers that the loops do not have.
+    __device__ inline void init(int lane_, int w4_, const TensorArg& t, int64_t base) {
         lane = lane_; w4 = w4_;
+        origin = t.ptr + 2 * base;
+        st = (int)t.st;
 #pragma unroll
         for (int i = 0; i < kPerWave; ++i) {
             int kl, c;
             where(w4 + 4 * i, lane, kl, c);
-            off[i] = 2u * (uint32_t)(kl * (int)st + c * 8);
+            off[i] = 2u * (uint32_t)(kl * st + c * 8);
         }
     }
-    __device__ inline void issue(const TensorArg& t, int64_t base, int row0, int len, char* tile) const {
-        const char* tile_base = t.ptr + 2 * (base + (int64_t)row0 * t.st);          // uniform
+    __device__ inline void issue(int row0, int len, char* tile) const {
+        const char* tile_base = origin + 2 * ((int64_t)row0 * st);          // uniform
         if (row0 + 64 <= len) {
 #pragma unroll
             for (int i = 0; i < kPerWave; ++i)
@@ -213,7 +218,7 @@ template <int D, bool kNatural = false> struct TileDma {      // kNatural: rows 
                 where(w4 + 4 * i, lane, kl, c);
                 kl = min(kl, len - 1 - row0);
                 __builtin_amdgcn_global_load_lds(
-                    (const __attribute__((address_space(1))) void*)(tile_base + 2 * ((int64_t)kl * t.st + c * 8)),
+                    (const __attribute__((address_space(1))) void*)(tile_base + 2 * ((int64_t)kl * st + c * 8)),
                     (__attribute__((address_space(3))) void*)(uintptr_t)(uint32_t)(uintptr_t)(tile + (w4 + 4 * i) * 1024),
                     16, 0, 0);
             }

@@ -61,11 +61,11 @@ __global__ __launch_bounds__(kThreads) void mfma_bwd_dq_kernel(KParams p) {
     const int64_t tabtok = tab_token(p, job, qi);
 
     TileDma<D> kc, vc;
-    kc.init(lane, wave, p.k.st);
-    vc.init(lane, wave, p.v.st);
+    kc.init(lane, wave, p.k, kbase);
+    vc.init(lane, wave, p.v, vbase);
     if (n_steps > 0) {
-        kc.issue(p.k, kbase, 0, job.len, lds);
-        vc.issue(p.v, vbase, 0, job.len, lds + kTile);
+        kc.issue(0, job.len, lds);
+        vc.issue(0, job.len, lds + kTile);
     }
 
     // carry-table traffic is kept off the critical path: the value of the NEXT step is loaded
@@ -93,8 +93,8 @@ __global__ __launch_bounds__(kThreads) void mfma_bwd_dq_kernel(KParams p) {
         if (more) {
             if (row_ok) Rnext = p.rtab[tix + tstride];
             // next tiles, straight into the other buffer (free since the last barrier)
-            kc.issue(p.k, kbase, (step + 1) * kKeyBlock, job.len, lds + (buf ^ 1) * 2 * kTile);
-            vc.issue(p.v, vbase, (step + 1) * kKeyBlock, job.len, lds + (buf ^ 1) * 2 * kTile + kTile);
+            kc.issue((step + 1) * kKeyBlock, job.len, lds + (buf ^ 1) * 2 * kTile);
+            vc.issue((step + 1) * kKeyBlock, job.len, lds + (buf ^ 1) * 2 * kTile + kTile);
         }
         if (!skip) {
             float x[32], beta[32], dp[32];
@@ -211,11 +211,11 @@ __global__ __launch_bounds__(2 * kThreads, 2) void mfma_bwd_dq2_kernel(KParams p
 
     // each group copies its own tiles (256 threads per tile pair)
     TileDma<D> kc, vc;
-    kc.init(lane, qs, p.k.st);
-    vc.init(lane, qs, p.v.st);
+    kc.init(lane, qs, p.k, kbase);
+    vc.init(lane, qs, p.v, vbase);
     if (grp < n_steps) {
-        kc.issue(p.k, kbase, grp * kKeyBlock, job.len, my_tiles);
-        vc.issue(p.v, vbase, grp * kKeyBlock, job.len, my_tiles + kTile);
+        kc.issue(grp * kKeyBlock, job.len, my_tiles);
+        vc.issue(grp * kKeyBlock, job.len, my_tiles + kTile);
     }
 
     // the forward's carry for this group's NEXT step is loaded while this one is computed
@@ -241,8 +241,8 @@ __global__ __launch_bounds__(2 * kThreads, 2) void mfma_bwd_dq2_kernel(KParams p
         if (more) {
             if (row_ok) Rnext = p.rtab[tix + 2 * tstride];
             // next tiles, straight into the other buffer (free since the last barrier)
-            kc.issue(p.k, kbase, (step + 2) * kKeyBlock, job.len, my_tiles + (buf ^ 1) * 4 * kTile);
-            vc.issue(p.v, vbase, (step + 2) * kKeyBlock, job.len, my_tiles + (buf ^ 1) * 4 * kTile + kTile);
+            kc.issue((step + 2) * kKeyBlock, job.len, my_tiles + (buf ^ 1) * 4 * kTile);
+            vc.issue((step + 2) * kKeyBlock, job.len, my_tiles + (buf ^ 1) * 4 * kTile + kTile);
         }
         float x[32], beta[32], dp[32];
         float total = 0.f, start = 0.f, Rlane = 1.f;
@@ -990,11 +990,11 @@ __global__ __launch_bounds__(kThreads, D == 64 ? 2 : 1) void mfma_bwd_dkv_own_ke
     const int n_steps = q_begin < job.len ? (job.len - q_begin + kStep - 1) / kStep : 0;
 
     TileDma<D, true> qc, dc;
-    qc.init(lane, wave, p.q.st);
-    dc.init(lane, wave, p.d_o.st);
+    qc.init(lane, wave, p.q, qbase);
+    dc.init(lane, wave, p.d_o, dobase);
     if (n_steps > 0) {
-        qc.issue(p.q, qbase, q_begin, job.len, lds);
-        dc.issue(p.d_o, dobase, q_begin, job.len, lds + kQTile);
+        qc.issue(q_begin, job.len, lds);
+        dc.issue(q_begin, job.len, lds + kQTile);
     }
 
     // carries of a (query, this wave's 32 keys) pair: the right half of a 64-key block takes the
@@ -1028,8 +1028,8 @@ __global__ __launch_bounds__(kThreads, D == 64 ? 2 : 1) void mfma_bwd_dkv_own_ke
 #pragma unroll
         for (int t = 0; t < 2; ++t) { Rin[t] = Rn[t]; Gin[t] = Gn[t]; dr[t] = bf16_to_f32((uint16_t)drn[t]); }
         if (more) {       // next tiles, straight into the other buffer (free since the last barrier)
-            qc.issue(p.q, qbase, q0 + kStep, job.len, lds + (buf ^ 1) * 2 * kQTile);
-            dc.issue(p.d_o, dobase, q0 + kStep, job.len, lds + (buf ^ 1) * 2 * kQTile + kQTile);
+            qc.issue(q0 + kStep, job.len, lds + (buf ^ 1) * 2 * kQTile);
+            dc.issue(q0 + kStep, job.len, lds + (buf ^ 1) * 2 * kQTile + kQTile);
             request_carries(q0 + kStep);
         }
         // whole step left of this wave's first key: nothing visible

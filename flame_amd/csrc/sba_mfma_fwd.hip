@@ -41,11 +41,11 @@ __global__ __launch_bounds__(kThreads) void mfma_fwd_kernel(KParams p) {
     const int64_t tabtok = tab_token(p, job, qi);
 
     TileDma<D> kc, vc;
-    kc.init(lane, wave, p.k.st);
-    vc.init(lane, wave, p.v.st);
+    kc.init(lane, wave, p.k, kbase);
+    vc.init(lane, wave, p.v, vbase);
     if (n_steps > 0) {
-        kc.issue(p.k, kbase, (n_steps - 1) * kKeyBlock, job.len, lds);
-        vc.issue(p.v, vbase, (n_steps - 1) * kKeyBlock, job.len, lds + kTile);
+        kc.issue((n_steps - 1) * kKeyBlock, job.len, lds);
+        vc.issue((n_steps - 1) * kKeyBlock, job.len, lds + kTile);
     }
     wait_global_memory();
     __syncthreads();
@@ -63,8 +63,8 @@ __global__ __launch_bounds__(kThreads) void mfma_fwd_kernel(KParams p) {
         if (!skip && p.save && h == 0 && qi < job.len)
             p.rtab[((int64_t)head * p.n_kb + step) * p.tab_tokens + tabtok] = R;
         if (more) {       // next tiles, straight into the other buffer (free since the last barrier)
-            kc.issue(p.k, kbase, (step - 1) * kKeyBlock, job.len, lds + (buf ^ 1) * 2 * kTile);
-            vc.issue(p.v, vbase, (step - 1) * kKeyBlock, job.len, lds + (buf ^ 1) * 2 * kTile + kTile);
+            kc.issue((step - 1) * kKeyBlock, job.len, lds + (buf ^ 1) * 2 * kTile);
+            vc.issue((step - 1) * kKeyBlock, job.len, lds + (buf ^ 1) * 2 * kTile + kTile);
         }
         if (!skip) {
             float x[32];
@@ -155,13 +155,13 @@ __global__ __launch_bounds__(2 * kThreads) void mfma_fwd2_kernel(KParams p) {
 
     // each group copies its own tiles (256 threads per tile pair)
     TileDma<D> kc, vc;
-    kc.init(lane, qs, p.k.st);
-    vc.init(lane, qs, p.v.st);
+    kc.init(lane, qs, p.k, kbase);
+    vc.init(lane, qs, p.v, vbase);
     {
         const int s0 = n_steps - 1 - grp;
         if (s0 >= 0) {
-            kc.issue(p.k, kbase, s0 * kKeyBlock, job.len, my_tiles);
-            vc.issue(p.v, vbase, s0 * kKeyBlock, job.len, my_tiles + kTile);
+            kc.issue(s0 * kKeyBlock, job.len, my_tiles);
+            vc.issue(s0 * kKeyBlock, job.len, my_tiles + kTile);
         }
     }
     wait_global_memory();
@@ -173,8 +173,8 @@ __global__ __launch_bounds__(2 * kThreads) void mfma_fwd2_kernel(KParams p) {
         const char* vtile = ktile + kTile;
         const bool more = step - 2 >= 0;
         if (more) {       // next tiles, straight into the other buffer (free since the last barrier)
-            kc.issue(p.k, kbase, (step - 2) * kKeyBlock, job.len, my_tiles + (buf ^ 1) * 4 * kTile);
-            vc.issue(p.v, vbase, (step - 2) * kKeyBlock, job.len, my_tiles + (buf ^ 1) * 4 * kTile + kTile);
+            kc.issue((step - 2) * kKeyBlock, job.len, my_tiles + (buf ^ 1) * 4 * kTile);
+            vc.issue((step - 2) * kKeyBlock, job.len, my_tiles + (buf ^ 1) * 4 * kTile + kTile);
         }
         const int key0 = step * kKeyBlock;
         const bool active = step >= 0 && !(key0 + strict > q0w + 31);
