@@ -697,7 +697,11 @@ __global__ __launch_bounds__(2 * kThreads, 2) void mfma_bwd_dkv_stream_kernel(KP
         u32x4 tx[8];
         float cR, cG;
         uint32_t cdr = 0;                      // bf16 bits
-        const int crow = lane >> 2, cch = 4 * dbw + (lane & 3);
+        // Four lanes fill the 64 bytes of a row that this wave reduces; an LDS write cycle takes eight
+        // lanes, i.e. two rows, whose swizzles must differ in the bit that selects the other half of the
+        // row's banks: rows r and r + 2 do (r and r + 1 would collide), hence the order 0 2 1 3 ...
+        const int crow4 = lane >> 2;
+        const int crow = (crow4 & ~3) | ((crow4 & 1) << 1) | ((crow4 >> 1) & 1), cch = 4 * dbw + (lane & 3);
         // The tile requests of a step are issued two at a time between the MFMAs of the
         // reduction: all CUs stream their tiles from L2 in the same phase of a step, the
         // memory pipe then accepts about one 1 KB wave load per 80 cycles, and a burst of
