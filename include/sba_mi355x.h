@@ -105,7 +105,8 @@ const char* sba_error_string(int code);
 /*
  * Bytes of device workspace the pair (sba_fwd with save_for_backward, sba_bwd) needs for
  * this problem.  The forward writes its per-key-block carry table there and the backward
- * reads it back, so the SAME buffer, untouched in between, must be given to both calls
+ * reads it back (and keeps three more tables of the same size there between its two
+ * kernels), so the SAME buffer, untouched in between, must be given to both calls
  * (the Python layer keeps it in the autograd context the way the reference keeps
  * neg_log_acc, sb_attn/__init__.py:30).  Only the size fields of `p` are read.
  */

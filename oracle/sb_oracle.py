@@ -29,7 +29,9 @@ so the oracle is pinned by (tests/test_oracle.py): closed forms (q = 0 gives
 A_ij = 2^-(i-j), rem_i = 2^-i), the identity sum_j A_ij + rem_i = 1, an independent
 float64 brute-force evaluation of the product formula written in C (oracle/sb_oracle.c,
 hand-derived gradients), central finite differences, equality of the literal einsum form
-with the cumulative-sum form, and the block-diagonal property of the packed layout.
+with the cumulative-sum form, the block-diagonal property of the packed layout, and the
+golden vectors of tests/golden (the product formula and central differences of the loss in
+50-digit arithmetic, tests/golden/make_vectors.py; reproduced to 1e-12 in tests/test_golden.py).
 The one behaviour none of these pins is sb_ref.py's rounding order when it is *run in
 bf16* (log_z / log_beta cast back to bf16 before the einsum): "parity unpinned" for
 that; all tolerances here are against the oracle evaluated in fp32/fp64 on the same
