@@ -423,6 +423,45 @@ __device__ inline float stick_weights_local(float (&x)[32], float (&beta)[kNeedB
     total = L * other;
     return (lane >= 32) ? 1.0f : other;
 }
+// Forward-only variants of the two functions above, one vector instruction per key cheaper:
+// the chain runs on W = prod (1 + e) with a fused multiply-add (W += W * e) and L = 1 / W, so the
+// add, the reciprocal's multiply and the subtraction of the plain chain become fma, rcp, sub.
+// W may overflow to +inf: then L = 0 and every further weight is 0, as it should be (the true
+// values are below 2^-128).  The one hazard is a key with e = 0 exactly (a logit below -126 in
+// base 2) AFTER the overflow: inf * 0 makes W, L and the weights NaN from there on, where 0 is
+// right.  The weights lie in [0, 1], so the multiplication by the carry that finishes them
+// carries the hardware's clamp modifier, which costs nothing and turns NaN into 0 (the kernels
+// run with the DX10 clamp mode on, the default); the carry itself is clamped once per step.
+// Masked keys (e = 0) come first in the chain, while W is still 1, and are exact.
+__device__ inline float clamp01(float v) { return __builtin_amdgcn_fmed3f(v, 0.0f, 1.0f); }
+__device__ inline float product_chain(float (&x)[32]) {
+    float W = 1.0f, L = 1.0f;
+#pragma unroll
+    for (int idx = 31; idx >= 0; --idx) {
+        const float e = __builtin_amdgcn_exp2f(x[idx]);
+        W = __builtin_fmaf(W, e, W);
+        const float Ln = __builtin_amdgcn_rcpf(W);
+        x[idx] = L - Ln;
+        L = Ln;
+    }
+    return clamp01(L);
+}
+__device__ inline void scale32_clamped(float (&x)[32], float f) {
+#pragma unroll
+    for (int idx = 0; idx < 32; ++idx) x[idx] = clamp01(x[idx] * f);
+}
+__device__ inline void stick_weights_product(float (&x)[32], float& R, int lane) {
+    const float L = product_chain(x);
+    const float other = __shfl_xor(L, 32);
+    scale32_clamped(x, (lane >= 32) ? R : R * other);
+    R = R * L * other;
+}
+__device__ inline float stick_weights_local_product(float (&x)[32], float& total, int lane) {
+    const float L = product_chain(x);
+    const float other = __shfl_xor(L, 32);
+    total = L * other;
+    return (lane >= 32) ? 1.0f : other;
+}
 __device__ inline void scale32(float (&x)[32], float f) {
 #pragma unroll
     for (int idx = 0; idx < 32; ++idx) x[idx] *= f;

@@ -109,6 +109,39 @@ def test_bf16_saturated_logits(D):
         assert rel_l2(g_.float().cpu(), ref) <= 5e-2
 
 
+@pytest.mark.parametrize("D,rep", [(64, 1), (64, 100), (128, 1)])
+def test_bf16_overflow_followed_by_exact_zero_inside_one_key_group(D, rep):
+    # Inside the 32 keys that one lane chains over: logits of +80 (the running product of
+    # 1 + e^z overflows) and, further left, logits of -200 (e^z is exactly 0 in fp32).  A chain
+    # kept as that product meets inf * 0 there; the result must be finite and right: all
+    # attention mass sits on the first +80 key, everything left of it gets weight 0.
+    # rep = 100 repeats the batch row so that the large-grid forward kernel runs too.
+    sb_attn, _ = _ops()
+    H, T = 2, 300
+    q, k, v = (randn((1, H, T, D), 140 + i, 0.5 if i < 2 else 1.0) for i in range(3))
+    q[:, :, 200:, :] = 0
+    q[:, :, 200:, 3] = 2.0 * math.sqrt(D)          # queries 200.. look along one coordinate
+    k[:, :, 150:158, :] = 0
+    k[:, :, 150:158, 3] = 40.0                     # logit +80
+    k[:, :, 130:138, :] = 0
+    k[:, :, 130:138, 3] = -100.0                   # logit -200
+    q, k, v = (x.to(torch.bfloat16) for x in (q, k, v))
+    z = (q.float() @ k.float().transpose(-1, -2)) / math.sqrt(D)
+    assert z.max() >= 79 and z.min() <= -199
+    do = randn((1, H, T, D), 144, 1.0, torch.bfloat16)
+    print(f"overflow-then-zero D{D} rep{rep}", flush=True)
+    qg, kg, vg = (x.expand(rep, -1, -1, -1).contiguous().cuda().requires_grad_(True) for x in (q, k, v))
+    o, rem = sb_attn(qg, kg, vg)
+    o_ref, rem_ref, dq_ref, dk_ref, dv_ref = O.sb_attn_grads_oracle(q, k, v, do, None, compute_dtype=torch.float64)
+    assert torch.isfinite(o).all() and torch.isfinite(rem).all()
+    for b in (0, rep - 1):
+        assert max_abs(o[b:b + 1].float().cpu(), o_ref) <= 2e-2 and max_abs(rem[b:b + 1].float().cpu(), rem_ref) <= 2e-2
+    (o.float() * do.expand(rep, -1, -1, -1).cuda().float()).sum().backward()
+    for g_, ref in ((qg.grad, dq_ref), (kg.grad, dk_ref), (vg.grad, dv_ref)):
+        assert torch.isfinite(g_).all()
+        assert rel_l2(g_[:1].float().cpu(), ref) <= 5e-2
+
+
 def _check_varlen(H, D, lens, dtype, attend_current=False, seed=0, in_scale=0.5):
     _, sb_attn_varlen = _ops()
     N = sum(lens)
