@@ -366,35 +366,55 @@ __device__ inline void score_tiles_o(float (&x)[32], const char* ktile, const La
 
 // In-place: x[idx] (base-2 logits, idx = key offset inside this lane's 32 keys; invalid
 // pairs already set to -inf) -> stick-breaking weights of this step, given the carry
-// `R` = product of (1 - beta) over all keys right of this 64-key step.
-//   e = 2^x, u = 1/(1+e) = 1 - beta;  a = beta * (product of u right of the key).
-// e may overflow to +inf for huge logits: then u = 0 and beta = 1 exactly, no NaN, so no
-// clamp is needed; -inf (masked) gives e = 0, u = 1, beta = 0.
-// The chain runs right-to-left inside the lane's 32 keys from 1; one exchange between
-// the half-waves supplies the factor the lower (left) half is missing.
+// `R` = product of (1 - beta) over all keys right of the step.
+//
+// The chain runs right-to-left inside the lane's 32 keys on  W = prod (1 + e),  e = 2^x:
+//     W' = fma(W, e, W),   L' = 1 / W'  (= product of 1 - beta so far),   a = L - L',
+//     beta = 1 - W / W' = fma(-W, L', 1)
+// i.e. exp, fma, rcp, sub (and one fma for beta) per key; forming u = 1 / (1 + e) and L' = L u
+// costs one instruction more.  Masked keys (x = -inf, e = 0) leave W unchanged and get a = 0,
+// beta = 0 exactly.  W may overflow to +inf: then L' = 0 and every weight left of that key is 0,
+// as it should be (the true values are below 2^-128).  Two expressions meet inf * 0 after such an
+// overflow, where the right value is 0: W' itself when a later e is exactly 0 (a logit below
+// -126), and beta (-inf * 0).  Both values lie in [0, 1], and so do the finished weights: the
+// instructions that produce them carry the hardware's clamp modifier, which costs nothing and
+// turns NaN into 0 (the kernels run with the DX10 clamp mode on, the default); the carry is
+// clamped once per step.  (With beta = 0 there, dz = g - beta * prefix = 0, which is right: all
+// g left of an overflow are 0.)
+// One exchange between the half-waves supplies the factor the lower (left) half is missing.
 // Outputs: x[idx] = A (attention weight); beta[idx] when kNeedBeta; R updated to the carry
-// for the next (left) step.
+// for the next (left) step; *lane_carry = the carry entering this lane's 32 keys.
+__device__ inline float clamp01(float v) { return __builtin_amdgcn_fmed3f(v, 0.0f, 1.0f); }
+
+template <bool kNeedBeta, int N>
+__device__ inline float product_chain(float (&x)[N], float (&beta)[kNeedBeta ? N : 1]) {
+    float W = 1.0f, L = 1.0f;
+#pragma unroll
+    for (int idx = N - 1; idx >= 0; --idx) {
+        const float e = __builtin_amdgcn_exp2f(x[idx]);
+        const float Wn = __builtin_fmaf(W, e, W);
+        const float Ln = __builtin_amdgcn_rcpf(Wn);
+        x[idx] = L - Ln;
+        if (kNeedBeta) beta[idx] = clamp01(__builtin_fmaf(-W, Ln, 1.0f));
+        W = Wn;
+        L = Ln;
+    }
+    return clamp01(L);
+}
+template <int N> __device__ inline void scale_clamped(float (&x)[N], float f) {
+#pragma unroll
+    for (int idx = 0; idx < N; ++idx) x[idx] = clamp01(x[idx] * f);
+}
+
 template <bool kNeedBeta>
 __device__ inline void stick_weights(float (&x)[32], float (&beta)[kNeedBeta ? 32 : 1], float& R, int lane,
                                      float* lane_carry = nullptr) {
-    float L = 1.0f;
-#pragma unroll
-    for (int idx = 31; idx >= 0; --idx) {
-        float e = __builtin_amdgcn_exp2f(x[idx]);
-        float u = __builtin_amdgcn_rcpf(1.0f + e);
-        // beta * L = L - u * L, and u * L is the next value of the chain anyway: one instruction
-        // less than forming beta first (the rounding error, one ulp of L, is the same)
-        const float Ln = L * u;
-        x[idx] = L - Ln;
-        L = Ln;
-        if (kNeedBeta) beta[idx] = 1.0f - u;
-    }
+    const float L = product_chain<kNeedBeta, 32>(x, beta);
     const float other = __shfl_xor(L, 32);
     // upper half-wave holds the right 32 keys: its chain starts from R itself
     const float F = (lane >= 32) ? R : R * other;
     if (lane_carry) *lane_carry = F;      // the carry entering this lane's 32 keys
-#pragma unroll
-    for (int idx = 0; idx < 32; ++idx) x[idx] *= F;
+    scale_clamped<32>(x, F);
     R = R * L * other;
 }
 
@@ -403,68 +423,14 @@ __device__ inline void stick_weights(float (&x)[32], float (&beta)[kNeedBeta ? 3
 //   part 1: x[idx] <- weights relative to the right edge of THIS lane's 32 keys; returns the
 //           factor that completes them inside the step (1 for the upper half-wave, the upper
 //           half's product for the lower) and, in `total`, the product over all 64 keys;
-//   part 2: x[idx] *= carry * factor.
+//   part 2: scale_clamped(x, carry * factor).
 template <bool kNeedBeta>
 __device__ inline float stick_weights_local(float (&x)[32], float (&beta)[kNeedBeta ? 32 : 1], float& total,
                                             int lane) {
-    float L = 1.0f;
-#pragma unroll
-    for (int idx = 31; idx >= 0; --idx) {
-        float e = __builtin_amdgcn_exp2f(x[idx]);
-        float u = __builtin_amdgcn_rcpf(1.0f + e);
-        // beta * L = L - u * L, and u * L is the next value of the chain anyway: one instruction
-        // less than forming beta first (the rounding error, one ulp of L, is the same)
-        const float Ln = L * u;
-        x[idx] = L - Ln;
-        L = Ln;
-        if (kNeedBeta) beta[idx] = 1.0f - u;
-    }
+    const float L = product_chain<kNeedBeta, 32>(x, beta);
     const float other = __shfl_xor(L, 32);
     total = L * other;
     return (lane >= 32) ? 1.0f : other;
-}
-// Forward-only variants of the two functions above, one vector instruction per key cheaper:
-// the chain runs on W = prod (1 + e) with a fused multiply-add (W += W * e) and L = 1 / W, so the
-// add, the reciprocal's multiply and the subtraction of the plain chain become fma, rcp, sub.
-// W may overflow to +inf: then L = 0 and every further weight is 0, as it should be (the true
-// values are below 2^-128).  The one hazard is a key with e = 0 exactly (a logit below -126 in
-// base 2) AFTER the overflow: inf * 0 makes W, L and the weights NaN from there on, where 0 is
-// right.  The weights lie in [0, 1], so the multiplication by the carry that finishes them
-// carries the hardware's clamp modifier, which costs nothing and turns NaN into 0 (the kernels
-// run with the DX10 clamp mode on, the default); the carry itself is clamped once per step.
-// Masked keys (e = 0) come first in the chain, while W is still 1, and are exact.
-__device__ inline float clamp01(float v) { return __builtin_amdgcn_fmed3f(v, 0.0f, 1.0f); }
-__device__ inline float product_chain(float (&x)[32]) {
-    float W = 1.0f, L = 1.0f;
-#pragma unroll
-    for (int idx = 31; idx >= 0; --idx) {
-        const float e = __builtin_amdgcn_exp2f(x[idx]);
-        W = __builtin_fmaf(W, e, W);
-        const float Ln = __builtin_amdgcn_rcpf(W);
-        x[idx] = L - Ln;
-        L = Ln;
-    }
-    return clamp01(L);
-}
-__device__ inline void scale32_clamped(float (&x)[32], float f) {
-#pragma unroll
-    for (int idx = 0; idx < 32; ++idx) x[idx] = clamp01(x[idx] * f);
-}
-__device__ inline void stick_weights_product(float (&x)[32], float& R, int lane) {
-    const float L = product_chain(x);
-    const float other = __shfl_xor(L, 32);
-    scale32_clamped(x, (lane >= 32) ? R : R * other);
-    R = R * L * other;
-}
-__device__ inline float stick_weights_local_product(float (&x)[32], float& total, int lane) {
-    const float L = product_chain(x);
-    const float other = __shfl_xor(L, 32);
-    total = L * other;
-    return (lane >= 32) ? 1.0f : other;
-}
-__device__ inline void scale32(float (&x)[32], float f) {
-#pragma unroll
-    for (int idx = 0; idx < 32; ++idx) x[idx] *= f;
 }
 
 // Sets the logits of invisible (query, key) pairs of a diagonal step to -inf.

@@ -921,20 +921,9 @@ __global__ __launch_bounds__(2 * kThreads, 2) void mfma_bwd_dkv_stream_kernel(KP
 // logit gradients go as bf16 [query][32 a | 32 dz] rows into a tile private to the wave and
 // come back transposed as the A operands of  dV += A^T dO  and  dK += dZ^T Q.
 __device__ inline void own_tile_weights(float (&x)[16], float (&beta)[16], float Rin, int lane) {
-    float L = 1.0f;
-#pragma unroll
-    for (int idx = 15; idx >= 0; --idx) {
-        const float e = __builtin_amdgcn_exp2f(x[idx]);
-        const float u = __builtin_amdgcn_rcpf(1.0f + e);
-        const float Ln = L * u;
-        x[idx] = L - Ln;
-        L = Ln;
-        beta[idx] = 1.0f - u;
-    }
+    const float L = product_chain<true, 16>(x, beta);
     const float other = __shfl_xor(L, 32);
-    const float F = (lane >= 32) ? Rin : Rin * other;       // upper half-wave: the right 16 keys
-#pragma unroll
-    for (int idx = 0; idx < 16; ++idx) x[idx] *= F;
+    scale_clamped<16>(x, (lane >= 32) ? Rin : Rin * other);       // upper half-wave: the right 16 keys
 }
 __device__ inline void own_tile_grads(const float (&a)[16], const float (&beta)[16], float (&dp)[16], float Gin,
                                       int lane) {

@@ -72,7 +72,8 @@ __global__ __launch_bounds__(kThreads) void mfma_fwd_kernel(KParams p) {
             if (key0 + 63 + strict > q0w) {     // diagonal region: mask invisible pairs
 mask_step(x, key0 + 32 * h, qi, strict);
             }
-            stick_weights_product(x, R, lane);
+            float dummy[1];
+            stick_weights<false>(x, dummy, R, lane);
             bf16x8 pf[4];
 #pragma unroll
             for (int c = 0; c < 4; ++c) pf[c] = pack8(&x[8 * c]);
@@ -182,7 +183,8 @@ __global__ __launch_bounds__(2 * kThreads) void mfma_fwd2_kernel(KParams p) {
         if (active) {
             score_tiles_o<D>(x, ktile, lo, qf, p.scale2);
             if (key0 + 63 + strict > q0w) mask_step(x, key0 + 32 * h, qi, strict);
-            fac = stick_weights_local_product(x, total, lane);
+            float dummy[1];
+            fac = stick_weights_local<false>(x, dummy, total, lane);
         }
         if (h == 0) xch[grp][32 * qs + n] = total;
         __syncthreads();
@@ -194,7 +196,7 @@ __global__ __launch_bounds__(2 * kThreads) void mfma_fwd2_kernel(KParams p) {
         if (active) {
             if (p.save && h == 0 && qi < job.len)
                 p.rtab[((int64_t)head * p.n_kb + step) * p.tab_tokens + tabtok] = Rmy;
-            scale32_clamped(x, fac * Rmy);
+            scale_clamped<32>(x, fac * Rmy);
             bf16x8 pf[4];
 #pragma unroll
             for (int c = 0; c < 4; ++c) pf[c] = pack8(&x[8 * c]);
