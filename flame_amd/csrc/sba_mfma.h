@@ -92,7 +92,16 @@ __device__ inline s16x4 lds_read_tr(const char* p) {
         (__attribute__((address_space(3))) s16x4*)(uintptr_t)(uint32_t)(uintptr_t)p);
 }
 
-// Same three fetches as fetch_rows / fetch_cols / fetch_cols_nat, from precomputed offsets.
+// The three operand fetches, from the precomputed lane offsets:
+//   fetch_rows_o  row fetch: lane (m = lane%32, h = lane/32) gets 8 bf16 of row 32*t + m, columns
+//                 16*ks + 8*h .. +7;
+//   fetch_cols_o  transposing fetch from an MFMA-order tile: lane (m, h) gets column 32*db + m of
+//                 the 8 keys key_local = 32*h + 8*c + j, j = 0..7.  Each ds_read_b64_tr_b16 makes 16
+//                 lanes read a [4 rows x 16 columns] block (lane s: row s/4, columns 4*(s%4)..+3)
+//                 and hands lane s column s of it;
+//   fetch_nat_o   the same from a tile whose rows are in NATURAL order (Q, dO, and the weight
+//                 tiles of the key-owner pass): lane (m, h) gets column 32*cb + m of rows
+//                 row0 + 8*h + j, j = 0..7.
 template <int D> __device__ inline bf16x8 fetch_rows_o(const char* tile, const LaneOffsets<D>& o, int t, int ks) {
     return *(const bf16x8*)(tile + o.rows[ks] + t * 32 * D * 2);
 }
@@ -161,14 +170,6 @@ template <int D> struct TileCopy {
         for (int r = 0; r < kPerThread; ++r)
             *(u32x4*)(tile + tile_offset<D>(mfma_row_of_key(kl + r * kRowStep), c)) = regs[r];
     }
-    // rows kept in their natural order (query tiles)
-    __device__ inline void store_nat(char* tile) const {
-        const int tid = threadIdx.x & (kThreads - 1);
-        const int kl = tid / (D / 8), c = tid % (D / 8);
-#pragma unroll
-        for (int r = 0; r < kPerThread; ++r)
-            *(u32x4*)(tile + tile_offset<D>(kl + r * kRowStep, c)) = regs[r];
-    }
 };
 
 // Global -> LDS copy of one 64-row tile that bypasses the registers: every instruction moves
@@ -225,33 +226,6 @@ template <int D, bool kNatural = false> struct TileDma {      // kNatural: rows 
         }
     }
 };
-
-// A operand, row fetch: lane (m = lane%32, h = lane/32) gets 8 bf16 of row 32*t + m,
-// columns 16*ks + 8*h .. +7.
-template <int D> __device__ inline bf16x8 fetch_rows(const char* tile, int t, int ks, int lane) {
-    int row = 32 * t + (lane & 31);
-    int chunk = 2 * ks + (lane >> 5);
-    return *(const bf16x8*)(tile + tile_offset<D>(row, chunk));
-}
-
-// A operand, transposing fetch: lane (m = lane%32, h = lane/32) gets column 32*db + m of
-// the 8 keys key_local = 32*h + 8*c + j, j = 0..7.  Each ds_read_b64_tr_b16 makes 16
-// lanes read a [4 rows x 16 columns] block (lane s: row s/4, columns 4*(s%4)..+3) and
-// hands lane s column s of it.
-template <int D> __device__ inline bf16x8 fetch_cols(const char* tile, int db, int c, int lane) {
-    const int h = lane >> 5, G1 = (lane >> 4) & 1, s = lane & 15;
-    const int chunk = 4 * db + 2 * G1 + ((s & 3) >> 1);
-    const int sub = (s & 1) << 3;
-    union { s16x4 v[2]; bf16x8 b; } u;
-#pragma unroll
-    for (int a = 0; a < 2; ++a) {
-        int row = 32 * (c >> 1) + 8 * (2 * (c & 1) + a) + 4 * h + (s >> 2);
-        const char* p = tile + tile_offset<D>(row, chunk) + sub;
-        u.v[a] = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-            (__attribute__((address_space(3))) s16x4*)(uintptr_t)(uint32_t)(uintptr_t)p);
-    }
-    return u.b;
-}
 
 // Epilogue of the key-owner kernels.  An accumulator tile (lane (n, h), register r -> row
 // 8*(r/4) + 4*h + r%4, column n) written straight to global memory is 16 two-byte stores per
@@ -318,17 +292,6 @@ __device__ inline f32x16 mfma(bf16x8 a, bf16x8 b, f32x16 c) {
 // them here, so the matrix cores run ahead of whatever vector work follows):
 // raw[t][r] = (K Q^T)[key_local = 32h + 16t + r][query n].
 template <int D>
-__device__ inline void score_raw(f32x16 (&raw)[2], const char* ktile, const bf16x8 (&qf)[D / 16], int lane) {
-#pragma unroll
-    for (int t = 0; t < 2; ++t) {
-        f32x16 acc = {0};
-#pragma unroll
-        for (int ks = 0; ks < D / 16; ++ks) acc = mfma(fetch_rows<D>(ktile, t, ks, lane), qf[ks], acc);
-        raw[t] = acc;
-    }
-}
-
-template <int D>
 __device__ inline void score_raw_o(f32x16 (&raw)[2], const char* ktile, const LaneOffsets<D>& o,
                                    const bf16x8 (&qf)[D / 16]) {
 #pragma unroll
@@ -346,14 +309,6 @@ __device__ inline void scale_scores(float (&x)[32], const f32x16 (&raw)[2], floa
     for (int t = 0; t < 2; ++t)
 #pragma unroll
         for (int r = 0; r < 16; ++r) x[16 * t + r] = raw[t][r] * scale2;
-}
-
-template <int D>
-__device__ inline void score_tiles(float (&x)[32], const char* ktile, const bf16x8 (&qf)[D / 16],
-                                   float scale2, int lane) {
-    f32x16 raw[2];
-    score_raw<D>(raw, ktile, qf, lane);
-    scale_scores(x, raw, scale2);
 }
 
 template <int D>
@@ -442,45 +397,12 @@ __device__ inline void mask_step(float (&x)[32], int key_first, int qi, int stri
         if (idx >= nvis) x[idx] = -INFINITY;
 }
 
-// Transposing fetch from a tile whose rows are in NATURAL order (Q, dO, and the weight
-// tiles of the key-owner pass): lane (m = lane%32, h = lane/32) gets column 32*cb + m of
-// rows row0 + 8*h + j, j = 0..7.  ROWD is the row length in bf16 (selects the swizzle).
-template <int ROWD> __device__ inline bf16x8 fetch_cols_nat(const char* tile, int row0, int cb, int lane) {
-    const int h = lane >> 5, G1 = (lane >> 4) & 1, s = lane & 15;
-    const int chunk = 4 * cb + 2 * G1 + ((s & 3) >> 1);
-    const int sub = (s & 1) << 3;
-    union { s16x4 v[2]; bf16x8 b; } u;
-#pragma unroll
-    for (int a = 0; a < 2; ++a) {
-        int row = row0 + 8 * h + 4 * a + (s >> 2);
-        const char* p = tile + tile_offset<ROWD>(row, chunk) + sub;
-        u.v[a] = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-            (__attribute__((address_space(3))) s16x4*)(uintptr_t)(uint32_t)(uintptr_t)p);
-    }
-    return u.b;
-}
-
 // Row fetch from a natural-order tile: 8 bf16 of row `row`, columns 16*ks + 8*h .. +7.
 template <int ROWD> __device__ inline bf16x8 fetch_row_nat(const char* tile, int row, int ks, int lane) {
     return *(const bf16x8*)(tile + tile_offset<ROWD>(row, 2 * ks + (lane >> 5)));
 }
 
 // dP^T tile pair: dp[16*t + r] = (V dO^T)[key_local][query] - drem[query].
-template <int D>
-__device__ inline void dp_tiles(float (&dp)[32], const char* vtile, const bf16x8 (&dof)[D / 16], float dr,
-                                int lane) {
-#pragma unroll
-    for (int t = 0; t < 2; ++t) {
-        f32x16 acc;
-#pragma unroll
-        for (int r = 0; r < 16; ++r) acc[r] = -dr;
-#pragma unroll
-        for (int ks = 0; ks < D / 16; ++ks) acc = mfma(fetch_rows<D>(vtile, t, ks, lane), dof[ks], acc);
-#pragma unroll
-        for (int r = 0; r < 16; ++r) dp[16 * t + r] = acc[r];
-    }
-}
-
 template <int D>
 __device__ inline void dp_tiles_o(float (&dp)[32], const char* vtile, const LaneOffsets<D>& o,
                                   const bf16x8 (&dof)[D / 16], float dr) {
