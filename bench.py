@@ -21,7 +21,7 @@ BF16_MFMA_PEAK_TFLOPS = 2516.6     # 256 CU x 2.4 GHz x 4096 FLOP/clk/CU (dense 
 # HBM bytes per launch (read + write) from the rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of the
 # cfg2 workload summarised in profiles/sba_cfg2_hbm_traffic.txt (counters cannot be read from
 # inside this process); other workloads report null.
-PROFILED_HBM_BYTES = {("cfg2", "fwd"): 42346590, ("cfg2", "bwd_dq"): 62739922, ("cfg2", "bwd_dkv"): 68240867}
+PROFILED_HBM_BYTES = {("cfg2", "fwd"): 42345120, ("cfg2", "bwd_dq"): 62807124, ("cfg2", "bwd_dkv"): 68223399}
 
 
 def _lognormal_lengths(total, seed, median=600.0, sigma=1.0, lo=16, hi=4096):
