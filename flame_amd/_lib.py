@@ -114,6 +114,25 @@ def usable(t: torch.Tensor) -> torch.Tensor:
     return t if ok else t.contiguous()
 
 
+def matrix_core_head_dim(t: torch.Tensor) -> int:
+    """Head dim that a bf16 problem runs with: the matrix-core kernels exist for 64 and 128, and any
+    other head dim up to 128 rides them zero-padded (zero columns add nothing to q.k and give zero
+    output columns), which is far faster than the generic kernels.  fp32 keeps its own head dim
+    (generic kernels, the tight-tolerance path), and so does everything under SBA_FORCE_GENERIC=1."""
+    D = t.shape[-1]
+    if t.dtype != torch.bfloat16 or D in (64, 128) or D > 128 or os.environ.get("SBA_FORCE_GENERIC") == "1":
+        return D
+    return 64 if D < 64 else 128
+
+
+def pad_head_dim(t: torch.Tensor, D: int) -> torch.Tensor:
+    return t if t.shape[-1] == D else torch.nn.functional.pad(t, (0, D - t.shape[-1]))
+
+
+def cut_head_dim(t: torch.Tensor, D: int) -> torch.Tensor:
+    return t if t.shape[-1] == D else t[..., :D].contiguous()
+
+
 SCHEDULE_INTS = 8      # int32 per row: {first_token, doc_len, row_block, doc_index} of job i, then of the i-th job in key-owner order
 
 

@@ -98,24 +98,26 @@ class StickBreakingAttention(torch.autograd.Function):
         if not (q.shape == k.shape == v.shape) or q.dim() != 4:
             raise ValueError("q, k, v must all be [B, H, T, D]")
         no_grad = not any(ctx.needs_input_grad[:3])
-        q, k, v = _lib.usable(q), _lib.usable(k), _lib.usable(v)
+        ctx.head_dim = q.shape[-1]
+        Dp = _lib.matrix_core_head_dim(q)
+        q, k, v = (_lib.usable(_lib.pad_head_dim(x, Dp)) for x in (q, k, v))
         o, rem, ws = _fwd(q, k, v, inv_temp, attend_current, no_grad)
         ctx.save_for_backward(q, k, v, ws)
         ctx.logit_scale = inv_temp
         ctx.attend_current = attend_current
         ctx.set_materialize_grads(False)
-        return o, rem
+        return _lib.cut_head_dim(o, ctx.head_dim), rem
 
     @staticmethod
     def backward(ctx, do, drem):
         q, k, v, ws = ctx.saved_tensors
         if do is None:
             do = torch.zeros_like(q)
-        do = _lib.usable(do)
+        do = _lib.usable(_lib.pad_head_dim(do, q.shape[-1]))
         if drem is not None:
             drem = drem.contiguous()
         dq, dk, dv = _bwd(do, drem, q, k, v, ws, ctx.logit_scale, ctx.attend_current)
-        return dq, dk, dv, None, None
+        return (*(_lib.cut_head_dim(g, ctx.head_dim) for g in (dq, dk, dv)), None, None)
 
 
 def sb_attn(q, k, v, inv_temp=None, zero_start=True, attend_current=False):

@@ -68,9 +68,17 @@ def test_bf16_unit_variance_inputs_and_custom_temperature():
     _check_dense(1, 4, 384, 64, torch.bfloat16, seed=5, in_scale=1.0, inv_temp=0.2)
 
 
-def test_bf16_other_head_dim_takes_generic_kernels():
+def test_bf16_other_head_dims_ride_the_matrix_core_kernels_zero_padded(monkeypatch):
+    # padded to 64 / 128 on the host side; the padding is invisible in shapes and results
     _check_dense(1, 2, 150, 32, torch.bfloat16, seed=11, in_scale=0.5)
     _check_dense(1, 2, 150, 80, torch.bfloat16, seed=12, in_scale=0.5)
+    _check_dense(2, 3, 300, 96, torch.bfloat16, attend_current=True, seed=14, in_scale=0.5)
+    _check_varlen(3, 48, [70, 1, 200, 129], torch.bfloat16, seed=15)
+    _check_varlen(2, 112, [300, 45], torch.bfloat16, attend_current=True, seed=16)
+    # and the generic kernels at those head dims stay reachable
+    monkeypatch.setenv("SBA_FORCE_GENERIC", "1")
+    _check_dense(1, 2, 150, 80, torch.bfloat16, seed=12, in_scale=0.5)
+    _check_varlen(3, 48, [70, 1, 200, 129], torch.bfloat16, seed=15)
 
 
 def test_bf16_no_drem_and_no_grad():
