@@ -8,10 +8,12 @@
 //           the forward's carry table, forms dz, accumulates dQ in registers, and records
 //           for every (query, key block) the prefix  sum_{j left of the block} g_ij  in a
 //           second table.
-//   pass 2  (key owner): a workgroup owns one 64-key block, sweeps the query blocks at or
-//           below the diagonal, recomputes weights and dz of its tile from the two tables,
-//           transposes them through LDS and accumulates dK = dZ^T Q and dV = P^T dO in
-//           registers.
+//   pass 2  (key owner): the owner of a block of keys sweeps the query blocks at or below the
+//           diagonal, recomputes weights and dz of its tiles from the tables, transposes them
+//           through LDS and accumulates dK = dZ^T Q and dV = P^T dO in registers.  Three
+//           kernels, chosen by grid size and head_dim: every wave owning 32 keys outright
+//           (large grids), a resident producer/consumer stream over 64-key items (d = 64,
+//           small grids), one workgroup per 64-key block (d = 128, small grids).
 //
 // Every element of the score matrix is therefore evaluated twice in the backward (once per
 // pass); in exchange nothing is reduced through memory.
