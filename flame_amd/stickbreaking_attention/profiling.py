@@ -4,6 +4,11 @@ A benchmark installs a ``KernelTimer``; the launch helpers then record an event 
 launch stream before and after every kernel (the backward is issued as its two kernels,
 one C call each, via SbaParams.bwd_phases).  With no timer installed -- the normal
 case -- nothing is recorded and the backward is a single C call.
+
+Every event record is a marker packet in the GPU queue that the neighbouring kernels wait
+for (several microseconds each, five per forward + backward), so a timer can sample:
+``KernelTimer(every=5)`` with ``next_step()`` called once per step instruments every fifth
+step and leaves the others untouched.
 """
 from __future__ import annotations
 
@@ -21,9 +26,16 @@ _TIMER: Optional["KernelTimer"] = None
 class KernelTimer:
     """Collects (name, start_event, end_event) triples; durations after a synchronize."""
 
-    def __init__(self):
+    def __init__(self, every: int = 1):
         self._last = None
         self._spans = []
+        self.every = max(1, int(every))
+        self._step = -1
+        self.active = True               # until next_step() is first called: every launch
+
+    def next_step(self):
+        self._step += 1
+        self.active = self._step % self.every == 0
 
     def mark(self, name: str):
         ev = torch.cuda.Event(enable_timing=True)
@@ -44,13 +56,17 @@ def install(timer: Optional[KernelTimer]):
     _TIMER = timer
 
 
+def _on() -> bool:
+    return _TIMER is not None and _TIMER.active
+
+
 def mark(name: str):
-    if _TIMER is not None:
+    if _on():
         _TIMER.mark(name)
 
 
 def launch_bwd(lib, p):
-    if _TIMER is None:
+    if not _on():
         _lib.check(lib.sba_bwd(C.byref(p)), "sba_bwd")
         return
     mark("start")
