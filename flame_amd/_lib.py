@@ -15,7 +15,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "csrc", "libsba_mi355x.so")
 
 SBA_DTYPE_F32, SBA_DTYPE_BF16 = 0, 1
-SBA_ABI_VERSION = 3
+SBA_ABI_VERSION = 4
 
 
 class SbaTensor(C.Structure):
@@ -37,7 +37,8 @@ class SbaParams(C.Structure):
         ("q", SbaTensor), ("k", SbaTensor), ("v", SbaTensor), ("o", SbaTensor),
         ("rem", SbaVector), ("d_o", SbaTensor), ("d_rem", SbaVector),
         ("dq", SbaTensor), ("dk", SbaTensor), ("dv", SbaTensor),
-        ("workspace", C.c_void_p), ("workspace_bytes", C.c_size_t), ("stream", C.c_void_p),
+        ("workspace", C.c_void_p), ("workspace_bytes", C.c_size_t),
+        ("bwd_scratch", C.c_void_p), ("bwd_scratch_bytes", C.c_size_t), ("stream", C.c_void_p),
     ]
 
 
@@ -63,6 +64,8 @@ def load() -> C.CDLL:
         lib.sba_error_string.argtypes = [C.c_int]
         lib.sba_workspace_bytes.restype = C.c_size_t
         lib.sba_workspace_bytes.argtypes = [C.POINTER(SbaParams)]
+        lib.sba_bwd_scratch_bytes.restype = C.c_size_t
+        lib.sba_bwd_scratch_bytes.argtypes = [C.POINTER(SbaParams)]
         lib.sba_build_schedule.restype = C.c_int
         lib.sba_build_schedule.argtypes = [C.POINTER(C.c_int32), C.c_int, C.POINTER(C.c_int32), C.c_int]
         lib.sba_row_block.restype = C.c_int
@@ -76,7 +79,7 @@ def load() -> C.CDLL:
     return _lib
 
 
-EXPORTED_SYMBOLS = ("sba_abi_version", "sba_error_string", "sba_workspace_bytes",
+EXPORTED_SYMBOLS = ("sba_abi_version", "sba_error_string", "sba_workspace_bytes", "sba_bwd_scratch_bytes",
                     "sba_build_schedule", "sba_row_block", "sba_fwd", "sba_bwd")
 
 
@@ -150,11 +153,17 @@ def build_schedule(cu_host: torch.Tensor) -> torch.Tensor:
 
 
 def workspace_upper_bound(n_heads: int, seq_len: int, tab_tokens: int, head_dim: int) -> int:
-    """Pure-Python bound on sba_workspace_bytes() (the four carry tables plus the generic
-    path's fp32 accumulators), usable while torch.compile traces, where no ctypes call can
-    be made.  Always >= what the library asks for."""
-    def up(x):
-        return (x + 255) & ~255
-    n_kb = (seq_len + 63) // 64
+    """Pure-Python bounds on sba_workspace_bytes() (one carry table) and sba_bwd_scratch_bytes()
+    (three more tables, or the generic path's fp32 accumulators), usable while torch.compile
+    traces, where no ctypes call can be made.  Always >= what the library asks for."""
+    return _table_bound(n_heads, seq_len, tab_tokens)
+
+
+def bwd_scratch_upper_bound(n_heads: int, seq_len: int, tab_tokens: int, head_dim: int) -> int:
     dp = 32 if head_dim <= 32 else (64 if head_dim <= 64 else 128)
-    return 4 * up(n_heads * n_kb * tab_tokens * 4) + up(2 * tab_tokens * n_heads * dp * 4)
+    acc = (2 * tab_tokens * n_heads * dp * 4 + 255) & ~255
+    return max(3 * _table_bound(n_heads, seq_len, tab_tokens), acc)
+
+
+def _table_bound(n_heads: int, seq_len: int, tab_tokens: int) -> int:
+    return (n_heads * ((seq_len + 63) // 64) * tab_tokens * 4 + 255) & ~255

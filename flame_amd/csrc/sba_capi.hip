@@ -84,15 +84,15 @@ KParams make_kparams(const SbaParams* p) {
     kp.rem = cvt(p->rem); kp.d_rem = cvt(p->d_rem);
     kp.n_kb = n_key_blocks(p);
     kp.tab_tokens = tab_tokens(p);
-    char* ws = (char*)p->workspace;
-    if (ws && use_mfma(p)) {
-        kp.rtab = (float*)ws;
-        kp.gtab = (float*)(ws + table_bytes(p));
-        kp.rmid = (float*)(ws + 2 * table_bytes(p));
-        kp.gmid = (float*)(ws + 3 * table_bytes(p));
-        ws += 4 * table_bytes(p);
+    if (p->workspace && use_mfma(p)) kp.rtab = (float*)p->workspace;
+    char* scratch = (char*)p->bwd_scratch;
+    if (scratch && use_mfma_bwd(p)) {
+        kp.gtab = (float*)scratch;
+        kp.rmid = (float*)(scratch + table_bytes(p));
+        kp.gmid = (float*)(scratch + 2 * table_bytes(p));
+    } else if (scratch) {
+        kp.dkv32 = (float*)scratch;
     }
-    if (ws && !use_mfma_bwd(p)) kp.dkv32 = (float*)ws;
     return kp;
 }
 
@@ -108,7 +108,7 @@ const char* sba_error_string(int code) {
         case SBA_ERR_NULL: return "a required pointer is NULL";
         case SBA_ERR_SHAPE: return "bad shape: sizes must be positive, head_dim <= 128, dense total_tokens == seq_len";
         case SBA_ERR_DTYPE: return "unsupported dtype (float32 and bfloat16 only)";
-        case SBA_ERR_WORKSPACE: return "workspace missing or smaller than sba_workspace_bytes()";
+        case SBA_ERR_WORKSPACE: return "workspace / bwd_scratch missing or smaller than sba_workspace_bytes() / sba_bwd_scratch_bytes()";
         case SBA_ERR_SCHEDULE: return "packed layout needs a row-block schedule from sba_build_schedule()";
         case SBA_ERR_LAUNCH: return "kernel launch failed";
         case SBA_ERR_ABI: return "SbaParams.struct_size does not match this library";
@@ -118,10 +118,12 @@ const char* sba_error_string(int code) {
 
 size_t sba_workspace_bytes(const SbaParams* p) {
     if (!p || p->n_heads <= 0 || p->seq_len <= 0 || p->head_dim <= 0 || p->head_dim > 128) return 0;
-    size_t b = 0;
-    if (use_mfma(p)) b += 4 * table_bytes(p);
-    if (!use_mfma_bwd(p)) b += generic_acc_bytes(p);
-    return b;
+    return use_mfma(p) ? table_bytes(p) : 0;
+}
+
+size_t sba_bwd_scratch_bytes(const SbaParams* p) {
+    if (!p || p->n_heads <= 0 || p->seq_len <= 0 || p->head_dim <= 0 || p->head_dim > 128) return 0;
+    return use_mfma_bwd(p) ? 3 * table_bytes(p) : generic_acc_bytes(p);
 }
 
 int sba_row_block(void) { return sba::kRowBlock; }
@@ -174,7 +176,8 @@ int sba_bwd(const SbaParams* p) {
     if (rc) return rc;
     if (!p->d_o.ptr || !p->dq.ptr || !p->dk.ptr || !p->dv.ptr) return SBA_ERR_NULL;
     if (p->bwd_phases < 0 || p->bwd_phases > 2) return SBA_ERR_SHAPE;
-    if (!p->workspace || p->workspace_bytes < sba_workspace_bytes(p)) return SBA_ERR_WORKSPACE;
+    if (use_mfma_bwd(p) && (!p->workspace || p->workspace_bytes < sba_workspace_bytes(p))) return SBA_ERR_WORKSPACE;
+    if (!p->bwd_scratch || p->bwd_scratch_bytes < sba_bwd_scratch_bytes(p)) return SBA_ERR_WORKSPACE;
     KParams kp = make_kparams(p);
     hipStream_t s = (hipStream_t)p->stream;
     // the generic backward is one piece: it all runs in phase 1

@@ -32,10 +32,19 @@ def _params(q, k, v, inv_temp, attend_current):
 
 
 def workspace_bytes(q, inv_temp=1.0) -> int:
+    """What lives from the forward to the backward (the forward's carry table)."""
     if torch.compiler.is_compiling():
         B, H, T, D = q.shape
         return _lib.workspace_upper_bound(H, T, B * T, D)
     return int(_lib.load().sba_workspace_bytes(C.byref(_params(q, q, q, inv_temp, False))))
+
+
+def bwd_scratch_bytes(q, inv_temp=1.0) -> int:
+    """What the backward needs for the duration of its call only."""
+    if torch.compiler.is_compiling():
+        B, H, T, D = q.shape
+        return _lib.bwd_scratch_upper_bound(H, T, B * T, D)
+    return int(_lib.load().sba_bwd_scratch_bytes(C.byref(_params(q, q, q, inv_temp, False))))
 
 
 # Same registered names as the reference (sb_fwd.py:177, sb_bwd.py:207); outputs are
@@ -56,10 +65,10 @@ def _compileable_fwd(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, logit_sc
     profiling.mark("fwd")
 
 
-@custom_op("attn_bwd", mutates_args=("dq", "dk", "dv", "ws"))
+@custom_op("attn_bwd", mutates_args=("dq", "dk", "dv", "scratch"))
 def _compileable_backward(do: torch.Tensor, dr: Optional[torch.Tensor], q: torch.Tensor, k: torch.Tensor,
-                          v: torch.Tensor, ws: torch.Tensor, logit_scale: float, attend_current: bool,
-                          dq: torch.Tensor, dk: torch.Tensor, dv: torch.Tensor) -> None:
+                          v: torch.Tensor, ws: torch.Tensor, scratch: torch.Tensor, logit_scale: float,
+                          attend_current: bool, dq: torch.Tensor, dk: torch.Tensor, dv: torch.Tensor) -> None:
     lib = _lib.load()
     p = _params(q, k, v, logit_scale, attend_current)
     p.d_o = _lib.tensor4(do)
@@ -67,6 +76,7 @@ def _compileable_backward(do: torch.Tensor, dr: Optional[torch.Tensor], q: torch
         p.d_rem = _lib.SbaVector(dr.data_ptr(), dr.stride(0), dr.stride(1))
     p.dq, p.dk, p.dv = _lib.tensor4(dq), _lib.tensor4(dk), _lib.tensor4(dv)
     p.workspace, p.workspace_bytes = ws.data_ptr(), ws.numel()
+    p.bwd_scratch, p.bwd_scratch_bytes = scratch.data_ptr(), scratch.numel()
     profiling.launch_bwd(lib, p)
 
 
@@ -81,7 +91,9 @@ def _fwd(q, k, v, logit_scale, attend_current=False, no_grad=False):
 
 def _bwd(do, dr, q, k, v, ws, logit_scale, attend_current=False):
     dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
-    _compileable_backward(do, dr, q, k, v, ws, float(logit_scale), bool(attend_current), dq, dk, dv)
+    # freed when this call returns: only the forward's table is kept between the two directions
+    scratch = torch.empty(max(bwd_scratch_bytes(q), 16), dtype=torch.uint8, device=q.device)
+    _compileable_backward(do, dr, q, k, v, ws, scratch, float(logit_scale), bool(attend_current), dq, dk, dv)
     return dq, dk, dv
 
 

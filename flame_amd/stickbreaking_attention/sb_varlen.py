@@ -69,12 +69,23 @@ def _bind_schedule(p, q, cu_seqlens, max_seqlens):
 
 
 def workspace_bytes(q, max_seqlens: int) -> int:
+    """What lives from the forward to the backward (the forward's carry table)."""
     if torch.compiler.is_compiling():
         H, N, D = q.shape
         return _lib.workspace_upper_bound(H, max_seqlens, N, D)
     p = _params(q, q, q, 1, max_seqlens, 1.0, False)
     p.cu_seqlens = 1          # only "packed or not" matters for the size
     return int(_lib.load().sba_workspace_bytes(C.byref(p)))
+
+
+def bwd_scratch_bytes(q, max_seqlens: int) -> int:
+    """What the backward needs for the duration of its call only."""
+    if torch.compiler.is_compiling():
+        H, N, D = q.shape
+        return _lib.bwd_scratch_upper_bound(H, max_seqlens, N, D)
+    p = _params(q, q, q, 1, max_seqlens, 1.0, False)
+    p.cu_seqlens = 1
+    return int(_lib.load().sba_bwd_scratch_bytes(C.byref(p)))
 
 
 # Registered names as in the reference (sb_varlen_fwd.py:449, sb_varlen_bwd.py:523).
@@ -96,11 +107,11 @@ def _compileable_forward(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, cu_s
     profiling.mark("fwd")
 
 
-@custom_op("varlen_bwd", mutates_args=("dq", "dk", "dv", "ws"))
+@custom_op("varlen_bwd", mutates_args=("dq", "dk", "dv", "scratch"))
 def _compileable_backward(do: torch.Tensor, dr: Optional[torch.Tensor], q: torch.Tensor, k: torch.Tensor,
                           v: torch.Tensor, cu_seqlens: torch.Tensor, max_seqlens: int, ws: torch.Tensor,
-                          logit_scale: float, attend_current: bool, dq: torch.Tensor, dk: torch.Tensor,
-                          dv: torch.Tensor) -> None:
+                          scratch: torch.Tensor, logit_scale: float, attend_current: bool, dq: torch.Tensor,
+                          dk: torch.Tensor, dv: torch.Tensor) -> None:
     lib = _lib.load()
     p = _params(q, k, v, cu_seqlens.numel() - 1, max_seqlens, logit_scale, attend_current)
     if _bind_schedule(p, q, cu_seqlens, max_seqlens) == 0:
@@ -110,6 +121,7 @@ def _compileable_backward(do: torch.Tensor, dr: Optional[torch.Tensor], q: torch
         p.d_rem = _lib.SbaVector(dr.data_ptr(), 0, dr.stride(0))
     p.dq, p.dk, p.dv = _lib.tensor3(dq), _lib.tensor3(dk), _lib.tensor3(dv)
     p.workspace, p.workspace_bytes = ws.data_ptr(), ws.numel()
+    p.bwd_scratch, p.bwd_scratch_bytes = scratch.data_ptr(), scratch.numel()
     profiling.launch_bwd(lib, p)
 
 
@@ -125,7 +137,9 @@ def varlen_fwd(q, k, v, cu_seqlens, max_seqlens, logit_scale, attend_current=Fal
 
 def varlen_bwd(do, dr, q, k, v, cu_seqlens, max_seqlens, ws, logit_scale, attend_current=False):
     dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
-    _compileable_backward(do, dr, q, k, v, cu_seqlens, int(max_seqlens), ws, float(logit_scale),
+    # freed when this call returns: only the forward's table is kept between the two directions
+    scratch = torch.empty(max(bwd_scratch_bytes(q, max_seqlens), 16), dtype=torch.uint8, device=q.device)
+    _compileable_backward(do, dr, q, k, v, cu_seqlens, int(max_seqlens), ws, scratch, float(logit_scale),
                           bool(attend_current), dq, dk, dv)
     return dq, dk, dv
 

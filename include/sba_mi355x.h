@@ -34,7 +34,7 @@
 extern "C" {
 #endif
 
-#define SBA_ABI_VERSION 3
+#define SBA_ABI_VERSION 4
 #define SBA_SCHEDULE_INTS 8   /* int32 per scheduled job, see sba_build_schedule() */
 
 enum { SBA_DTYPE_F32 = 0, SBA_DTYPE_BF16 = 1 };
@@ -44,7 +44,7 @@ enum {
     SBA_ERR_NULL = -1,        /* a required pointer is NULL */
     SBA_ERR_SHAPE = -2,       /* non-positive size, head_dim unsupported, bad strides */
     SBA_ERR_DTYPE = -3,       /* unknown dtype */
-    SBA_ERR_WORKSPACE = -4,   /* workspace missing or too small */
+    SBA_ERR_WORKSPACE = -4,   /* workspace or bwd_scratch missing or too small */
     SBA_ERR_SCHEDULE = -5,    /* packed layout without a row-block schedule */
     SBA_ERR_LAUNCH = -6,      /* hipGetLastError() after a launch was not hipSuccess */
     SBA_ERR_ABI = -7          /* struct_size does not match this library */
@@ -91,8 +91,10 @@ typedef struct SbaParams {
     SbaVector d_rem;           /* backward input  (grad of rem); ptr may be NULL = zeros */
     SbaTensor dq, dk, dv;      /* backward outputs */
 
-    void*    workspace;        /* device scratch, see sba_workspace_bytes() */
+    void*    workspace;        /* device memory that lives from sba_fwd to sba_bwd, see sba_workspace_bytes() */
     size_t   workspace_bytes;
+    void*    bwd_scratch;      /* backward only: device memory for the call, see sba_bwd_scratch_bytes() */
+    size_t   bwd_scratch_bytes;
     void*    stream;           /* hipStream_t */
 } SbaParams;
 
@@ -103,14 +105,21 @@ int sba_abi_version(void);
 const char* sba_error_string(int code);
 
 /*
- * Bytes of device workspace the pair (sba_fwd with save_for_backward, sba_bwd) needs for
+ * Bytes of device workspace the pair (sba_fwd with save_for_backward, sba_bwd) shares for
  * this problem.  The forward writes its per-key-block carry table there and the backward
- * reads it back (and keeps three more tables of the same size there between its two
- * kernels), so the SAME buffer, untouched in between, must be given to both calls
+ * reads it back, so the SAME buffer, untouched in between, must be given to both calls
  * (the Python layer keeps it in the autograd context the way the reference keeps
  * neg_log_acc, sb_attn/__init__.py:30).  Only the size fields of `p` are read.
  */
 size_t sba_workspace_bytes(const SbaParams* p);
+
+/*
+ * Bytes of device memory sba_bwd needs for the duration of the call only (three more
+ * tables between its two kernels, or the generic path's fp32 accumulators): allocate before
+ * the call, free after it has run.  With bwd_phases 1 and 2 issued as two calls, the same
+ * buffer goes to both.
+ */
+size_t sba_bwd_scratch_bytes(const SbaParams* p);
 
 /*
  * Row-block schedule for the packed layout, built on the host from host cu_seqlens

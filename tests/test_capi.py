@@ -30,7 +30,7 @@ def test_exports_every_declared_symbol(lib):
 
 
 def test_abi_version_and_struct_size(lib):
-    assert lib.sba_abi_version() == 3
+    assert lib.sba_abi_version() == 4
     p = _lib.SbaParams()
     p.struct_size = C.sizeof(_lib.SbaParams) - 8
     assert lib.sba_fwd(C.byref(p)) == -7          # SBA_ERR_ABI, before anything touches a GPU
@@ -57,10 +57,12 @@ def test_workspace_bytes(lib):
     p.struct_size = C.sizeof(_lib.SbaParams)
     p.dtype = _lib.SBA_DTYPE_BF16
     p.n_seq, p.n_heads, p.seq_len, p.total_tokens, p.head_dim = 1, 16, 4096, 4096, 64
-    n = lib.sba_workspace_bytes(C.byref(p))
-    assert n >= 2 * 16 * 64 * 4096 * 4            # two carry tables [H][T/64][T] fp32
-    p.dtype = _lib.SBA_DTYPE_F32
-    assert lib.sba_workspace_bytes(C.byref(p)) == 2 * 4096 * 16 * 64 * 4
+    table = 16 * 64 * 4096 * 4                      # one carry table [H][T/64][T] fp32
+    assert lib.sba_workspace_bytes(C.byref(p)) == table          # what the forward hands to the backward
+    assert lib.sba_bwd_scratch_bytes(C.byref(p)) == 3 * table    # what the backward needs for itself
+    p.dtype = _lib.SBA_DTYPE_F32                    # generic kernels: nothing kept, fp32 dk|dv accumulators
+    assert lib.sba_workspace_bytes(C.byref(p)) == 0
+    assert lib.sba_bwd_scratch_bytes(C.byref(p)) == 2 * 4096 * 16 * 64 * 4
 
 
 def test_schedule_builder(lib):
@@ -100,3 +102,4 @@ def test_python_workspace_bound_covers_the_library(lib):
             p.dtype = dtype
             p.n_seq, p.n_heads, p.seq_len, p.total_tokens, p.head_dim = B, H, T, T, D
             assert _lib.workspace_upper_bound(H, T, B * T, D) >= lib.sba_workspace_bytes(C.byref(p))
+            assert _lib.bwd_scratch_upper_bound(H, T, B * T, D) >= lib.sba_bwd_scratch_bytes(C.byref(p))
