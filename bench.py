@@ -18,10 +18,10 @@ if ROOT not in sys.path:
 
 BF16_MFMA_PEAK_TFLOPS = 2516.6     # 256 CU x 2.4 GHz x 4096 FLOP/clk/CU (dense bf16)
 
+KERNEL_TIMING_SAMPLES = 5      # steps of the timed region whose kernels are timed with events
 # HBM bytes per launch (read + write) from the rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs
 # summarised in profiles/sba_cfg{2,3,4}_hbm_traffic.txt (counters cannot be read from inside this
 # process).
-KERNEL_TIMING_SAMPLES = 5      # steps of the timed region whose kernels are timed with events
 PROFILED_HBM_BYTES = {("cfg2", "fwd"): 42341848, ("cfg2", "bwd_dq"): 62815891, ("cfg2", "bwd_dkv"): 68231451,
                       ("cfg3", "fwd"): 2078049827, ("cfg3", "bwd_dq"): 2391520113, ("cfg3", "bwd_dkv"): 2279290798,
                       ("cfg4", "fwd"): 744411843, ("cfg4", "bwd_dq"): 1344925113, ("cfg4", "bwd_dkv"): 1396909288}
