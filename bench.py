@@ -23,7 +23,7 @@ KERNEL_TIMING_SAMPLES = 5      # steps of the timed region whose kernels are tim
 # summarised in profiles/sba_cfg{2,3,4}_hbm_traffic.txt (counters cannot be read from inside this
 # process).
 PROFILED_HBM_BYTES = {("cfg2", "fwd"): 42341848, ("cfg2", "bwd_dq"): 62815891, ("cfg2", "bwd_dkv"): 68231451,
-                      ("cfg3", "fwd"): 2078049827, ("cfg3", "bwd_dq"): 2391520113, ("cfg3", "bwd_dkv"): 2279290798,
+                      ("cfg3", "fwd"): 901280529, ("cfg3", "bwd_dq"): 984098943, ("cfg3", "bwd_dkv"): 1128992455,
                       ("cfg4", "fwd"): 744411843, ("cfg4", "bwd_dq"): 1344925113, ("cfg4", "bwd_dkv"): 1396909288}
 
 

@@ -67,7 +67,7 @@ def load() -> C.CDLL:
         lib.sba_bwd_scratch_bytes.restype = C.c_size_t
         lib.sba_bwd_scratch_bytes.argtypes = [C.POINTER(SbaParams)]
         lib.sba_build_schedule.restype = C.c_int
-        lib.sba_build_schedule.argtypes = [C.POINTER(C.c_int32), C.c_int, C.POINTER(C.c_int32), C.c_int]
+        lib.sba_build_schedule.argtypes = [C.POINTER(C.c_int32), C.c_int, C.c_int, C.POINTER(C.c_int32), C.c_int]
         lib.sba_row_block.restype = C.c_int
         lib.sba_fwd.restype = C.c_int
         lib.sba_fwd.argtypes = [C.POINTER(SbaParams)]
@@ -139,15 +139,19 @@ def cut_head_dim(t: torch.Tensor, D: int) -> torch.Tensor:
 SCHEDULE_INTS = 8      # int32 per row: {first_token, doc_len, row_block, doc_index} of job i, then of the i-th job in key-owner order
 
 
-def build_schedule(cu_host: torch.Tensor) -> torch.Tensor:
-    """Host int32 cu_seqlens (leading 0) -> host int32 [n_jobs, 8] schedule."""
+DOC_MAJOR_GRID = 8192  # workgroups (jobs x heads) from which the schedule is document-major
+
+
+def build_schedule(cu_host: torch.Tensor, n_heads: int = 0) -> torch.Tensor:
+    """Host int32 cu_seqlens (leading 0) -> host int32 [n_jobs, 8] schedule for launches with
+    `n_heads` heads (the job order depends on the launch size)."""
     lib = load()
     cu = cu_host.to(torch.int32).contiguous()
     n_seq = cu.numel() - 1
     ptr = C.cast(cu.data_ptr(), C.POINTER(C.c_int32))
-    n = lib.sba_build_schedule(ptr, n_seq, None, 0)
+    n = lib.sba_build_schedule(ptr, n_seq, n_heads, None, 0)
     out = torch.empty((max(n, 1), SCHEDULE_INTS), dtype=torch.int32)
-    got = lib.sba_build_schedule(ptr, n_seq, C.cast(out.data_ptr(), C.POINTER(C.c_int32)), n)
+    got = lib.sba_build_schedule(ptr, n_seq, n_heads, C.cast(out.data_ptr(), C.POINTER(C.c_int32)), n)
     assert got == n
     return out[:n]
 

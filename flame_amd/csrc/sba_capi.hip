@@ -128,7 +128,7 @@ size_t sba_bwd_scratch_bytes(const SbaParams* p) {
 
 int sba_row_block(void) { return sba::kRowBlock; }
 
-int sba_build_schedule(const int32_t* cu, int n_seq, int32_t* out, int capacity) {
+int sba_build_schedule(const int32_t* cu, int n_seq, int n_heads, int32_t* out, int capacity) {
     if (!cu || n_seq <= 0) return 0;
     struct J { int32_t tok0, len, rb, doc; };
     std::vector<J> jobs;
@@ -138,16 +138,29 @@ int sba_build_schedule(const int32_t* cu, int n_seq, int32_t* out, int capacity)
         int n_rb = (len + sba::kRowBlock - 1) / sba::kRowBlock;
         for (int rb = 0; rb < n_rb; ++rb) jobs.push_back(J{cu[s], len, rb, s});
     }
-    // longest sweeps first; a stable order keeps the schedule deterministic
-    std::stable_sort(jobs.begin(), jobs.end(), [](const J& a, const J& b) { return a.rb > b.rb; });
     int n = (int)jobs.size();
+    // Longest sweeps first; a stable order keeps the schedule deterministic.  Very large launches
+    // keep the jobs of a document together instead (longest document first, its longest sweeps
+    // first): with thousands of workgroups the balance takes care of itself, and the K/V of the
+    // documents in flight then fit the L2 of the XCD that runs them.
+    const bool doc_major = (int64_t)n * n_heads >= SBA_DOC_MAJOR_GRID;
+    if (doc_major)
+        std::stable_sort(jobs.begin(), jobs.end(), [](const J& a, const J& b) {
+            return a.len != b.len ? a.len > b.len : a.doc != b.doc ? a.doc < b.doc : a.rb > b.rb; });
+    else
+        std::stable_sort(jobs.begin(), jobs.end(), [](const J& a, const J& b) { return a.rb > b.rb; });
     if (out && capacity >= n) {
         // second half of row i: the job that comes i-th for the key-owner kernels, whose sweep
         // from a job's row-block to the end of its sequence is (blocks of the sequence - rb) long
         std::vector<int> key_order(n);
         for (int i = 0; i < n; ++i) key_order[i] = i;
         auto key_len = [&](int i) { return (jobs[i].len + sba::kRowBlock - 1) / sba::kRowBlock - jobs[i].rb; };
-        std::stable_sort(key_order.begin(), key_order.end(), [&](int a, int b) { return key_len(a) > key_len(b); });
+        if (doc_major)      // `jobs` is document-major already; the key owners want rb ascending inside a document
+            std::stable_sort(key_order.begin(), key_order.end(), [&](int a, int b) {
+                const J& x = jobs[a]; const J& y = jobs[b];
+                return x.len != y.len ? x.len > y.len : x.doc != y.doc ? x.doc < y.doc : x.rb < y.rb; });
+        else
+            std::stable_sort(key_order.begin(), key_order.end(), [&](int a, int b) { return key_len(a) > key_len(b); });
         for (int i = 0; i < n; ++i) {
             int32_t* o = out + (size_t)sba::kScheduleInts * i;
             const J& k = jobs[key_order[i]];

@@ -25,23 +25,26 @@ from .utils import custom_op
 _SCHEDULES: dict = {}
 
 
-def _schedule_for(cu_seqlens: torch.Tensor):
-    """(cu int32 on device with leading 0, schedule on device, n_jobs, max_len, total)."""
-    key = id(cu_seqlens)
-    hit = _SCHEDULES.get(key)
+def _schedule_for(cu_seqlens: torch.Tensor, n_heads: int):
+    """(cu int32 on device with leading 0, schedule on device, n_jobs, max_len, total).  The job
+    order depends on the launch size (jobs x heads): one entry per cu_seqlens tensor and order."""
+    hit = _SCHEDULES.get(id(cu_seqlens))
     if hit is not None and hit[0]() is cu_seqlens and hit[1] == cu_seqlens._version:
-        return hit[2]
+        entry = hit[2]
+        if (entry[2] * n_heads >= _lib.DOC_MAJOR_GRID) == hit[3]:
+            return entry
+    key = id(cu_seqlens)
     cu_host = cu_seqlens.detach().to("cpu", torch.int32)   # one host sync per new packing
     if cu_host.numel() < 2 or int(cu_host[0]) != 0:
         raise ValueError("cu_seqlens must start with 0 and hold at least one document")
     lens = cu_host[1:] - cu_host[:-1]
     if bool((lens < 0).any()):
         raise ValueError("cu_seqlens must be non-decreasing")
-    sched = _lib.build_schedule(cu_host)
+    sched = _lib.build_schedule(cu_host, n_heads)
     dev = cu_seqlens.device
     entry = (cu_host.to(dev), sched.to(dev), sched.shape[0], int(lens.max()), int(cu_host[-1]))
     ref = weakref.ref(cu_seqlens, lambda _r, key=key: _SCHEDULES.pop(key, None))
-    _SCHEDULES[key] = (ref, cu_seqlens._version, entry)
+    _SCHEDULES[key] = (ref, cu_seqlens._version, entry, sched.shape[0] * n_heads >= _lib.DOC_MAJOR_GRID)
     return entry
 
 
@@ -59,7 +62,7 @@ def _params(q, k, v, n_docs, max_seqlens, inv_temp, attend_current):
 
 
 def _bind_schedule(p, q, cu_seqlens, max_seqlens):
-    cu_dev, sched, n_jobs, max_len, total = _schedule_for(cu_seqlens)
+    cu_dev, sched, n_jobs, max_len, total = _schedule_for(cu_seqlens, q.shape[0])
     if total != q.shape[1]:
         raise ValueError(f"cu_seqlens ends at {total} but q has {q.shape[1]} tokens")
     if max_len > max_seqlens:

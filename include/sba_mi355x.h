@@ -36,6 +36,7 @@ extern "C" {
 
 #define SBA_ABI_VERSION 4
 #define SBA_SCHEDULE_INTS 8   /* int32 per scheduled job, see sba_build_schedule() */
+#define SBA_DOC_MAJOR_GRID 8192 /* workgroups from which the schedule is document-major */
 
 enum { SBA_DTYPE_F32 = 0, SBA_DTYPE_BF16 = 1 };
 
@@ -128,12 +129,16 @@ size_t sba_bwd_scratch_bytes(const SbaParams* p);
  * {first_token, doc_len, row_block, doc_index} of the i-th job, longest row-blocks first;
  * ints 4-7 are the same four of the job that comes i-th for the dK/dV kernel, whose sweeps
  * run from a row-block to the END of its document (or the number needed when
- * `out` is NULL or capacity is too small).  The caller copies it to the device and passes
- * it as SbaParams.schedule.  Replaces the reference's 3-D launch grid
+ * `out` is NULL or capacity is too small).  `n_heads` is the head count the schedule will be
+ * launched with (0 if unknown): from SBA_DOC_MAJOR_GRID workgroups (jobs x heads) on, the
+ * jobs of a document stay together, longest document first, so that its K and V stay in
+ * the L2 of one XCD (a third of the HBM reads); smaller launches need the strict
+ * longest-first order for their balance.  The caller copies the schedule to the device and
+ * passes it as SbaParams.schedule.  Replaces the reference's 3-D launch grid
  * (n_docs, ceil(H/2), ceil(max_len/64)+1) and its long/short head pairing
  * (sb_varlen_fwd.py:288-289, 472-475).
  */
-int sba_build_schedule(const int32_t* cu_seqlens_host, int n_seq, int32_t* out, int capacity);
+int sba_build_schedule(const int32_t* cu_seqlens_host, int n_seq, int n_heads, int32_t* out, int capacity);
 
 /* Rows of queries one scheduled job covers (the kernels' row-block height). */
 int sba_row_block(void);

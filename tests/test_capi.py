@@ -82,9 +82,20 @@ def test_schedule_builder(lib):
     assert key_len == sorted(key_len, reverse=True) and key_len[0] == 5
     # capacity too small: returns the count needed and writes nothing
     out = torch.full((2, 8), -1, dtype=torch.int32)
-    n = lib.sba_build_schedule(C.cast(cu.data_ptr(), C.POINTER(C.c_int32)), 5,
+    n = lib.sba_build_schedule(C.cast(cu.data_ptr(), C.POINTER(C.c_int32)), 5, 0,
                                C.cast(out.data_ptr(), C.POINTER(C.c_int32)), 2)
     assert n == len(expect) and bool((out == -1).all())
+    # a launch of SBA_DOC_MAJOR_GRID workgroups or more: same jobs, document-major (longest
+    # document first; row blocks descending for the row owners, ascending for the key owners)
+    heads = -(-_lib.DOC_MAJOR_GRID // len(jobs))
+    d = _lib.build_schedule(cu, heads)
+    assert sorted(tuple(r[:4]) for r in d.tolist()) == sorted(jobs)
+    assert sorted(tuple(r[4:8]) for r in d.tolist()) == sorted(jobs)
+    row_order = [(r[3], r[2]) for r in d.tolist()]
+    assert row_order == [(3, 4), (3, 3), (3, 2), (3, 1), (3, 0), (1, 2), (1, 1), (1, 0), (0, 0), (2, 0)]
+    key_order = [(r[7], r[6]) for r in d.tolist()]
+    assert key_order == [(3, 0), (3, 1), (3, 2), (3, 3), (3, 4), (1, 0), (1, 1), (1, 2), (0, 0), (2, 0)]
+    assert _lib.build_schedule(cu, heads - 1).tolist() == s.tolist()      # just below: the usual order
 
 
 def test_op_refuses_cpu_tensors():
