@@ -117,6 +117,13 @@ def usable(t: torch.Tensor) -> torch.Tensor:
     return t if ok else t.contiguous()
 
 
+def recompute_carries() -> bool:
+    """SBA_RECOMPUTE_CARRIES=1: keep nothing between forward and backward (the reference keeps one
+    float per query, the default here one carry table of H x T/64 x tokens floats); the backward
+    then repeats the forward's sweep for the carries alone, about 15 % more time per fwd + bwd."""
+    return os.environ.get("SBA_RECOMPUTE_CARRIES") == "1"
+
+
 def matrix_core_head_dim(t: torch.Tensor) -> int:
     """Head dim that a bf16 problem runs with: the matrix-core kernels exist for 64 and 128, and any
     other head dim up to 128 rides them zero-padded (zero columns add nothing to q.k and give zero
@@ -166,7 +173,7 @@ def workspace_upper_bound(n_heads: int, seq_len: int, tab_tokens: int, head_dim:
 def bwd_scratch_upper_bound(n_heads: int, seq_len: int, tab_tokens: int, head_dim: int) -> int:
     dp = 32 if head_dim <= 32 else (64 if head_dim <= 64 else 128)
     acc = (2 * tab_tokens * n_heads * dp * 4 + 255) & ~255
-    return max(3 * _table_bound(n_heads, seq_len, tab_tokens), acc)
+    return max(4 * _table_bound(n_heads, seq_len, tab_tokens), acc)     # four: also covers the recompute mode
 
 
 def _table_bound(n_heads: int, seq_len: int, tab_tokens: int) -> int:

@@ -90,6 +90,7 @@ KParams make_kparams(const SbaParams* p) {
         kp.gtab = (float*)scratch;
         kp.rmid = (float*)(scratch + table_bytes(p));
         kp.gmid = (float*)(scratch + 2 * table_bytes(p));
+        if (!p->workspace) kp.rtab = (float*)(scratch + 3 * table_bytes(p));   // recomputed by sba_bwd
     } else if (scratch) {
         kp.dkv32 = (float*)scratch;
     }
@@ -123,7 +124,8 @@ size_t sba_workspace_bytes(const SbaParams* p) {
 
 size_t sba_bwd_scratch_bytes(const SbaParams* p) {
     if (!p || p->n_heads <= 0 || p->seq_len <= 0 || p->head_dim <= 0 || p->head_dim > 128) return 0;
-    return use_mfma_bwd(p) ? 3 * table_bytes(p) : generic_acc_bytes(p);
+    // without a workspace the backward recomputes the forward's table first, into a fourth slot
+    return use_mfma_bwd(p) ? (p->workspace ? 3 : 4) * table_bytes(p) : generic_acc_bytes(p);
 }
 
 int sba_row_block(void) { return sba::kRowBlock; }
@@ -189,10 +191,18 @@ int sba_bwd(const SbaParams* p) {
     if (rc) return rc;
     if (!p->d_o.ptr || !p->dq.ptr || !p->dk.ptr || !p->dv.ptr) return SBA_ERR_NULL;
     if (p->bwd_phases < 0 || p->bwd_phases > 2) return SBA_ERR_SHAPE;
-    if (use_mfma_bwd(p) && (!p->workspace || p->workspace_bytes < sba_workspace_bytes(p))) return SBA_ERR_WORKSPACE;
+    if (use_mfma_bwd(p) && p->workspace && p->workspace_bytes < sba_workspace_bytes(p)) return SBA_ERR_WORKSPACE;
     if (!p->bwd_scratch || p->bwd_scratch_bytes < sba_bwd_scratch_bytes(p)) return SBA_ERR_WORKSPACE;
     KParams kp = make_kparams(p);
     hipStream_t s = (hipStream_t)p->stream;
+    if (use_mfma_bwd(p) && !p->workspace && p->bwd_phases != 2) {
+        // no table from the forward: run its sweep again for the carries alone (no P*V, no outputs)
+        KParams carry = kp;
+        carry.save = 1;
+        carry.carry_only = 1;
+        rc = sba_launch_mfma_fwd(carry, s);
+        if (rc) return rc;
+    }
     // the generic backward is one piece: it all runs in phase 1
     if (!use_mfma_bwd(p) && p->bwd_phases == 2) return SBA_OK;
     return use_mfma_bwd(p) ? sba_launch_mfma_bwd(kp, p->bwd_phases, s) : sba_launch_generic_bwd(kp, p->dtype, s);

@@ -21,6 +21,7 @@ struct VectorArg { char* ptr; int64_t sb, sh; };
 // Kernel-side copy of SbaParams (by value in the launch).
 struct KParams {
     int n_seq, n_heads, seq_len, total_tokens, head_dim, attend_current, save, n_jobs;
+    int carry_only;                // forward kernels: write the carry table and nothing else (no P*V, no o / rem)
     float scale2;                  // scale * log2(e): logits in base-2 units
     float scale;                   // natural-unit scale (for dq/dk)
     const int32_t* cu_seqlens;

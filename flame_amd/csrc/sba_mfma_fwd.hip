@@ -7,7 +7,9 @@
 
 namespace sba {
 
-template <int D>
+// kCarryOnly: write the carry table and nothing else (no P*V, no o / rem): the backward's way of
+// getting the table when the forward kept none.
+template <int D, bool kCarryOnly>
 __global__ __launch_bounds__(kThreads) void mfma_fwd_kernel(KParams p) {
     constexpr int kTile = 64 * D * 2;            // bytes per K or V tile
     __shared__ __attribute__((aligned(16))) char lds[4 * kTile];   // K0 V0 K1 V1
@@ -45,7 +47,7 @@ __global__ __launch_bounds__(kThreads) void mfma_fwd_kernel(KParams p) {
     vc.init(lane, wave, p.v, vbase);
     if (n_steps > 0) {
         kc.issue((n_steps - 1) * kKeyBlock, job.len, lds);
-        vc.issue((n_steps - 1) * kKeyBlock, job.len, lds + kTile);
+        if (!kCarryOnly) vc.issue((n_steps - 1) * kKeyBlock, job.len, lds + kTile);
     }
     wait_global_memory();
     __syncthreads();
@@ -64,7 +66,7 @@ __global__ __launch_bounds__(kThreads) void mfma_fwd_kernel(KParams p) {
             p.rtab[((int64_t)head * p.n_kb + step) * p.tab_tokens + tabtok] = R;
         if (more) {       // next tiles, straight into the other buffer (free since the last barrier)
             kc.issue((step - 1) * kKeyBlock, job.len, lds + (buf ^ 1) * 2 * kTile);
-            vc.issue((step - 1) * kKeyBlock, job.len, lds + (buf ^ 1) * 2 * kTile + kTile);
+            if (!kCarryOnly) vc.issue((step - 1) * kKeyBlock, job.len, lds + (buf ^ 1) * 2 * kTile + kTile);
         }
         if (!skip) {
             float x[32];
@@ -74,20 +76,22 @@ mask_step(x, key0 + 32 * h, qi, strict);
             }
             float dummy[1];
             stick_weights<false>(x, dummy, R, lane);
-            bf16x8 pf[4];
+            if (!kCarryOnly) {
+                bf16x8 pf[4];
 #pragma unroll
-            for (int c = 0; c < 4; ++c) pf[c] = pack8(&x[8 * c]);
+                for (int c = 0; c < 4; ++c) pf[c] = pack8(&x[8 * c]);
 #pragma unroll
-            for (int db = 0; db < D / 32; ++db)
+                for (int db = 0; db < D / 32; ++db)
 #pragma unroll
-                for (int c = 0; c < 4; ++c)
-                    oacc[db] = mfma(fetch_cols_o<D>(vtile, lo, db, c), pf[c], oacc[db]);
+                    for (int c = 0; c < 4; ++c)
+                        oacc[db] = mfma(fetch_cols_o<D>(vtile, lo, db, c), pf[c], oacc[db]);
+            }
         }
         wait_global_memory();                  // the next tiles have landed
         __syncthreads();
     }
 
-    if (qi < job.len) {
+    if (qi < job.len && !kCarryOnly) {
         const int64_t obase = (int64_t)job.seq * p.o.sb + (int64_t)head * p.o.sh + (int64_t)(job.tok0 + qi) * p.o.st;
 #pragma unroll
         for (int db = 0; db < D / 32; ++db)
@@ -116,7 +120,7 @@ mask_step(x, key0 + 32 * h, qi, strict);
 // right group's total into its carry, and each group accumulates its own partial O, summed once
 // at the end.  The longest dependent chain of a kernel launch (the sweep of the last row-block)
 // is halved, which is what bounds the time when the whole problem is only two waves per SIMD.
-template <int D>
+template <int D, bool kCarryOnly>
 __global__ __launch_bounds__(2 * kThreads) void mfma_fwd2_kernel(KParams p) {
     constexpr int kTile = 64 * D * 2;
     // tile(buf, grp, kv) = lds + ((buf * 2 + grp) * 2 + kv) * kTile
@@ -161,7 +165,7 @@ __global__ __launch_bounds__(2 * kThreads) void mfma_fwd2_kernel(KParams p) {
         const int s0 = n_steps - 1 - grp;
         if (s0 >= 0) {
             kc.issue(s0 * kKeyBlock, job.len, my_tiles);
-            vc.issue(s0 * kKeyBlock, job.len, my_tiles + kTile);
+            if (!kCarryOnly) vc.issue(s0 * kKeyBlock, job.len, my_tiles + kTile);
         }
     }
     wait_global_memory();
@@ -174,7 +178,7 @@ __global__ __launch_bounds__(2 * kThreads) void mfma_fwd2_kernel(KParams p) {
         const bool more = step - 2 >= 0;
         if (more) {       // next tiles, straight into the other buffer (free since the last barrier)
             kc.issue((step - 2) * kKeyBlock, job.len, my_tiles + (buf ^ 1) * 4 * kTile);
-            vc.issue((step - 2) * kKeyBlock, job.len, my_tiles + (buf ^ 1) * 4 * kTile + kTile);
+            if (!kCarryOnly) vc.issue((step - 2) * kKeyBlock, job.len, my_tiles + (buf ^ 1) * 4 * kTile + kTile);
         }
         const int key0 = step * kKeyBlock;
         const bool active = step >= 0 && !(key0 + strict > q0w + 31);
@@ -196,19 +200,22 @@ __global__ __launch_bounds__(2 * kThreads) void mfma_fwd2_kernel(KParams p) {
         if (active) {
             if (p.save && h == 0 && qi < job.len)
                 p.rtab[((int64_t)head * p.n_kb + step) * p.tab_tokens + tabtok] = Rmy;
-            scale_clamped<32>(x, fac * Rmy);
-            bf16x8 pf[4];
+            if (!kCarryOnly) {
+                scale_clamped<32>(x, fac * Rmy);
+                bf16x8 pf[4];
 #pragma unroll
-            for (int c = 0; c < 4; ++c) pf[c] = pack8(&x[8 * c]);
+                for (int c = 0; c < 4; ++c) pf[c] = pack8(&x[8 * c]);
 #pragma unroll
-            for (int db = 0; db < D / 32; ++db)
+                for (int db = 0; db < D / 32; ++db)
 #pragma unroll
-                for (int c = 0; c < 4; ++c)
-                    oacc[db] = mfma(fetch_cols_o<D>(vtile, lo, db, c), pf[c], oacc[db]);
+                    for (int c = 0; c < 4; ++c)
+                        oacc[db] = mfma(fetch_cols_o<D>(vtile, lo, db, c), pf[c], oacc[db]);
+            }
         }
         wait_global_memory();                  // the next tiles have landed
         __syncthreads();
     }
+    if (kCarryOnly) return;
 
     // ---- O = O(group 0) + O(group 1): group 1 parks its accumulators in LDS
     float* park = (float*)lds;                              // [qs][db][r][lane]
@@ -251,11 +258,18 @@ int sba_launch_mfma_fwd(const sba::KParams& kp, hipStream_t s) {
     // by throughput, where the 4-wave kernel (3 waves per SIMD) is ahead (measured: already at
     // 640 workgroups).
     const bool small_grid = grid.x <= sba_two_step_max_grid();
-    if (kp.head_dim == 64 && small_grid)
-        hipLaunchKernelGGL((mfma_fwd2_kernel<64>), grid, dim3(2 * kThreads), 0, s, kp);
+    if (kp.carry_only) {
+        if (kp.head_dim == 64 && small_grid)
+            hipLaunchKernelGGL((mfma_fwd2_kernel<64, true>), grid, dim3(2 * kThreads), 0, s, kp);
+        else if (kp.head_dim == 64)
+            hipLaunchKernelGGL((mfma_fwd_kernel<64, true>), grid, dim3(kThreads), 0, s, kp);
+        else
+            hipLaunchKernelGGL((mfma_fwd_kernel<128, true>), grid, dim3(kThreads), 0, s, kp);
+    } else if (kp.head_dim == 64 && small_grid)
+        hipLaunchKernelGGL((mfma_fwd2_kernel<64, false>), grid, dim3(2 * kThreads), 0, s, kp);
     else if (kp.head_dim == 64)
-        hipLaunchKernelGGL((mfma_fwd_kernel<64>), grid, dim3(kThreads), 0, s, kp);
+        hipLaunchKernelGGL((mfma_fwd_kernel<64, false>), grid, dim3(kThreads), 0, s, kp);
     else
-        hipLaunchKernelGGL((mfma_fwd_kernel<128>), grid, dim3(kThreads), 0, s, kp);
+        hipLaunchKernelGGL((mfma_fwd_kernel<128, false>), grid, dim3(kThreads), 0, s, kp);
     return hipGetLastError() == hipSuccess ? SBA_OK : SBA_ERR_LAUNCH;
 }

@@ -39,12 +39,15 @@ def workspace_bytes(q, inv_temp=1.0) -> int:
     return int(_lib.load().sba_workspace_bytes(C.byref(_params(q, q, q, inv_temp, False))))
 
 
-def bwd_scratch_bytes(q, inv_temp=1.0) -> int:
-    """What the backward needs for the duration of its call only."""
+def bwd_scratch_bytes(q, have_workspace=True) -> int:
+    """What the backward needs for the duration of its call only (one table more when the forward
+    kept none)."""
     if torch.compiler.is_compiling():
         B, H, T, D = q.shape
         return _lib.bwd_scratch_upper_bound(H, T, B * T, D)
-    return int(_lib.load().sba_bwd_scratch_bytes(C.byref(_params(q, q, q, inv_temp, False))))
+    p = _params(q, q, q, 1.0, False)
+    p.workspace = 1 if have_workspace else None       # only NULL or not is looked at
+    return int(_lib.load().sba_bwd_scratch_bytes(C.byref(p)))
 
 
 # Same registered names as the reference (sb_fwd.py:177, sb_bwd.py:207); outputs are
@@ -75,7 +78,8 @@ def _compileable_backward(do: torch.Tensor, dr: Optional[torch.Tensor], q: torch
     if dr is not None:
         p.d_rem = _lib.SbaVector(dr.data_ptr(), dr.stride(0), dr.stride(1))
     p.dq, p.dk, p.dv = _lib.tensor4(dq), _lib.tensor4(dk), _lib.tensor4(dv)
-    p.workspace, p.workspace_bytes = ws.data_ptr(), ws.numel()
+    if ws.numel() > 16:                   # a 16-byte stand-in means: nothing was kept, recompute the carries
+        p.workspace, p.workspace_bytes = ws.data_ptr(), ws.numel()
     p.bwd_scratch, p.bwd_scratch_bytes = scratch.data_ptr(), scratch.numel()
     profiling.launch_bwd(lib, p)
 
@@ -83,16 +87,17 @@ def _compileable_backward(do: torch.Tensor, dr: Optional[torch.Tensor], q: torch
 def _fwd(q, k, v, logit_scale, attend_current=False, no_grad=False):
     o = torch.empty_like(q)              # same strides as q (sb_fwd.py:144 does the same)
     rem = torch.empty(q.shape[:-1], dtype=q.dtype, device=q.device)
-    nbytes = 16 if no_grad else max(workspace_bytes(q), 16)
+    keep = not (no_grad or _lib.recompute_carries())
+    nbytes = max(workspace_bytes(q), 16) if keep else 16
     ws = torch.empty(nbytes, dtype=torch.uint8, device=q.device)
-    _compileable_fwd(q, k, v, float(logit_scale), bool(attend_current), not no_grad, o, rem, ws)
+    _compileable_fwd(q, k, v, float(logit_scale), bool(attend_current), keep, o, rem, ws)
     return o, rem, ws
 
 
 def _bwd(do, dr, q, k, v, ws, logit_scale, attend_current=False):
     dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
     # freed when this call returns: only the forward's table is kept between the two directions
-    scratch = torch.empty(max(bwd_scratch_bytes(q), 16), dtype=torch.uint8, device=q.device)
+    scratch = torch.empty(max(bwd_scratch_bytes(q, ws.numel() > 16), 16), dtype=torch.uint8, device=q.device)
     _compileable_backward(do, dr, q, k, v, ws, scratch, float(logit_scale), bool(attend_current), dq, dk, dv)
     return dq, dk, dv
 

@@ -81,13 +81,15 @@ def workspace_bytes(q, max_seqlens: int) -> int:
     return int(_lib.load().sba_workspace_bytes(C.byref(p)))
 
 
-def bwd_scratch_bytes(q, max_seqlens: int) -> int:
-    """What the backward needs for the duration of its call only."""
+def bwd_scratch_bytes(q, max_seqlens: int, have_workspace=True) -> int:
+    """What the backward needs for the duration of its call only (one table more when the forward
+    kept none)."""
     if torch.compiler.is_compiling():
         H, N, D = q.shape
         return _lib.bwd_scratch_upper_bound(H, max_seqlens, N, D)
     p = _params(q, q, q, 1, max_seqlens, 1.0, False)
     p.cu_seqlens = 1
+    p.workspace = 1 if have_workspace else None       # only NULL or not is looked at
     return int(_lib.load().sba_bwd_scratch_bytes(C.byref(p)))
 
 
@@ -123,7 +125,8 @@ def _compileable_backward(do: torch.Tensor, dr: Optional[torch.Tensor], q: torch
     if dr is not None:
         p.d_rem = _lib.SbaVector(dr.data_ptr(), 0, dr.stride(0))
     p.dq, p.dk, p.dv = _lib.tensor3(dq), _lib.tensor3(dk), _lib.tensor3(dv)
-    p.workspace, p.workspace_bytes = ws.data_ptr(), ws.numel()
+    if ws.numel() > 16:                   # a 16-byte stand-in means: nothing was kept, recompute the carries
+        p.workspace, p.workspace_bytes = ws.data_ptr(), ws.numel()
     p.bwd_scratch, p.bwd_scratch_bytes = scratch.data_ptr(), scratch.numel()
     profiling.launch_bwd(lib, p)
 
@@ -131,17 +134,18 @@ def _compileable_backward(do: torch.Tensor, dr: Optional[torch.Tensor], q: torch
 def varlen_fwd(q, k, v, cu_seqlens, max_seqlens, logit_scale, attend_current=False, no_grad=False):
     o = torch.empty_like(q)
     rem = torch.empty(q.shape[:-1], dtype=q.dtype, device=q.device)
-    nbytes = 16 if no_grad else max(workspace_bytes(q, max_seqlens), 16)
+    keep = not (no_grad or _lib.recompute_carries())
+    nbytes = max(workspace_bytes(q, max_seqlens), 16) if keep else 16
     ws = torch.empty(nbytes, dtype=torch.uint8, device=q.device)
     _compileable_forward(q, k, v, cu_seqlens, int(max_seqlens), float(logit_scale), bool(attend_current),
-                         not no_grad, o, rem, ws)
+                         keep, o, rem, ws)
     return o, rem, ws
 
 
 def varlen_bwd(do, dr, q, k, v, cu_seqlens, max_seqlens, ws, logit_scale, attend_current=False):
     dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
     # freed when this call returns: only the forward's table is kept between the two directions
-    scratch = torch.empty(max(bwd_scratch_bytes(q, max_seqlens), 16), dtype=torch.uint8, device=q.device)
+    scratch = torch.empty(max(bwd_scratch_bytes(q, max_seqlens, ws.numel() > 16), 16), dtype=torch.uint8, device=q.device)
     _compileable_backward(do, dr, q, k, v, cu_seqlens, int(max_seqlens), ws, scratch, float(logit_scale),
                           bool(attend_current), dq, dk, dv)
     return dq, dk, dv

@@ -119,6 +119,11 @@ size_t sba_workspace_bytes(const SbaParams* p);
  * tables between its two kernels, or the generic path's fp32 accumulators): allocate before
  * the call, free after it has run.  With bwd_phases 1 and 2 issued as two calls, the same
  * buffer goes to both.
+ *
+ * Memory-lean mode: a forward run WITHOUT save_for_backward keeps nothing, and sba_bwd called
+ * with workspace = NULL first repeats the forward's sweep for the carries alone (about 0.7 of
+ * a forward) into a fourth table of the scratch; this function then asks for four tables
+ * (it looks at whether p->workspace is NULL).
  */
 size_t sba_bwd_scratch_bytes(const SbaParams* p);
 

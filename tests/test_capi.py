@@ -59,7 +59,10 @@ def test_workspace_bytes(lib):
     p.n_seq, p.n_heads, p.seq_len, p.total_tokens, p.head_dim = 1, 16, 4096, 4096, 64
     table = 16 * 64 * 4096 * 4                      # one carry table [H][T/64][T] fp32
     assert lib.sba_workspace_bytes(C.byref(p)) == table          # what the forward hands to the backward
+    assert lib.sba_bwd_scratch_bytes(C.byref(p)) == 4 * table    # no workspace: the backward recomputes that table
+    p.workspace = 1
     assert lib.sba_bwd_scratch_bytes(C.byref(p)) == 3 * table    # what the backward needs for itself
+    p.workspace = None
     p.dtype = _lib.SBA_DTYPE_F32                    # generic kernels: nothing kept, fp32 dk|dv accumulators
     assert lib.sba_workspace_bytes(C.byref(p)) == 0
     assert lib.sba_bwd_scratch_bytes(C.byref(p)) == 2 * 4096 * 16 * 64 * 4

@@ -551,3 +551,33 @@ def test_forward_backward_captured_in_a_graph_replays_like_eager():
         torch.cuda.synchronize()
         for a, b in zip(got, want):
             assert torch.equal(a, b), f"replay {rep}"
+
+
+@pytest.mark.parametrize("D", [64, 128])
+def test_recomputing_the_carries_in_the_backward_gives_the_same_bits(D, monkeypatch):
+    # SBA_RECOMPUTE_CARRIES=1: the forward keeps no table and the backward repeats its sweep for the
+    # carries alone.  Same kernels, same arithmetic: every result must be bit-identical.
+    sb_attn, sb_attn_varlen = _ops()
+    lens = [300, 1, 129, 700]
+    cu = cu_from_lengths(lens).cuda()
+    q, k, v, do = (randn((3, sum(lens), D), 400 + i, 0.5 if i < 3 else 1.0, torch.bfloat16).cuda() for i in range(4))
+    drem = randn((3, sum(lens)), 405, 1.0, torch.bfloat16).cuda()
+
+    def packed():
+        qq, kk, vv = (x.clone().requires_grad_(True) for x in (q, k, v))
+        o, rem = sb_attn_varlen(qq, kk, vv, cu, max(lens))
+        torch.autograd.backward([o, rem], [do, drem])
+        return o, rem, qq.grad, kk.grad, vv.grad
+
+    def dense(rep):
+        qq, kk, vv = (x[None].expand(rep, -1, -1, -1).contiguous().requires_grad_(True) for x in (q, k, v))
+        o, rem = sb_attn(qq, kk, vv, attend_current=True)
+        torch.autograd.backward([o, rem], [do[None].expand(rep, -1, -1, -1).contiguous(), drem[None].expand(rep, -1, -1).contiguous()])
+        return o, rem, qq.grad, kk.grad, vv.grad
+
+    kept = [packed(), dense(1), dense(30)]              # small and large grids
+    monkeypatch.setenv("SBA_RECOMPUTE_CARRIES", "1")
+    again = [packed(), dense(1), dense(30)]
+    for a, b in zip(kept, again):
+        for x, y in zip(a, b):
+            assert torch.equal(x, y)
