@@ -402,15 +402,19 @@ template <int ROWD> __device__ inline bf16x8 fetch_row_nat(const char* tile, int
     return *(const bf16x8*)(tile + tile_offset<ROWD>(row, 2 * ks + (lane >> 5)));
 }
 
-// dP^T tile pair: dp[16*t + r] = (V dO^T)[key_local][query] - drem[query].
+// dP^T tile pair: dp[16*t + r] = (V dO^T)[key_local][query].  The gradient of `rem` is not
+// subtracted here: with g = a * dP taken from the plain dP, the term it contributes to the logit
+// gradient is  -beta_ik * d_rem_i * rem_i  (the weights of a row and its remainder sum to one),
+// i.e. a constant d_rem_i * rem_i added to the running prefix of g -- which is how the prefix
+// tables carry it (see the dQ kernels).  `init` is what the accumulators start from (zero).
 template <int D>
 __device__ inline void dp_tiles_o(float (&dp)[32], const char* vtile, const LaneOffsets<D>& o,
-                                  const bf16x8 (&dof)[D / 16], float dr) {
+                                  const bf16x8 (&dof)[D / 16], float init = 0.f) {
 #pragma unroll
     for (int t = 0; t < 2; ++t) {
         f32x16 acc;
 #pragma unroll
-        for (int r = 0; r < 16; ++r) acc[r] = -dr;
+        for (int r = 0; r < 16; ++r) acc[r] = init;
 #pragma unroll
         for (int ks = 0; ks < D / 16; ++ks) acc = mfma(fetch_rows_o<D>(vtile, o, t, ks), dof[ks], acc);
 #pragma unroll

@@ -7,7 +7,9 @@
 //   pass 1  (row owner, like the forward): recomputes the weights of each 64-key step from
 //           the forward's carry table, forms dz, accumulates dQ in registers, and records
 //           for every (query, key block) the prefix  sum_{j left of the block} g_ij  in a
-//           second table.
+//           second table.  g_ij = a_ij * (dO_i . v_j) here: the gradient of rem enters as the
+//           constant d_rem_i * rem_i that every prefix of row i starts from, which is all it
+//           contributes to dz (sum_j a_ij + rem_i = 1), so pass 2 never reads d_rem.
 //   pass 2  (key owner): the owner of a block of keys sweeps the query blocks at or below the
 //           diagonal, recomputes weights and dz of its tiles from the tables, transposes them
 //           through LDS and accumulates dK = dZ^T Q and dV = P^T dO in registers.  Three
@@ -77,8 +79,8 @@ __global__ __launch_bounds__(kThreads) void mfma_bwd_dq_kernel(KParams p) {
     const int64_t tix0 = (int64_t)head * p.n_kb * p.tab_tokens + tabtok;
     float Rnext = (row_ok && n_steps > 0) ? p.rtab[tix0] : 1.0f;
     float* mid_table = h == 0 ? p.rmid : p.gmid;
-    float mid = 0.f;
-    bool mid_pending = false;
+    float mid = 0.f, Genter = 0.f;
+    bool mid_pending = false, g_pending = false;
     wait_global_memory();
     __syncthreads();
     for (int step = 0, buf = 0; step < n_steps; ++step, buf ^= 1) {
@@ -88,9 +90,12 @@ __global__ __launch_bounds__(kThreads) void mfma_bwd_dq_kernel(KParams p) {
         const int key0 = step * kKeyBlock;
         const bool skip = key0 + strict > q0w + 31;
         const int64_t tix = tix0 + step * tstride;
+        // the prefix that entered the previous step (the first block's is only known once that
+        // block's weights are: it starts at d_rem * rem, see below)
+        if (g_pending && row_ok && h == 0) p.gtab[tix - tstride] = Genter;
         if (mid_pending && row_ok && p.rmid) mid_table[tix - tstride] = mid;
         mid_pending = false;
-        if (!skip && row_ok && h == 0) p.gtab[tix] = Gc;
+        g_pending = false;
         float R = Rnext;
         if (more) {
             if (row_ok) Rnext = p.rtab[tix + tstride];
@@ -108,7 +113,7 @@ mask_step(x, key0 + 32 * h, qi, strict);
             if (D == 128) {
                 // dP does not depend on the weights: its 16 MFMAs are spread under their vector
                 // arithmetic (measured: a gain at head_dim 128, none at 64)
-                dp_tiles_o<D>(dp, vtile, lo, dof, dr);
+                dp_tiles_o<D>(dp, vtile, lo, dof);
                 stick_weights<true>(x, beta, R, lane, &Rlane);
 #pragma unroll
                 for (int i = 0; i < 2 * (D / 16); ++i) {
@@ -118,8 +123,14 @@ mask_step(x, key0 + 32 * h, qi, strict);
                 }
             } else {
                 stick_weights<true>(x, beta, R, lane, &Rlane);
-                dp_tiles_o<D>(dp, vtile, lo, dof, dr);
+                dp_tiles_o<D>(dp, vtile, lo, dof);
             }
+            // The gradient of rem rides in the prefix: g is formed from the plain dP, and the term
+            // -beta_ik * d_rem_i * rem_i that d_rem adds to dz_ik is a constant d_rem_i * rem_i in
+            // the running prefix.  After the leftmost block R is the product over all keys, rem_i.
+            if (step == 0) Gc = dr * R;
+            Genter = Gc;
+            g_pending = true;
             logit_grads<false>(x, beta, dp, Gc, lane, &Glane);
             // carries in the middle of the block, for the key-owner pass whose waves own 32 keys:
             // the left half-wave holds the product entering the left 32 keys, the right half-wave
@@ -138,6 +149,7 @@ mask_step(x, key0 + 32 * h, qi, strict);
         wait_global_memory();                  // the next tiles have landed
         __syncthreads();
     }
+    if (g_pending && row_ok && h == 0) p.gtab[tix0 + (n_steps - 1) * tstride] = Genter;
     if (mid_pending && row_ok && p.rmid) mid_table[tix0 + (n_steps - 1) * tstride] = mid;
 
     if (row_ok) {
@@ -203,6 +215,11 @@ __global__ __launch_bounds__(2 * kThreads, 2) void mfma_bwd_dq2_kernel(KParams p
 #pragma unroll
     for (int db = 0; db < D / 32; ++db) dqacc[db] = f32x16{0};
     float Gc = 0.f;
+    // dP's accumulators start from a zero the compiler cannot see through, i.e. from sixteen
+    // registers kept at zero, rather than from the instruction's inline constant: the schedule
+    // that results is 1 us faster at 512 workgroups (measured)
+    float zero_block = 0.f;
+    asm volatile("" : "+v"(zero_block));
 
     const int imax = min(m0 + kRowBlock - 1, job.len - 1);
     const int kmax = imax - strict;
@@ -253,8 +270,16 @@ __global__ __launch_bounds__(2 * kThreads, 2) void mfma_bwd_dq2_kernel(KParams p
             if (key0 + 63 + strict > q0w) mask_step(x, key0 + 32 * h, qi, strict);
             float Rc = R;
             stick_weights<true>(x, beta, Rc, lane, &Rlane);
-            dp_tiles_o<D>(dp, vtile, lo, dof, dr);
+            dp_tiles_o<D>(dp, vtile, lo, dof, zero_block);
             start = logit_grads_local(x, dp, total, lane);
+            // the gradient of rem rides in the prefix as the constant d_rem * rem (see the one-step
+            // kernel).  The leftmost block is group 0's first step: the constant joins its total
+            // (which carries it to the other group and into Gc) and its own prefix
+            if (step == 0) {
+                const float c0 = dr * Rc;
+                total += c0;
+                start += c0;
+            }
         }
         if (h == 0) xch[grp][32 * qs + n] = total;
         __syncthreads();
@@ -263,11 +288,12 @@ __global__ __launch_bounds__(2 * kThreads, 2) void mfma_bwd_dq2_kernel(KParams p
         const float Gmy = grp == 0 ? Gc : Gc + other;
         Gc = Gc + total + other;
         if (active) {
-            if (row_ok && h == 0) p.gtab[tix] = Gmy;
+            const float Glane = Gmy + start;       // the prefix entering this lane's 32 keys
+            if (row_ok && h == 0) p.gtab[tix] = Glane;
             // carries in the middle of the block (see the one-step kernel)
-            mid = h == 0 ? Rlane : Gmy + start;
+            mid = h == 0 ? Rlane : Glane;
             mid_pending = true;
-            logit_grads_apply(beta, dp, Gmy + start);
+            logit_grads_apply(beta, dp, Glane);
             bf16x8 zf[4];
 #pragma unroll
             for (int c = 0; c < 4; ++c) zf[c] = pack8(&dp[8 * c]);
@@ -355,7 +381,6 @@ __global__ __launch_bounds__(kThreads, 2) void mfma_bwd_dkv_kernel(KParams p) {
     const int64_t kbase = (int64_t)job.seq * p.k.sb + (int64_t)head * p.k.sh + (int64_t)job.tok0 * p.k.st;
     const int64_t vbase = (int64_t)job.seq * p.v.sb + (int64_t)head * p.v.sh + (int64_t)job.tok0 * p.v.st;
     const int64_t dobase = (int64_t)job.seq * p.d_o.sb + (int64_t)head * p.d_o.sh + (int64_t)job.tok0 * p.d_o.st;
-    const int64_t dr_base = (int64_t)job.seq * p.d_rem.sb + (int64_t)head * p.d_rem.sh + job.tok0;
     const int64_t trow = ((int64_t)head * p.n_kb + kb) * p.tab_tokens;
     const int n_qb = (job.len + kRowBlock - 1) / kRowBlock;
     const int kh = wave & 1;                   // which 32 keys this wave reduces
@@ -380,7 +405,6 @@ __global__ __launch_bounds__(kThreads, 2) void mfma_bwd_dkv_kernel(KParams p) {
     const int qb0 = job.rb;
     // prefetched state of the first step
     float Rn = 1.0f, Gn = 0.0f;
-    uint32_t drn = 0;                          // bf16 bits, widened where used: converting here would wait for the load
     bf16x8 qfn[D / 16];
     {
         const int qi0 = qb0 * kRowBlock + 32 * wave + n;
@@ -388,7 +412,6 @@ __global__ __launch_bounds__(kThreads, 2) void mfma_bwd_dkv_kernel(KParams p) {
         if (qi0 < job.len) {
             const int64_t t = trow + tab_token(p, job, qi0);
             Rn = p.rtab[t]; Gn = p.gtab[t];
-            if (p.d_rem.ptr) drn = ((const uint16_t*)p.d_rem.ptr)[dr_base + qi0];
         }
     }
     __syncthreads();                           // K, V tiles visible
@@ -407,15 +430,13 @@ __global__ __launch_bounds__(kThreads, 2) void mfma_bwd_dkv_kernel(KParams p) {
         for (int ks = 0; ks < D / 16; ++ks) qf[ks] = qfn[ks];
         load_row_frags<D>(dof, p.d_o, dobase, qi, job.len, lane);
         float R = Rn, Gc = Gn;
-        const uint32_t dr_bits = drn;
         if (qb + 1 < n_qb) {
             const int qin = qi + kRowBlock;
             load_row_frags<D>(qfn, p.q, qbase, qin, job.len, lane);
-            Rn = 1.0f; Gn = 0.0f; drn = 0;
+            Rn = 1.0f; Gn = 0.0f;
             if (qin < job.len) {
                 const int64_t t = trow + tab_token(p, job, qin);
                 Rn = p.rtab[t]; Gn = p.gtab[t];
-                if (p.d_rem.ptr) drn = ((const uint16_t*)p.d_rem.ptr)[dr_base + qin];
             }
         }
         // (2) row 32*wave + n of the shared Q tile (every wave passed the barrier that ends the
@@ -434,7 +455,7 @@ __global__ __launch_bounds__(kThreads, 2) void mfma_bwd_dkv_kernel(KParams p) {
 #pragma unroll
             for (int ks = 0; ks < D / 16; ++ks)
                 *(bf16x8*)(dotile + tile_offset<D>(32 * wave + n, 2 * ks + h)) = dof[ks];
-            dp_tiles_o<D>(dp, vtile, lo, dof, bf16_to_f32((uint16_t)dr_bits));
+            dp_tiles_o<D>(dp, vtile, lo, dof);
             logit_grads<true>(x, beta, dp, Gc, lane);
         } else {
 #pragma unroll
@@ -532,7 +553,7 @@ __global__ __launch_bounds__(2 * kThreads, 2) void mfma_bwd_dkv_stream_kernel(KP
     constexpr int kQTile = 128 * D * 2;        // Q or dO tile (128 queries)
     constexpr int kZTile = 128 * 64 * 2;       // weights of one step, [query][key] bf16
     constexpr int kBuf = 2 * kZTile + 2 * kQTile;
-    constexpr int kCarry = kRowBlock * 16;     // {R, G, d_rem, -} per query
+    constexpr int kCarry = kRowBlock * 8;      // {R, G} per query
     __shared__ __attribute__((aligned(1024))) char lds[3 * kTile + 2 * kCarry + 2 * kBuf];
     __shared__ int consumers_done;             // consumer waves that have finished a reduction, running total
     __shared__ int producers_took_k;           // producer waves that hold an item's K fragments, running total
@@ -604,7 +625,7 @@ __global__ __launch_bounds__(2 * kThreads, 2) void mfma_bwd_dkv_stream_kernel(KP
                 float x[32], beta[32], dp[32];
                 float Gc = 0.f;
                 if (!skip) {
-                    const float4 cv = *(const float4*)(carry + (s & 1) * kCarry + (32 * w4 + n) * 16);
+                    const float2 cv = *(const float2*)(carry + (s & 1) * kCarry + (32 * w4 + n) * 8);
                     // rows past the end of the sequence hold copies of its last row: a zero carry
                     // makes their weights and gradients exactly zero
                     float R = qi < len ? cv.x : 0.f;
@@ -625,16 +646,14 @@ __global__ __launch_bounds__(2 * kThreads, 2) void mfma_bwd_dkv_stream_kernel(KP
                     }
                     scale_scores(x, raw, p.scale2);
                     if (key0 + 63 + strict > q0w) mask_step(x, key0 + 32 * h, qi, strict);
-                    // dP = dO V^T - d_rem does not depend on the weights: its eight MFMAs are spread
+                    // dP = dO V^T does not depend on the weights: its eight MFMAs are spread
                     // under the weights' vector arithmetic.  (Only instructions of ONE wave overlap
                     // this way: a SIMD does not issue another wave's vector instructions while a
                     // wave's back-to-back MFMAs wait for the matrix pipe.)
-                    const float dr = bf16_to_f32((uint16_t)__float_as_uint(cv.z));
                     f32x16 dacc[2];
 #pragma unroll
                     for (int t = 0; t < 2; ++t) {
-#pragma unroll
-                        for (int r = 0; r < 16; ++r) dacc[t][r] = -dr;
+                        dacc[t] = f32x16{0};
 #pragma unroll
                         for (int ks = 0; ks < D / 16; ++ks) dacc[t] = mfma(vfr[t][ks], dof[ks], dacc[t]);
                     }
@@ -698,7 +717,6 @@ __global__ __launch_bounds__(2 * kThreads, 2) void mfma_bwd_dkv_stream_kernel(KP
         // some path, so the compiler's wait-count bookkeeping stays exact.
         u32x4 tx[8];
         float cR, cG;
-        uint32_t cdr = 0;                      // bf16 bits
         // Four lanes fill the 64 bytes of a row that this wave reduces; an LDS write cycle takes eight
         // lanes, i.e. two rows, whose swizzles must differ in the bit that selects the other half of the
         // row's banks: rows r and r + 2 do (r and r + 1 would collide), hence the order 0 2 1 3 ...
@@ -717,10 +735,8 @@ __global__ __launch_bounds__(2 * kThreads, 2) void mfma_bwd_dkv_stream_kernel(KP
         struct ItemPtrs {
             const char* x;                     // Q or dO: row 0 of the sequence, this head, this thread's chunk
             const float *rt, *gt;              // carries of this (head, key block), query 0
-            const uint16_t* dr;                // d_rem of the sequence, query 0
             int row0, len;                     // first query of the item's sweep; sequence length
         };
-        const bool has_dr = p.d_rem.ptr != nullptr;
         auto item_ptrs = [&](const KeyItem& t) {
             ItemPtrs r;
             const TensorArg& xt = is_dv ? p.d_o : p.q;
@@ -728,10 +744,9 @@ __global__ __launch_bounds__(2 * kThreads, 2) void mfma_bwd_dkv_stream_kernel(KP
             const int64_t tk = ((int64_t)t.head * p.n_kb + t.kb) * p.tab_tokens + tab_token(p, t.job, 0);
             r.rt = p.rtab + tk;
             r.gt = p.gtab + tk;
-            r.dr = (const uint16_t*)p.d_rem.ptr + ((int64_t)t.job.seq * p.d_rem.sb + (int64_t)t.head * p.d_rem.sh + t.job.tok0);
             r.row0 = t.job.rb * kRowBlock;
             r.len = t.job.len;
-            asm volatile("" : "+v"(r.x), "+v"(r.rt), "+v"(r.gt), "+v"(r.dr));
+            asm volatile("" : "+v"(r.x), "+v"(r.rt), "+v"(r.gt));
             return r;
         };
         const uint32_t x_st2 = 2u * (uint32_t)(is_dv ? p.d_o.st : p.q.st);
@@ -745,7 +760,6 @@ __global__ __launch_bounds__(2 * kThreads, 2) void mfma_bwd_dkv_stream_kernel(KP
         auto request_carry = [&](const ItemPtrs& t, int row0) {
             const int qi = min(row0 + (ct & (kRowBlock - 1)), t.len - 1);
             cR = t.rt[qi]; cG = t.gt[qi];
-            if (has_dr) cdr = t.dr[qi];
         };
         // K and V tiles of an item go straight from global memory into LDS (no registers, and
         // nothing for the wait-count bookkeeping to track): every instruction moves 64 x 16 bytes
@@ -776,7 +790,7 @@ __global__ __launch_bounds__(2 * kThreads, 2) void mfma_bwd_dkv_stream_kernel(KP
 #pragma unroll
             for (int i = 0; i < 8; ++i) *(u32x4*)(xtile + tile_offset<D>(crow + 16 * i, cch)) = tx[i];
             if (ct < kRowBlock)
-                *(float4*)(carry + (s & 1) * kCarry + ct * 16) = float4{cR, cG, __uint_as_float(cdr), 0.f};
+                *(float2*)(carry + (s & 1) * kCarry + ct * 8) = float2{cR, cG};
         };
         auto store_staged = [&](int idx, const char* staging) {
             const KeyItem t = decode_item(p, idx);
@@ -997,9 +1011,7 @@ __global__ __launch_bounds__(kThreads, D == 64 ? 2 : 1) void mfma_bwd_dkv_own_ke
     const int kb64 = min((q_begin + 32 * wave) / kKeyBlock, p.n_kb - 1);   // (waves past the end have no work)
     const float* rsrc = ((wave & 1) ? p.rtab : p.rmid) + ((int64_t)head * p.n_kb + kb64) * p.tab_tokens;
     const float* gsrc = ((wave & 1) ? p.gmid : p.gtab) + ((int64_t)head * p.n_kb + kb64) * p.tab_tokens;
-    const char* drsrc = p.d_rem.ptr ? p.d_rem.ptr + 2 * ((int64_t)job.seq * p.d_rem.sb + (int64_t)head * p.d_rem.sh + job.tok0) : nullptr;
     float Rn[2] = {1.f, 1.f}, Gn[2] = {0.f, 0.f};
-    uint32_t drn[2] = {0u, 0u};
     auto request_carries = [&](int q0) {
 #pragma unroll
         for (int t = 0; t < 2; ++t) {
@@ -1007,7 +1019,6 @@ __global__ __launch_bounds__(kThreads, D == 64 ? 2 : 1) void mfma_bwd_dkv_own_ke
             const int64_t tok = tab_token(p, job, qi);
             Rn[t] = rsrc[tok];
             Gn[t] = gsrc[tok];
-            if (drsrc) drn[t] = ((const uint16_t*)drsrc)[qi];
         }
     };
     if (n_steps > 0) request_carries(q_begin);
@@ -1019,9 +1030,9 @@ __global__ __launch_bounds__(kThreads, D == 64 ? 2 : 1) void mfma_bwd_dkv_own_ke
         const char* dotile = qtile + kQTile;
         const int q0 = q_begin + step * kStep;
         const bool more = step + 1 < n_steps;
-        float Rin[2], Gin[2], dr[2];
+        float Rin[2], Gin[2];
 #pragma unroll
-        for (int t = 0; t < 2; ++t) { Rin[t] = Rn[t]; Gin[t] = Gn[t]; dr[t] = bf16_to_f32((uint16_t)drn[t]); }
+        for (int t = 0; t < 2; ++t) { Rin[t] = Rn[t]; Gin[t] = Gn[t]; }
         if (more) {       // next tiles, straight into the other buffer (free since the last barrier)
             qc.issue(q0 + kStep, job.len, lds + (buf ^ 1) * 2 * kQTile);
             dc.issue(q0 + kStep, job.len, lds + (buf ^ 1) * 2 * kQTile + kQTile);
@@ -1055,9 +1066,7 @@ __global__ __launch_bounds__(kThreads, D == 64 ? 2 : 1) void mfma_bwd_dkv_own_ke
                 }
                 own_tile_weights(x, beta, Rt, lane);
                 {
-                    f32x16 acc;
-#pragma unroll
-                    for (int r = 0; r < 16; ++r) acc[r] = -dr[t];
+                    f32x16 acc = {0};
 #pragma unroll
                     for (int ks = 0; ks < D / 16; ++ks)
                         acc = mfma(vfr[ks], fetch_row_nat<D>(dotile, 32 * t + n, ks, lane), acc);

@@ -404,6 +404,26 @@ def test_small_and_large_grids_take_different_backward_kernels_and_agree(D):
         assert rel_l2(a.float().cpu(), r) <= 5e-2 and rel_l2(b[39:].float().cpu(), r) <= 5e-2
 
 
+@pytest.mark.parametrize("D", [64, 128])
+@pytest.mark.parametrize("rep", [1, 40])
+def test_gradient_of_rem_alone(D, rep):
+    # dO = 0: everything comes from d_rem, which the matrix-core backward carries as the constant
+    # d_rem * rem in its prefix tables (dz_ik = -beta_ik d_rem_i rem_i); dV must be exactly zero.
+    # rep = 1 / 40: the small-grid and the large-grid kernels of both passes.
+    sb_attn, _ = _ops()
+    base = [randn((1, 4, 700, D), 140 + i, 0.5, torch.bfloat16).cuda() for i in range(3)]
+    drem = randn((1, 4, 700), 143, 1.0, torch.bfloat16).cuda()
+    q, k, v = (x.expand(rep, -1, -1, -1).contiguous().requires_grad_() for x in base)
+    o, rem = sb_attn(q, k, v)
+    torch.autograd.backward([o, rem], [torch.zeros_like(o), drem.expand(rep, -1, -1).contiguous()])
+    assert torch.count_nonzero(v.grad) == 0
+    qc, kc, vc = (x.cpu() for x in base)
+    ref = O.sb_attn_grads_oracle(qc, kc, vc, torch.zeros_like(qc), drem.cpu())
+    for g, r in zip((q.grad, k.grad), ref[-3:-1]):
+        assert rel_l2(g[rep - 1:].float().cpu(), r) <= 5e-2
+        assert torch.equal(g[0], g[rep - 1])
+
+
 def _full_size_properties(fwd_bwd, v_shape_like, check_docs=None):
     """Size-independent properties of a forward+backward at a full BASELINE size (no O(T^2)
     oracle needed): the backward is linear in the upstream gradients and bit-reproducible,
