@@ -339,6 +339,18 @@ __device__ inline void score_tiles_o(float (&x)[32], const char* ktile, const La
 // One exchange between the half-waves supplies the factor the lower (left) half is missing.
 // Outputs: x[idx] = A (attention weight); beta[idx] when kNeedBeta; R updated to the carry
 // for the next (left) step; *lane_carry = the carry entering this lane's 32 keys.
+// The two lanes (n, 0) and (n, 1) that share a query exchange one value per step.  The hardware
+// swaps the upper half of one register with the lower half of another in a single vector
+// instruction (v_permlane32_swap): started from two copies of `v`, one register ends up holding
+// the lower half-wave's value in every lane and the other the upper half-wave's.  No LDS round
+// trip (ds_bpermute) in the middle of the dependent chain.
+__device__ inline void half_values(float v, float& lower, float& upper) {
+    typedef unsigned u32x2 __attribute__((ext_vector_type(2)));
+    const u32x2 r = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    lower = __uint_as_float(r[0]);
+    upper = __uint_as_float(r[1]);
+}
+
 __device__ inline float clamp01(float v) { return __builtin_amdgcn_fmed3f(v, 0.0f, 1.0f); }
 
 template <bool kNeedBeta, int N>
@@ -365,12 +377,13 @@ template <bool kNeedBeta>
 __device__ inline void stick_weights(float (&x)[32], float (&beta)[kNeedBeta ? 32 : 1], float& R, int lane,
                                      float* lane_carry = nullptr) {
     const float L = product_chain<kNeedBeta, 32>(x, beta);
-    const float other = __shfl_xor(L, 32);
+    float Llo, Lup;
+    half_values(L, Llo, Lup);
     // upper half-wave holds the right 32 keys: its chain starts from R itself
-    const float F = (lane >= 32) ? R : R * other;
+    const float F = (lane >= 32) ? R : R * Lup;
     if (lane_carry) *lane_carry = F;      // the carry entering this lane's 32 keys
     scale_clamped<32>(x, F);
-    R = R * L * other;
+    R = R * Llo * Lup;
 }
 
 // The same in two parts, for kernels in which another wave-group handles the neighbouring
@@ -383,9 +396,10 @@ template <bool kNeedBeta>
 __device__ inline float stick_weights_local(float (&x)[32], float (&beta)[kNeedBeta ? 32 : 1], float& total,
                                             int lane) {
     const float L = product_chain<kNeedBeta, 32>(x, beta);
-    const float other = __shfl_xor(L, 32);
-    total = L * other;
-    return (lane >= 32) ? 1.0f : other;
+    float Llo, Lup;
+    half_values(L, Llo, Lup);
+    total = Llo * Lup;
+    return (lane >= 32) ? 1.0f : Lup;
 }
 
 // Sets the logits of invisible (query, key) pairs of a diagonal step to -inf.
@@ -423,7 +437,7 @@ __device__ inline void dp_tiles_o(float (&dp)[32], const char* vtile, const Lane
 }
 
 // Gradient of the logits for one step.  In: a[idx] attention weights, beta[idx],
-// dp[idx] = dO.v - drem, Gc = sum of g over all keys LEFT of this step.
+// dp[idx] = dO.v, Gc = sum of g over all keys LEFT of this step (plus d_rem * rem).
 // Out: dp[idx] <- dz = g - beta * prefix_sum(g);  Gc advanced past this step.
 // The inclusive prefix runs left-to-right inside the lane's 32 keys; the upper (right)
 // half-wave adds the lower half's total.  kLowReg trades one more add per element for
@@ -438,15 +452,16 @@ __device__ inline void logit_grads(const float (&a)[32], const float (&beta)[32]
             dp[idx] = a[idx] * dp[idx];     // g
             c += dp[idx];
         }
-        const float other = __shfl_xor(c, 32);
-        float run = (lane >= 32) ? Gc + other : Gc;
+        float clo, cup;
+        half_values(c, clo, cup);
+        float run = (lane >= 32) ? Gc + clo : Gc;
         if (lane_prefix) *lane_prefix = run;     // the prefix entering this lane's 32 keys
 #pragma unroll
         for (int idx = 0; idx < 32; ++idx) {
             run += dp[idx];
             dp[idx] = __builtin_fmaf(-beta[idx], run, dp[idx]);
         }
-        Gc = Gc + c + other;
+        Gc = Gc + clo + cup;
     } else {
         float pre[32];
 #pragma unroll
@@ -455,12 +470,13 @@ __device__ inline void logit_grads(const float (&a)[32], const float (&beta)[32]
             c += dp[idx];
             pre[idx] = c;
         }
-        const float other = __shfl_xor(c, 32);
-        const float F = (lane >= 32) ? Gc + other : Gc;
+        float clo, cup;
+        half_values(c, clo, cup);
+        const float F = (lane >= 32) ? Gc + clo : Gc;
         if (lane_prefix) *lane_prefix = F;       // the prefix entering this lane's 32 keys
 #pragma unroll
         for (int idx = 0; idx < 32; ++idx) dp[idx] = __builtin_fmaf(-beta[idx], pre[idx] + F, dp[idx]);
-        Gc = Gc + c + other;
+        Gc = Gc + clo + cup;
     }
 }
 
@@ -474,9 +490,10 @@ __device__ inline float logit_grads_local(const float (&a)[32], float (&dp)[32],
         dp[idx] = a[idx] * dp[idx];     // g
         c += dp[idx];
     }
-    const float other = __shfl_xor(c, 32);
-    total = c + other;
-    return (lane >= 32) ? other : 0.0f;
+    float clo, cup;
+    half_values(c, clo, cup);
+    total = clo + cup;
+    return (lane >= 32) ? clo : 0.0f;
 }
 __device__ inline void logit_grads_apply(const float (&beta)[32], float (&dp)[32], float start) {
     float run = start;

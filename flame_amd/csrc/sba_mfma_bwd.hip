@@ -938,8 +938,9 @@ __global__ __launch_bounds__(2 * kThreads, 2) void mfma_bwd_dkv_stream_kernel(KP
 // come back transposed as the A operands of  dV += A^T dO  and  dK += dZ^T Q.
 __device__ inline void own_tile_weights(float (&x)[16], float (&beta)[16], float Rin, int lane) {
     const float L = product_chain<true, 16>(x, beta);
-    const float other = __shfl_xor(L, 32);
-    scale_clamped<16>(x, (lane >= 32) ? Rin : Rin * other);       // upper half-wave: the right 16 keys
+    float Llo, Lup;
+    half_values(L, Llo, Lup);
+    scale_clamped<16>(x, (lane >= 32) ? Rin : Rin * Lup);         // upper half-wave: the right 16 keys
 }
 __device__ inline void own_tile_grads(const float (&a)[16], const float (&beta)[16], float (&dp)[16], float Gin,
                                       int lane) {
@@ -950,8 +951,9 @@ __device__ inline void own_tile_grads(const float (&a)[16], const float (&beta)[
         c += dp[idx];
         pre[idx] = c;
     }
-    const float other = __shfl_xor(c, 32);
-    const float F = (lane >= 32) ? Gin + other : Gin;
+    float clo, cup;
+    half_values(c, clo, cup);
+    const float F = (lane >= 32) ? Gin + clo : Gin;
 #pragma unroll
     for (int idx = 0; idx < 16; ++idx) dp[idx] = __builtin_fmaf(-beta[idx], pre[idx] + F, dp[idx]);
 }
