@@ -368,6 +368,29 @@ __device__ inline float product_chain(float (&x)[N], float (&beta)[kNeedBeta ? N
     }
     return clamp01(L);
 }
+// The same chain with a hook: `between(seg)` runs after every four keys (seg = 0 .. N/4 - 1) and
+// a scheduling fence keeps what it issues at that place.  The exp/rcp of the chain overlap MFMAs
+// in flight (plain vector instructions do not), so a kernel hands the chain the MFMAs that do
+// not depend on the weights, a few per segment.
+template <bool kNeedBeta, int N, class Between>
+__device__ inline float product_chain_with(float (&x)[N], float (&beta)[kNeedBeta ? N : 1], Between&& between) {
+    float W = 1.0f, L = 1.0f;
+#pragma unroll
+    for (int idx = N - 1; idx >= 0; --idx) {
+        const float e = __builtin_amdgcn_exp2f(x[idx]);
+        const float Wn = __builtin_fmaf(W, e, W);
+        const float Ln = __builtin_amdgcn_rcpf(Wn);
+        x[idx] = L - Ln;
+        if (kNeedBeta) beta[idx] = clamp01(__builtin_fmaf(-W, Ln, 1.0f));
+        W = Wn;
+        L = Ln;
+        if ((idx & 3) == 0) {
+            between((N - 1 - idx) >> 2);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    }
+    return clamp01(L);
+}
 template <int N> __device__ inline void scale_clamped(float (&x)[N], float f) {
 #pragma unroll
     for (int idx = 0; idx < N; ++idx) x[idx] = clamp01(x[idx] * f);
@@ -384,6 +407,54 @@ __device__ inline void stick_weights(float (&x)[32], float (&beta)[kNeedBeta ? 3
     if (lane_carry) *lane_carry = F;      // the carry entering this lane's 32 keys
     scale_clamped<32>(x, F);
     R = R * Llo * Lup;
+}
+
+// stick_weights<true> with a hook between the eight segments of the chain (see product_chain_with).
+template <class Between>
+__device__ inline void stick_weights_hooked(float (&x)[32], float (&beta)[32], float& R, int lane, float* lane_carry,
+                                            Between&& between) {
+    const float L = product_chain_with<true, 32>(x, beta, between);
+    float Llo, Lup;
+    half_values(L, Llo, Lup);
+    const float F = (lane >= 32) ? R : R * Lup;
+    if (lane_carry) *lane_carry = F;
+    scale_clamped<32>(x, F);
+    R = R * Llo * Lup;
+}
+
+// stick_weights<true> with the dP MFMAs of the step (dp[16t + r] = (V dO^T)[key][query], see
+// dp_tiles_o) issued between the segments of the chain, their operands fetched one segment ahead.
+template <int D>
+__device__ inline void stick_weights_and_dp(float (&x)[32], float (&beta)[32], float (&dp)[32], float& R, int lane,
+                                            float* lane_carry, const char* vtile, const LaneOffsets<D>& o,
+                                            const bf16x8 (&dof)[D / 16]) {
+    constexpr int kPer = D / 64;               // MFMAs per segment: 2 tiles x D/16 slices over 8 segments
+    f32x16 dacc[2];
+    bf16x8 nx[kPer];
+    // MFMA m (0 .. D/8 - 1): tile t = m & 1, slice ks = m >> 1 (neighbours use different accumulators)
+#pragma unroll
+    for (int i = 0; i < kPer; ++i) nx[i] = fetch_rows_o<D>(vtile, o, i & 1, i >> 1);
+    stick_weights_hooked(x, beta, R, lane, lane_carry, [&](int seg) {
+        bf16x8 cur[kPer];
+#pragma unroll
+        for (int i = 0; i < kPer; ++i) cur[i] = nx[i];
+        if (seg < 7) {
+#pragma unroll
+            for (int i = 0; i < kPer; ++i) {
+                const int m = kPer * (seg + 1) + i;
+                nx[i] = fetch_rows_o<D>(vtile, o, m & 1, m >> 1);
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < kPer; ++i) {
+            const int m = kPer * seg + i, t = m & 1, ks = m >> 1;
+            dacc[t] = mfma(cur[i], dof[ks], ks == 0 ? f32x16{0} : dacc[t]);
+        }
+    });
+#pragma unroll
+    for (int t = 0; t < 2; ++t)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) dp[16 * t + r] = dacc[t][r];
 }
 
 // The same in two parts, for kernels in which another wave-group handles the neighbouring

@@ -110,21 +110,9 @@ __global__ __launch_bounds__(kThreads) void mfma_bwd_dq_kernel(KParams p) {
             if (key0 + 63 + strict > q0w) {
 mask_step(x, key0 + 32 * h, qi, strict);
             }
-            if (D == 128) {
-                // dP does not depend on the weights: its 16 MFMAs are spread under their vector
-                // arithmetic (measured: a gain at head_dim 128, none at 64)
-                dp_tiles_o<D>(dp, vtile, lo, dof);
-                stick_weights<true>(x, beta, R, lane, &Rlane);
-#pragma unroll
-                for (int i = 0; i < 2 * (D / 16); ++i) {
-                    __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);     // one LDS read (the MFMA's A operand)
-                    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);     // one MFMA
-                    __builtin_amdgcn_sched_group_barrier(0x002, 8, 0);     // eight vector instructions
-                }
-            } else {
-                stick_weights<true>(x, beta, R, lane, &Rlane);
-                dp_tiles_o<D>(dp, vtile, lo, dof);
-            }
+            // dP does not depend on the weights: its MFMAs go between the segments of the chain,
+            // where the chain's exp/rcp overlap them
+            stick_weights_and_dp<D>(x, beta, dp, R, lane, &Rlane, vtile, lo, dof);
             // The gradient of rem rides in the prefix: g is formed from the plain dP, and the term
             // -beta_ik * d_rem_i * rem_i that d_rem adds to dz_ik is a constant d_rem_i * rem_i in
             // the running prefix.  After the leftmost block R is the product over all keys, rem_i.
@@ -215,11 +203,6 @@ __global__ __launch_bounds__(2 * kThreads, 2) void mfma_bwd_dq2_kernel(KParams p
 #pragma unroll
     for (int db = 0; db < D / 32; ++db) dqacc[db] = f32x16{0};
     float Gc = 0.f;
-    // dP's accumulators start from a zero the compiler cannot see through, i.e. from sixteen
-    // registers kept at zero, rather than from the instruction's inline constant: the schedule
-    // that results is 1 us faster at 512 workgroups (measured)
-    float zero_block = 0.f;
-    asm volatile("" : "+v"(zero_block));
 
     const int imax = min(m0 + kRowBlock - 1, job.len - 1);
     const int kmax = imax - strict;
@@ -269,8 +252,7 @@ __global__ __launch_bounds__(2 * kThreads, 2) void mfma_bwd_dq2_kernel(KParams p
             score_tiles_o<D>(x, ktile, lo, qf, p.scale2);
             if (key0 + 63 + strict > q0w) mask_step(x, key0 + 32 * h, qi, strict);
             float Rc = R;
-            stick_weights<true>(x, beta, Rc, lane, &Rlane);
-            dp_tiles_o<D>(dp, vtile, lo, dof, zero_block);
+            stick_weights_and_dp<D>(x, beta, dp, Rc, lane, &Rlane, vtile, lo, dof);
             start = logit_grads_local(x, dp, total, lane);
             // the gradient of rem rides in the prefix as the constant d_rem * rem (see the one-step
             // kernel).  The leftmost block is group 0's first step: the constant joins its total
@@ -646,23 +628,14 @@ __global__ __launch_bounds__(2 * kThreads, 2) void mfma_bwd_dkv_stream_kernel(KP
                     }
                     scale_scores(x, raw, p.scale2);
                     if (key0 + 63 + strict > q0w) mask_step(x, key0 + 32 * h, qi, strict);
-                    // dP = dO V^T does not depend on the weights: its eight MFMAs are spread
-                    // under the weights' vector arithmetic.  (Only instructions of ONE wave overlap
-                    // this way: a SIMD does not issue another wave's vector instructions while a
-                    // wave's back-to-back MFMAs wait for the matrix pipe.)
+                    // dP = dO V^T does not depend on the weights: its eight MFMAs go between the
+                    // segments of the chain, where the chain's exp/rcp overlap them
+                    static_assert(D == 64, "one dP MFMA per chain segment");
                     f32x16 dacc[2];
-#pragma unroll
-                    for (int t = 0; t < 2; ++t) {
-                        dacc[t] = f32x16{0};
-#pragma unroll
-                        for (int ks = 0; ks < D / 16; ++ks) dacc[t] = mfma(vfr[t][ks], dof[ks], dacc[t]);
-                    }
-                    stick_weights<true>(x, beta, R, lane);
-#pragma unroll
-                    for (int i = 0; i < 2 * (D / 16); ++i) {
-                        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);     // one MFMA
-                        __builtin_amdgcn_sched_group_barrier(0x002, 36, 0);    // 36 vector instructions
-                    }
+                    stick_weights_hooked(x, beta, R, lane, nullptr, [&](int seg) {
+                        const int t = seg & 1, ks = seg >> 1;
+                        dacc[t] = mfma(vfr[t][ks], dof[ks], ks == 0 ? f32x16{0} : dacc[t]);
+                    });
 #pragma unroll
                     for (int t = 0; t < 2; ++t)
 #pragma unroll
