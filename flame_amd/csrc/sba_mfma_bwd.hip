@@ -909,8 +909,9 @@ __global__ __launch_bounds__(2 * kThreads, 2) void mfma_bwd_dkv_stream_kernel(KP
 // a 64-key block that touches the edge, the mid-block ones for the other half.  Weights and
 // logit gradients go as bf16 [query][32 a | 32 dz] rows into a tile private to the wave and
 // come back transposed as the A operands of  dV += A^T dO  and  dK += dZ^T Q.
-__device__ inline void own_tile_weights(float (&x)[16], float (&beta)[16], float Rin, int lane) {
-    const float L = product_chain<true, 16>(x, beta);
+template <class Between>
+__device__ inline void own_tile_weights(float (&x)[16], float (&beta)[16], float Rin, int lane, Between&& between) {
+    const float L = product_chain_with<true, 16>(x, beta, between);
     float Llo, Lup;
     half_values(L, Llo, Lup);
     scale_clamped<16>(x, (lane >= 32) ? Rin : Rin * Lup);         // upper half-wave: the right 16 keys
@@ -1039,7 +1040,34 @@ __global__ __launch_bounds__(kThreads, D == 64 ? 2 : 1) void mfma_bwd_dkv_own_ke
                     for (int idx = 0; idx < 16; ++idx)
                         if (idx >= nvis) x[idx] = -INFINITY;
                 }
-                own_tile_weights(x, beta, Rt, lane);
+                if (t == 0) {
+                    own_tile_weights(x, beta, Rt, lane, [](int) {});
+                } else {
+                    // The reduction over the first tile's 32 queries only needs that tile's weights, which
+                    // this wave wrote above: its MFMAs go between the segments of the second tile's chain,
+                    // whose exp/rcp overlap them.  Segment 2kk: dV += A^T dO, segment 2kk + 1: dK += dZ^T Q.
+                    auto red_a = [&](int seg) { return fetch_nat_o<64>(ztile, lz, 16 * (seg >> 1), seg & 1); };
+                    auto red_b = [&](int seg, int db) { return fetch_nat_o<D>((seg & 1) ? qtile : dotile, lo, 16 * (seg >> 1), db); };
+                    bf16x8 na = red_a(0), nb[D / 32];
+#pragma unroll
+                    for (int db = 0; db < D / 32; ++db) nb[db] = red_b(0, db);
+                    own_tile_weights(x, beta, Rt, lane, [&](int seg) {
+                        const bf16x8 ca = na;
+                        bf16x8 cb[D / 32];
+#pragma unroll
+                        for (int db = 0; db < D / 32; ++db) cb[db] = nb[db];
+                        if (seg < 3) {
+                            na = red_a(seg + 1);
+#pragma unroll
+                            for (int db = 0; db < D / 32; ++db) nb[db] = red_b(seg + 1, db);
+                        }
+#pragma unroll
+                        for (int db = 0; db < D / 32; ++db) {
+                            if (seg & 1) dkacc[db] = mfma(ca, cb[db], dkacc[db]);
+                            else dvacc[db] = mfma(ca, cb[db], dvacc[db]);
+                        }
+                    });
+                }
                 {
                     f32x16 acc = {0};
 #pragma unroll
@@ -1057,7 +1085,7 @@ __global__ __launch_bounds__(kThreads, D == 64 ? 2 : 1) void mfma_bwd_dkv_own_ke
             }
             // dV += A^T dO, dK += dZ^T Q over the 64 queries of the step
 #pragma unroll
-            for (int kk = 0; kk < 4; ++kk) {
+            for (int kk = 2; kk < 4; ++kk) {       // the second tile's queries (the first tile's went with its chain)
                 const bf16x8 af = fetch_nat_o<64>(ztile, lz, 16 * kk, 0);
                 const bf16x8 zf = fetch_nat_o<64>(ztile, lz, 16 * kk, 1);
 #pragma unroll
