@@ -937,7 +937,13 @@ __global__ __launch_bounds__(kThreads, D == 64 ? 2 : 1) void mfma_bwd_dkv_own_ke
     constexpr int kQTile = 64 * D * 2;           // Q or dO tile of one step (64 queries)
     constexpr int kZTile = 64 * 64 * 2;          // per wave: [64 queries][32 a | 32 dz] bf16
     constexpr int kStep = 64;
-    __shared__ __attribute__((aligned(16))) char lds[4 * kQTile + 4 * kZTile];   // Q0 dO0 Q1 dO1 | one Z tile per wave
+    // At head_dim 128 a SIMD holds one wave, so nothing but the wave itself can keep the matrix cores
+    // busy during its exp/rcp: there the reduction over a step's second tile waits for the NEXT step
+    // and goes between the segments of that step's first chain.  The Q / dO tiles of a step then
+    // have to outlive it by one step: three tile buffers instead of two.
+    constexpr bool kDefer = D == 128;
+    constexpr int kNBuf = kDefer ? 3 : 2;
+    __shared__ __attribute__((aligned(16))) char lds[2 * kNBuf * kQTile + 4 * kZTile];   // Q, dO per buffer | one Z tile per wave
 
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -951,7 +957,7 @@ __global__ __launch_bounds__(kThreads, D == 64 ? 2 : 1) void mfma_bwd_dkv_own_ke
     const int strict = p.attend_current ? 0 : 1;
     const int q_begin = job.rb * kRowBlock;            // first key of the block = first query that may see it
     const int kb0 = q_begin + 32 * wave;               // first key of this wave
-    char* ztile = lds + 4 * kQTile + wave * kZTile;
+    char* ztile = lds + 2 * kNBuf * kQTile + wave * kZTile;
 
     const int64_t qbase = (int64_t)job.seq * p.q.sb + (int64_t)head * p.q.sh + (int64_t)job.tok0 * p.q.st;
     const int64_t kbase = (int64_t)job.seq * p.k.sb + (int64_t)head * p.k.sh + (int64_t)job.tok0 * p.k.st;
@@ -1001,17 +1007,34 @@ __global__ __launch_bounds__(kThreads, D == 64 ? 2 : 1) void mfma_bwd_dkv_own_ke
     wait_global_memory();
     __syncthreads();
 
-    for (int step = 0, buf = 0; step < n_steps; ++step, buf ^= 1) {
+    auto second_tile_reduction = [&](const char* qt, const char* dot) {
+#pragma unroll
+        for (int kk = 2; kk < 4; ++kk) {
+            const bf16x8 af = fetch_nat_o<64>(ztile, lz, 16 * kk, 0);
+            const bf16x8 zf = fetch_nat_o<64>(ztile, lz, 16 * kk, 1);
+#pragma unroll
+            for (int db = 0; db < D / 32; ++db) {
+                dvacc[db] = mfma(af, fetch_nat_o<D>(dot, lo, 16 * kk, db), dvacc[db]);
+                dkacc[db] = mfma(zf, fetch_nat_o<D>(qt, lo, 16 * kk, db), dkacc[db]);
+            }
+        }
+    };
+    bool pending = false;                      // the previous step left its second tile's reduction to this one
+    int buf = 0, pbuf = 0;
+    for (int step = 0; step < n_steps; ++step) {
         const char* qtile = lds + buf * 2 * kQTile;
         const char* dotile = qtile + kQTile;
+        const char* pqtile = lds + pbuf * 2 * kQTile;        // the previous step's tiles (kDefer)
+        const char* pdotile = pqtile + kQTile;
+        const int nbuf = buf + 1 == kNBuf ? 0 : buf + 1;
         const int q0 = q_begin + step * kStep;
         const bool more = step + 1 < n_steps;
         float Rin[2], Gin[2];
 #pragma unroll
         for (int t = 0; t < 2; ++t) { Rin[t] = Rn[t]; Gin[t] = Gn[t]; }
-        if (more) {       // next tiles, straight into the other buffer (free since the last barrier)
-            qc.issue(q0 + kStep, job.len, lds + (buf ^ 1) * 2 * kQTile);
-            dc.issue(q0 + kStep, job.len, lds + (buf ^ 1) * 2 * kQTile + kQTile);
+        if (more) {       // next tiles, straight into the next buffer (nobody reads it since the last barrier)
+            qc.issue(q0 + kStep, job.len, lds + nbuf * 2 * kQTile);
+            dc.issue(q0 + kStep, job.len, lds + nbuf * 2 * kQTile + kQTile);
             request_carries(q0 + kStep);
         }
         // whole step left of this wave's first key: nothing visible
@@ -1040,7 +1063,31 @@ __global__ __launch_bounds__(kThreads, D == 64 ? 2 : 1) void mfma_bwd_dkv_own_ke
                     for (int idx = 0; idx < 16; ++idx)
                         if (idx >= nvis) x[idx] = -INFINITY;
                 }
-                if (t == 0) {
+                if (t == 0 && kDefer && pending) {
+                    // the previous step's second tile: rows 32.. of the wave's weight tile (not yet
+                    // overwritten: this step's second tile comes later) and of the previous Q / dO tiles
+                    auto red_a = [&](int seg) { return fetch_nat_o<64>(ztile, lz, 32 + 16 * (seg >> 1), seg & 1); };
+                    auto red_b = [&](int seg, int db) { return fetch_nat_o<D>((seg & 1) ? pqtile : pdotile, lo, 32 + 16 * (seg >> 1), db); };
+                    bf16x8 na = red_a(0), nb[D / 32];
+#pragma unroll
+                    for (int db = 0; db < D / 32; ++db) nb[db] = red_b(0, db);
+                    own_tile_weights(x, beta, Rt, lane, [&](int seg) {
+                        const bf16x8 ca = na;
+                        bf16x8 cb[D / 32];
+#pragma unroll
+                        for (int db = 0; db < D / 32; ++db) cb[db] = nb[db];
+                        if (seg < 3) {
+                            na = red_a(seg + 1);
+#pragma unroll
+                            for (int db = 0; db < D / 32; ++db) nb[db] = red_b(seg + 1, db);
+                        }
+#pragma unroll
+                        for (int db = 0; db < D / 32; ++db) {
+                            if (seg & 1) dkacc[db] = mfma(ca, cb[db], dkacc[db]);
+                            else dvacc[db] = mfma(ca, cb[db], dvacc[db]);
+                        }
+                    });
+                } else if (t == 0) {
                     own_tile_weights(x, beta, Rt, lane, [](int) {});
                 } else {
                     // The reduction over the first tile's 32 queries only needs that tile's weights, which
@@ -1083,21 +1130,17 @@ __global__ __launch_bounds__(kThreads, D == 64 ? 2 : 1) void mfma_bwd_dkv_own_ke
                 *(bf16x8*)(ztile + tile_offset<64>(32 * t + n, 4 + 2 * h)) = pack8(&dp[0]);
                 *(bf16x8*)(ztile + tile_offset<64>(32 * t + n, 4 + 2 * h + 1)) = pack8(&dp[8]);
             }
-            // dV += A^T dO, dK += dZ^T Q over the 64 queries of the step
-#pragma unroll
-            for (int kk = 2; kk < 4; ++kk) {       // the second tile's queries (the first tile's went with its chain)
-                const bf16x8 af = fetch_nat_o<64>(ztile, lz, 16 * kk, 0);
-                const bf16x8 zf = fetch_nat_o<64>(ztile, lz, 16 * kk, 1);
-#pragma unroll
-                for (int db = 0; db < D / 32; ++db) {
-                    dvacc[db] = mfma(af, fetch_nat_o<D>(dotile, lo, 16 * kk, db), dvacc[db]);
-                    dkacc[db] = mfma(zf, fetch_nat_o<D>(qtile, lo, 16 * kk, db), dkacc[db]);
-                }
-            }
+            // dV += A^T dO, dK += dZ^T Q over the second tile's queries (the first tile's went with the
+            // second chain): now, or with the next step's first chain
+            if (!kDefer) second_tile_reduction(qtile, dotile);
+            pending = kDefer;
         }
         wait_global_memory();                  // the next tiles and carries have landed
         __syncthreads();
+        pbuf = buf;
+        buf = nbuf;
     }
+    if (kDefer && pending) second_tile_reduction(lds + pbuf * 2 * kQTile, lds + pbuf * 2 * kQTile + kQTile);
 
     // ---- rows kb0.. of dK (scaled) and dV, through the wave's own tile as coalesced 16-byte stores
 #pragma unroll
