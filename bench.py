@@ -127,7 +127,7 @@ def settle_clocks(step, seconds=0.3):
 
 
 def bench_model(args, dev):
-    """BASELINE config 5: full SBA-340M training step, one packed row of 8192 tokens."""
+    """benchmark configuration 5: full SBA-340M training step, one packed row of 8192 tokens."""
     import torch
     from flame_amd.modeling_sba import SBAConfig, SBAForCausalLM
     from flame_amd.train_step import make_optimizer, train_step

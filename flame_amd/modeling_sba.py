@@ -1,4 +1,4 @@
-"""SBA language model for the single-GPU training step (BASELINE config 5).
+"""SBA language model for the single-GPU training step (benchmark configuration 5).
 
 Plain-PyTorch counterpart of custom_models/sba/modeling_sba.py:34-407 and config_sba.py:
 pre-norm blocks [RMSNorm -> SBA -> +res -> RMSNorm -> SwiGLU MLP -> +res]

@@ -1,4 +1,4 @@
-"""One single-GPU training step of the SBA language model (BASELINE config 5):
+"""One single-GPU training step of the SBA language model (benchmark configuration 5):
 bf16 autocast, fp32 master weights, AdamW (betas 0.9/0.95, eps 1e-15 and gradient
 clipping 1.0 as in the reference's flame/models/fla.toml), one packed varlen sequence."""
 from __future__ import annotations

@@ -47,7 +47,7 @@ def _check_dense(B, H, T, D, dtype, attend_current=False, seed=0, in_scale=1.0, 
 
 
 def test_config1_fp32_forward_and_grads():
-    # BASELINE config 1: B=2, H=4, T=512, d=64, fp32, N(0,1), scale 1/sqrt(64)
+    # benchmark configuration 1: B=2, H=4, T=512, d=64, fp32, N(0,1), scale 1/sqrt(64)
     _check_dense(2, 4, 512, 64, torch.float32, seed=0)
 
 
@@ -252,7 +252,7 @@ def test_forward_is_bitwise_repeatable():
 
 
 def test_row_mass_invariant_at_config2_size():
-    # full size of BASELINE config 2 (T=4096, H=16, d=64, bf16): size-independent properties
+    # full size of benchmark configuration 2 (T=4096, H=16, d=64, bf16): size-independent properties
     # instead of the O(T^2)-memory oracle: with v = ones, o_i = sum_j A_ij = 1 - rem_i
     sb_attn, _ = _ops()
     B, H, T, D = 1, 16, 4096, 64
@@ -425,7 +425,7 @@ def test_gradient_of_rem_alone(D, rep):
 
 
 def _full_size_properties(fwd_bwd, v_shape_like, check_docs=None):
-    """Size-independent properties of a forward+backward at a full BASELINE size (no O(T^2)
+    """Size-independent properties of a forward+backward at a full benchmark size (no O(T^2)
     oracle needed): the backward is linear in the upstream gradients and bit-reproducible,
     and every result is finite."""
     do1, do2, dr1, dr2 = v_shape_like
@@ -441,7 +441,7 @@ def _full_size_properties(fwd_bwd, v_shape_like, check_docs=None):
 
 
 def test_config3_size_packed_invariants():
-    # full size of BASELINE config 3: 65536 packed tokens, H=16, d=64, bf16, log-normal documents
+    # full size of benchmark configuration 3: 65536 packed tokens, H=16, d=64, bf16, log-normal documents
     _, sb_attn_varlen = _ops()
     H, N, D = 16, 65536, 64
     lens = lognormal_lengths(N, seed=0)
@@ -472,7 +472,7 @@ def test_config3_size_packed_invariants():
 
 
 def test_config4_size_invariants():
-    # full size of BASELINE config 4: B=1, H=16, T=16384, d=128, bf16
+    # full size of benchmark configuration 4: B=1, H=16, T=16384, d=128, bf16
     sb_attn, _ = _ops()
     B, H, T, D = 1, 16, 16384, 128
     q, k = (randn((B, H, T, D), 150 + i, 0.5, torch.bfloat16).cuda() for i in range(2))

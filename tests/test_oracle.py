@@ -185,7 +185,7 @@ def test_attend_current_relation_to_strict():
 
 
 def test_config1_shape_fp32_matches_fp64():
-    # BASELINE config 1 (B=2,H=4,T=512,d=64, N(0,1), scale 1/8): the fp32 oracle that the
+    # benchmark configuration 1 (B=2,H=4,T=512,d=64, N(0,1), scale 1/8): the fp32 oracle that the
     # 1e-4 GPU tolerance is measured against is itself within 1e-5 of float64
     q, k, v = (randn((2, 4, 512, 64), s) for s in (0, 1, 2))
     o32, r32 = O.sb_attn_oracle(q, k, v)
