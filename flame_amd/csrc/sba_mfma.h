@@ -294,8 +294,10 @@ __device__ inline f32x16 mfma(bf16x8 a, bf16x8 b, f32x16 c) {
 template <int D>
 __device__ inline void score_raw_o(f32x16 (&raw)[2], const char* ktile, const LaneOffsets<D>& o,
                                    const bf16x8 (&qf)[D / 16]) {
+    // tile 1 first: the product chain starts at its keys (the right half of the lane's 32), and
+    // can begin while the MFMAs of tile 0 are still in flight
 #pragma unroll
-    for (int t = 0; t < 2; ++t) {
+    for (int t = 1; t >= 0; --t) {
         f32x16 acc = {0};
 #pragma unroll
         for (int ks = 0; ks < D / 16; ++ks) acc = mfma(fetch_rows_o<D>(ktile, o, t, ks), qf[ks], acc);
