@@ -1051,10 +1051,15 @@ __global__ __launch_bounds__(kThreads, D == 64 ? 2 : 1) void mfma_bwd_dkv_own_ke
                 const float Gt = sees_wave ? Gin[t] : 0.0f;
                 float x[16], beta[16], dp[16];
                 {
+                    // with one wave on the SIMD (d = 128) nothing hides an LDS round trip in front of
+                    // each MFMA: all operands of the tile are requested first
+                    bf16x8 bq[D / 16];
+#pragma unroll
+                    for (int ks = 0; ks < D / 16; ++ks) bq[ks] = fetch_row_nat<D>(qtile, 32 * t + n, ks, lane);
+                    if (D == 128) __builtin_amdgcn_sched_barrier(0);
                     f32x16 acc = {0};
 #pragma unroll
-                    for (int ks = 0; ks < D / 16; ++ks)
-                        acc = mfma(kfr[ks], fetch_row_nat<D>(qtile, 32 * t + n, ks, lane), acc);
+                    for (int ks = 0; ks < D / 16; ++ks) acc = mfma(kfr[ks], bq[ks], acc);
 #pragma unroll
                     for (int r = 0; r < 16; ++r) x[r] = acc[r] * p.scale2;
                 }
@@ -1116,10 +1121,13 @@ __global__ __launch_bounds__(kThreads, D == 64 ? 2 : 1) void mfma_bwd_dkv_own_ke
                     });
                 }
                 {
+                    bf16x8 bd[D / 16];
+#pragma unroll
+                    for (int ks = 0; ks < D / 16; ++ks) bd[ks] = fetch_row_nat<D>(dotile, 32 * t + n, ks, lane);
+                    if (D == 128) __builtin_amdgcn_sched_barrier(0);
                     f32x16 acc = {0};
 #pragma unroll
-                    for (int ks = 0; ks < D / 16; ++ks)
-                        acc = mfma(vfr[ks], fetch_row_nat<D>(dotile, 32 * t + n, ks, lane), acc);
+                    for (int ks = 0; ks < D / 16; ++ks) acc = mfma(vfr[ks], bd[ks], acc);
 #pragma unroll
                     for (int r = 0; r < 16; ++r) dp[r] = acc[r];
                 }
