@@ -298,9 +298,15 @@ __device__ inline void score_raw_o(f32x16 (&raw)[2], const char* ktile, const La
     // can begin while the MFMAs of tile 0 are still in flight
 #pragma unroll
     for (int t = 1; t >= 0; --t) {
+        // all operands of the tile are requested before its first MFMA: at head_dim 128 the kernels
+        // run one or two waves per SIMD, and nothing else hides an LDS round trip per MFMA
+        bf16x8 a[D / 16];
+#pragma unroll
+        for (int ks = 0; ks < D / 16; ++ks) a[ks] = fetch_rows_o<D>(ktile, o, t, ks);
+        if (D == 128) __builtin_amdgcn_sched_barrier(0);
         f32x16 acc = {0};
 #pragma unroll
-        for (int ks = 0; ks < D / 16; ++ks) acc = mfma(fetch_rows_o<D>(ktile, o, t, ks), qf[ks], acc);
+        for (int ks = 0; ks < D / 16; ++ks) acc = mfma(a[ks], qf[ks], acc);
         raw[t] = acc;
     }
 }

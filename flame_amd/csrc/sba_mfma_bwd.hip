@@ -129,10 +129,14 @@ mask_step(x, key0 + 32 * h, qi, strict);
 #pragma unroll
             for (int c = 0; c < 4; ++c) zf[c] = pack8(&dp[8 * c]);
 #pragma unroll
-            for (int db = 0; db < D / 32; ++db)
+            for (int c = 0; c < 4; ++c) {      // (operands of a key group requested together, see score_raw_o)
+                bf16x8 kt[D / 32];
 #pragma unroll
-                for (int c = 0; c < 4; ++c)
-                    dqacc[db] = mfma(fetch_cols_o<D>(ktile, lo, db, c), zf[c], dqacc[db]);
+                for (int db = 0; db < D / 32; ++db) kt[db] = fetch_cols_o<D>(ktile, lo, db, c);
+                if (D == 128) __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int db = 0; db < D / 32; ++db) dqacc[db] = mfma(kt[db], zf[c], dqacc[db]);
+            }
         }
         wait_global_memory();                  // the next tiles have landed
         __syncthreads();

@@ -80,11 +80,23 @@ mask_step(x, key0 + 32 * h, qi, strict);
                 bf16x8 pf[4];
 #pragma unroll
                 for (int c = 0; c < 4; ++c) pf[c] = pack8(&x[8 * c]);
+                if (D == 128) {
 #pragma unroll
-                for (int db = 0; db < D / 32; ++db)
+                    for (int c = 0; c < 4; ++c) {      // (operands of a key group requested together, see score_raw_o)
+                        bf16x8 vt[D / 32];
 #pragma unroll
-                    for (int c = 0; c < 4; ++c)
-                        oacc[db] = mfma(fetch_cols_o<D>(vtile, lo, db, c), pf[c], oacc[db]);
+                        for (int db = 0; db < D / 32; ++db) vt[db] = fetch_cols_o<D>(vtile, lo, db, c);
+                        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                        for (int db = 0; db < D / 32; ++db) oacc[db] = mfma(vt[db], pf[c], oacc[db]);
+                    }
+                } else {
+#pragma unroll
+                    for (int db = 0; db < D / 32; ++db)
+#pragma unroll
+                        for (int c = 0; c < 4; ++c)
+                            oacc[db] = mfma(fetch_cols_o<D>(vtile, lo, db, c), pf[c], oacc[db]);
+                }
             }
         }
         wait_global_memory();                  // the next tiles have landed
