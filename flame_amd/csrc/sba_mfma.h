@@ -291,7 +291,7 @@ __device__ inline f32x16 mfma(bf16x8 a, bf16x8 b, f32x16 c) {
 // S^T tile pair for one wave, raw MFMA accumulators (no vector-ALU instruction touches
 // them here, so the matrix cores run ahead of whatever vector work follows):
 // raw[t][r] = (K Q^T)[key_local = 32h + 16t + r][query n].
-template <int D>
+template <int D, bool kBatch = (D == 128)>
 __device__ inline void score_raw_o(f32x16 (&raw)[2], const char* ktile, const LaneOffsets<D>& o,
                                    const bf16x8 (&qf)[D / 16]) {
     // tile 1 first: the product chain starts at its keys (the right half of the lane's 32), and
@@ -303,7 +303,7 @@ __device__ inline void score_raw_o(f32x16 (&raw)[2], const char* ktile, const La
         bf16x8 a[D / 16];
 #pragma unroll
         for (int ks = 0; ks < D / 16; ++ks) a[ks] = fetch_rows_o<D>(ktile, o, t, ks);
-        if (D == 128) __builtin_amdgcn_sched_barrier(0);
+        if (kBatch) __builtin_amdgcn_sched_barrier(0);
         f32x16 acc = {0};
 #pragma unroll
         for (int ks = 0; ks < D / 16; ++ks) acc = mfma(a[ks], qf[ks], acc);
@@ -319,11 +319,11 @@ __device__ inline void scale_scores(float (&x)[32], const f32x16 (&raw)[2], floa
         for (int r = 0; r < 16; ++r) x[16 * t + r] = raw[t][r] * scale2;
 }
 
-template <int D>
+template <int D, bool kBatch = (D == 128)>
 __device__ inline void score_tiles_o(float (&x)[32], const char* ktile, const LaneOffsets<D>& o,
                                      const bf16x8 (&qf)[D / 16], float scale2) {
     f32x16 raw[2];
-    score_raw_o<D>(raw, ktile, o, qf);
+    score_raw_o<D, kBatch>(raw, ktile, o, qf);
     scale_scores(x, raw, scale2);
 }
 

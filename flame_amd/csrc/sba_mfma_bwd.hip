@@ -253,7 +253,7 @@ __global__ __launch_bounds__(2 * kThreads, 2) void mfma_bwd_dq2_kernel(KParams p
         float x[32], beta[32], dp[32];
         float total = 0.f, start = 0.f, Rlane = 1.f;
         if (active) {
-            score_tiles_o<D>(x, ktile, lo, qf, p.scale2);
+            score_tiles_o<D, true>(x, ktile, lo, qf, p.scale2);
             if (key0 + 63 + strict > q0w) mask_step(x, key0 + 32 * h, qi, strict);
             float Rc = R;
             stick_weights_and_dp<D>(x, beta, dp, Rc, lane, &Rlane, vtile, lo, dof);

@@ -197,7 +197,7 @@ __global__ __launch_bounds__(2 * kThreads) void mfma_fwd2_kernel(KParams p) {
         float x[32];
         float total = 1.0f, fac = 1.0f;
         if (active) {
-            score_tiles_o<D>(x, ktile, lo, qf, p.scale2);
+            score_tiles_o<D, true>(x, ktile, lo, qf, p.scale2);
             if (key0 + 63 + strict > q0w) mask_step(x, key0 + 32 * h, qi, strict);
             float dummy[1];
             fac = stick_weights_local<false>(x, dummy, total, lane);
