@@ -218,10 +218,18 @@ __global__ __launch_bounds__(2 * kThreads) void mfma_fwd2_kernel(KParams p) {
 #pragma unroll
                 for (int c = 0; c < 4; ++c) pf[c] = pack8(&x[8 * c]);
 #pragma unroll
-                for (int db = 0; db < D / 32; ++db)
+                for (int c2 = 0; c2 < 2; ++c2) {   // operands of two key groups requested together, ahead of their MFMAs
+                    bf16x8 vt[2][D / 32];
 #pragma unroll
-                    for (int c = 0; c < 4; ++c)
-                        oacc[db] = mfma(fetch_cols_o<D>(vtile, lo, db, c), pf[c], oacc[db]);
+                    for (int cc = 0; cc < 2; ++cc)
+#pragma unroll
+                        for (int db = 0; db < D / 32; ++db) vt[cc][db] = fetch_cols_o<D>(vtile, lo, db, 2 * c2 + cc);
+                    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                    for (int cc = 0; cc < 2; ++cc)
+#pragma unroll
+                        for (int db = 0; db < D / 32; ++db) oacc[db] = mfma(vt[cc][db], pf[2 * c2 + cc], oacc[db]);
+                }
             }
         }
         wait_global_memory();                  // the next tiles have landed
