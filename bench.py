@@ -22,9 +22,9 @@ KERNEL_TIMING_SAMPLES = 5      # steps of the timed region whose kernels are tim
 # HBM bytes per launch (read + write) from the rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs
 # summarised in profiles/sba_cfg{2,3,4}_hbm_traffic.txt (counters cannot be read from inside this
 # process).
-PROFILED_HBM_BYTES = {("cfg2", "fwd"): 42339740, ("cfg2", "bwd_dq"): 62702723, ("cfg2", "bwd_dkv"): 68208530,
-                      ("cfg3", "fwd"): 892244515, ("cfg3", "bwd_dq"): 994203036, ("cfg3", "bwd_dkv"): 1127833918,
-                      ("cfg4", "fwd"): 751723244, ("cfg4", "bwd_dq"): 1344916197, ("cfg4", "bwd_dkv"): 1400281853}
+PROFILED_HBM_BYTES = {("cfg2", "fwd"): 42339781, ("cfg2", "bwd_dq"): 62778117, ("cfg2", "bwd_dkv"): 68197370,
+                      ("cfg3", "fwd"): 888532081, ("cfg3", "bwd_dq"): 992826534, ("cfg3", "bwd_dkv"): 1127845107,
+                      ("cfg4", "fwd"): 758484392, ("cfg4", "bwd_dq"): 1344916988, ("cfg4", "bwd_dkv"): 1401200275}
 
 
 def _lognormal_lengths(total, seed, median=600.0, sigma=1.0, lo=16, hi=4096):
