@@ -699,10 +699,6 @@ __global__ __launch_bounds__(2 * kThreads, 2) void mfma_bwd_dkv_stream_kernel(KP
         // row's banks: rows r and r + 2 do (r and r + 1 would collide), hence the order 0 2 1 3 ...
         const int crow4 = lane >> 2;
         const int crow = (crow4 & ~3) | ((crow4 & 1) << 1) | ((crow4 >> 1) & 1), cch = 4 * dbw + (lane & 3);
-        // The tile requests of a step are issued two at a time between the MFMAs of the
-        // reduction: all CUs stream their tiles from L2 in the same phase of a step, the
-        // memory pipe then accepts about one 1 KB wave load per 80 cycles, and a burst of
-        // eight would stall this wave on a full queue.
         // Per-item base pointers, worked out once per item and held in VECTOR registers (which
         // the consumers have to spare): a step's requests then cost a few vector instructions.
         // Left to itself the compiler keeps such uniform values in scalar registers, runs out
@@ -787,7 +783,7 @@ __global__ __launch_bounds__(2 * kThreads, 2) void mfma_bwd_dkv_stream_kernel(KP
         // The operands of four 16-query groups are fetched as one batch, so that the MFMAs wait
         // for LDS once per batch rather than once each; `between(b)` (the tile requests) goes
         // behind the fetches of batch b.
-        auto reduce = [&](int s_done, auto&& between) {
+        auto reduce = [&](int s_done) {
             const char* zt = bufs + (s_done & 1) * kBuf + (is_dv ? 0 : kZTile);            // a or dz
             const char* xt = bufs + (s_done & 1) * kBuf + 2 * kZTile + (is_dv ? kQTile : 0); // dO or Q
 #pragma unroll
@@ -800,7 +796,6 @@ __global__ __launch_bounds__(2 * kThreads, 2) void mfma_bwd_dkv_stream_kernel(KP
                     aw[j][1] = fetch_nat_2<64>(zt, za[1][0], za[1][1], 16 * c2);
                     bx[j] = fetch_nat_2<D>(xt, qb0o, qb1o, 16 * c2);
                 }
-                between(b);
 #pragma unroll
                 for (int j = 0; j < 4; ++j) {
                     acc[0] = mfma(aw[j][0], bx[j], acc[0]);
@@ -841,13 +836,14 @@ __global__ __launch_bounds__(2 * kThreads, 2) void mfma_bwd_dkv_stream_kernel(KP
                 store_pending = false;
                 __syncthreads();               // X: the producers may overwrite the staging
             }
+            // The next step's carries and tiles are requested in one go ahead of the reduction: the
+            // answers are only needed at this iteration's deposit, a whole reduction away.  (Spread
+            // between the reduction's MFMAs, as an earlier version had them, the last requests were
+            // still in flight when the deposit came: 4 % of the kernel.)
             request_carry(rq, rq_row0);
-            if (s > 0) {
-                reduce(s - 1, [&](int b) { request_tile(rq, rq_row0, 2 * b); request_tile(rq, rq_row0, 2 * b + 1); });
-            } else {
 #pragma unroll
-                for (int part = 0; part < 4; ++part) request_tile(rq, rq_row0, part);
-            }
+            for (int part = 0; part < 4; ++part) request_tile(rq, rq_row0, part);
+            if (s > 0) reduce(s - 1);
             // B, only where a finished dK/dV is staged into the Z buffer just reduced: every
             // consumer must be through with it
             if (finish_after_reduce) consumer_sync();
@@ -894,7 +890,7 @@ __global__ __launch_bounds__(2 * kThreads, 2) void mfma_bwd_dkv_stream_kernel(KP
         }
         // draining iteration: the last step of the last item
         if (store_pending) store_staged(fin_store, bufs + (s & 1) * kBuf);
-        reduce(s - 1, [&](int) {});
+        reduce(s - 1);
         consumer_sync();                       // B
         stage(bufs + ((s - 1) & 1) * kBuf);
         __syncthreads();                       // A (consumers only need each other's staging)
