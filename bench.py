@@ -22,9 +22,9 @@ KERNEL_TIMING_SAMPLES = 5      # steps of the timed region whose kernels are tim
 # HBM bytes per launch (read + write) from the rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs
 # summarised in profiles/sba_cfg{2,3,4}_hbm_traffic.txt (counters cannot be read from inside this
 # process).
-PROFILED_HBM_BYTES = {("cfg2", "fwd"): 42339781, ("cfg2", "bwd_dq"): 62778117, ("cfg2", "bwd_dkv"): 68197370,
-                      ("cfg3", "fwd"): 888532081, ("cfg3", "bwd_dq"): 992826534, ("cfg3", "bwd_dkv"): 1127845107,
-                      ("cfg4", "fwd"): 758484392, ("cfg4", "bwd_dq"): 1344916988, ("cfg4", "bwd_dkv"): 1401200275}
+PROFILED_HBM_BYTES = {("cfg2", "fwd"): 42339771, ("cfg2", "bwd_dq"): 63414370, ("cfg2", "bwd_dkv"): 68069661,
+                      ("cfg3", "fwd"): 865755241, ("cfg3", "bwd_dq"): 990492784, ("cfg3", "bwd_dkv"): 1126127762,
+                      ("cfg4", "fwd"): 754136986, ("cfg4", "bwd_dq"): 1344713737, ("cfg4", "bwd_dkv"): 1401608381}
 
 
 def _lognormal_lengths(total, seed, median=600.0, sigma=1.0, lo=16, hi=4096):
