@@ -73,6 +73,8 @@ def load() -> C.CDLL:
         lib.sba_fwd.argtypes = [C.POINTER(SbaParams)]
         lib.sba_bwd.restype = C.c_int
         lib.sba_bwd.argtypes = [C.POINTER(SbaParams)]
+        lib.sba_bwd_static.restype = C.c_int
+        lib.sba_bwd_static.argtypes = [C.POINTER(SbaParams)]
         if lib.sba_abi_version() != SBA_ABI_VERSION:
             raise RuntimeError("libsba_mi355x.so ABI version mismatch; rebuild it")
         _lib = lib
@@ -80,7 +82,9 @@ def load() -> C.CDLL:
 
 
 EXPORTED_SYMBOLS = ("sba_abi_version", "sba_error_string", "sba_workspace_bytes", "sba_bwd_scratch_bytes",
-                    "sba_build_schedule", "sba_row_block", "sba_fwd", "sba_bwd")
+                    "sba_build_schedule", "sba_row_block", "sba_fwd", "sba_bwd", "sba_bwd_static")
+
+STATIC_SCRATCH_BYTES = 64 << 20     # SBA_STATIC_SCRATCH_BYTES: what sba_bwd_static() holds per GPU
 
 
 def check(rc: int, what: str) -> None:

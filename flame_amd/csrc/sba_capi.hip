@@ -5,7 +5,13 @@
 #include <algorithm>
 #include <cstdlib>
 #include <cstring>
+#include <mutex>
 #include <vector>
+
+// Backward scratch of sba_bwd_static(): one array per GPU that loads this library, held until
+// the process ends.  In host code this name is only a handle of the symbol, never a device
+// address: the address on a given GPU comes from hipGetSymbolAddress (static_scratch() below).
+static __device__ __align__(256) unsigned char scratch[SBA_STATIC_SCRATCH_BYTES];
 
 namespace {
 
@@ -85,16 +91,34 @@ KParams make_kparams(const SbaParams* p) {
     kp.n_kb = n_key_blocks(p);
     kp.tab_tokens = tab_tokens(p);
     if (p->workspace && use_mfma(p)) kp.rtab = (float*)p->workspace;
-    char* scratch = (char*)p->bwd_scratch;
-    if (scratch && use_mfma_bwd(p)) {
-        kp.gtab = (float*)scratch;
-        kp.rmid = (float*)(scratch + table_bytes(p));
-        kp.gmid = (float*)(scratch + 2 * table_bytes(p));
-        if (!p->workspace) kp.rtab = (float*)(scratch + 3 * table_bytes(p));   // recomputed by sba_bwd
-    } else if (scratch) {
-        kp.dkv32 = (float*)scratch;
+    char* bs = (char*)p->bwd_scratch;
+    if (bs && use_mfma_bwd(p)) {
+        kp.gtab = (float*)bs;
+        kp.rmid = (float*)(bs + table_bytes(p));
+        kp.gmid = (float*)(bs + 2 * table_bytes(p));
+        if (!p->workspace) kp.rtab = (float*)(bs + 3 * table_bytes(p));   // recomputed by sba_bwd
+    } else if (bs) {
+        kp.dkv32 = (float*)bs;
     }
     return kp;
+}
+
+// Device address of the static scratch array on the CURRENT device: asked once per device
+// (every GPU holds its own copy of the array at its own address) and kept.
+int static_scratch(void** out) {
+    constexpr int kMaxDevices = 64;
+    static void* ptrs[kMaxDevices] = {nullptr};
+    static std::mutex mu;
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return SBA_ERR_LAUNCH;
+    std::lock_guard<std::mutex> lock(mu);
+    if (!ptrs[dev]) {
+        void* ptr = nullptr;
+        if (hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)) != hipSuccess || !ptr) return SBA_ERR_LAUNCH;
+        ptrs[dev] = ptr;
+    }
+    *out = ptrs[dev];
+    return SBA_OK;
 }
 
 }  // namespace
@@ -113,6 +137,7 @@ const char* sba_error_string(int code) {
         case SBA_ERR_SCHEDULE: return "packed layout needs a row-block schedule from sba_build_schedule()";
         case SBA_ERR_LAUNCH: return "kernel launch failed";
         case SBA_ERR_ABI: return "SbaParams.struct_size does not match this library";
+        case SBA_ERR_STATIC_LIMIT: return "problem needs more backward scratch than sba_bwd_static() holds (SBA_STATIC_SCRATCH_BYTES); use sba_bwd() with a caller-allocated bwd_scratch";
         default: return "unknown error";
     }
 }
@@ -206,6 +231,21 @@ int sba_bwd(const SbaParams* p) {
     // the generic backward is one piece: it all runs in phase 1
     if (!use_mfma_bwd(p) && p->bwd_phases == 2) return SBA_OK;
     return use_mfma_bwd(p) ? sba_launch_mfma_bwd(kp, p->bwd_phases, s) : sba_launch_generic_bwd(kp, p->dtype, s);
+}
+
+int sba_bwd_static(const SbaParams* p) {
+    int rc = check_common(p);
+    if (rc) return rc;
+    if (sba_bwd_scratch_bytes(p) > (size_t)SBA_STATIC_SCRATCH_BYTES) return SBA_ERR_STATIC_LIMIT;
+    void* ptr = nullptr;
+    rc = static_scratch(&ptr);
+    if (rc) return rc;
+    // Nothing in the array has to start at zero: the matrix-core kernels write every table entry
+    // before they read it, and the generic path clears its accumulators with a fill kernel.
+    SbaParams q = *p;
+    q.bwd_scratch = ptr;
+    q.bwd_scratch_bytes = SBA_STATIC_SCRATCH_BYTES;
+    return sba_bwd(&q);
 }
 
 }  // extern "C"

@@ -48,7 +48,8 @@ enum {
     SBA_ERR_WORKSPACE = -4,   /* workspace or bwd_scratch missing or too small */
     SBA_ERR_SCHEDULE = -5,    /* packed layout without a row-block schedule */
     SBA_ERR_LAUNCH = -6,      /* hipGetLastError() after a launch was not hipSuccess */
-    SBA_ERR_ABI = -7          /* struct_size does not match this library */
+    SBA_ERR_ABI = -7,         /* struct_size does not match this library */
+    SBA_ERR_STATIC_LIMIT = -8 /* sba_bwd_static(): the problem needs more scratch than the library holds */
 };
 
 /* One tensor of q/k/v/o/do/dq/dk/dv shape. */
@@ -153,6 +154,22 @@ int sba_fwd(const SbaParams* p);
 
 /* Backward: dq, dk, dv from d_o, d_rem, q, k, v and the forward's carry table. */
 int sba_bwd(const SbaParams* p);
+
+/*
+ * Backward without any allocation.  No counterpart in the reference: it is for callers that
+ * cannot allocate device memory around the call (code under HIP graph capture, tight serving
+ * loops, harnesses that forbid hipMalloc).  Same contract as sba_bwd(), except that
+ * p->bwd_scratch / p->bwd_scratch_bytes are ignored: the scratch is an array of
+ * SBA_STATIC_SCRATCH_BYTES that the library itself holds on every GPU it runs on, until the
+ * process ends.  Problems with sba_bwd_scratch_bytes(p) above that limit are refused with
+ * SBA_ERR_STATIC_LIMIT and nothing is launched.  The call allocates nothing and frees nothing;
+ * the very first call on a device looks up the array's address there (make one call before a
+ * graph capture starts).  All calls on one GPU share the one array, which keeps the previous
+ * call's contents: calls that overlap on the same GPU (different streams or threads) race and
+ * must be serialised by the caller; calls on different GPUs are independent.
+ */
+#define SBA_STATIC_SCRATCH_BYTES (64u << 20)
+int sba_bwd_static(const SbaParams* p);
 
 #ifdef __cplusplus
 }

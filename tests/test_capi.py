@@ -68,6 +68,20 @@ def test_workspace_bytes(lib):
     assert lib.sba_bwd_scratch_bytes(C.byref(p)) == 2 * 4096 * 16 * 64 * 4
 
 
+def test_static_backward_refuses_oversize_without_gpu(lib):
+    # the size check of sba_bwd_static() comes before anything touches a GPU
+    p = _lib.SbaParams()
+    p.struct_size = C.sizeof(_lib.SbaParams)
+    p.dtype = _lib.SBA_DTYPE_BF16
+    p.n_seq, p.n_heads, p.seq_len, p.total_tokens, p.head_dim = 1, 16, 16384, 16384, 128
+    for t in ("q", "k", "v", "d_o", "dq", "dk", "dv"):
+        getattr(p, t).ptr = 256                     # never dereferenced
+    p.workspace = 256
+    assert lib.sba_bwd_scratch_bytes(C.byref(p)) > _lib.STATIC_SCRATCH_BYTES
+    assert lib.sba_bwd_static(C.byref(p)) == -8
+    assert b"sba_bwd_static" in lib.sba_error_string(-8)
+
+
 def test_schedule_builder(lib):
     cu = torch.tensor([0, 100, 400, 401, 1000, 1000], dtype=torch.int32)   # last doc empty
     s = _lib.build_schedule(cu)
