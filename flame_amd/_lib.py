@@ -15,7 +15,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "csrc", "libsba_mi355x.so")
 
 SBA_DTYPE_F32, SBA_DTYPE_BF16 = 0, 1
-SBA_ABI_VERSION = 4
+SBA_ABI_VERSION = 5
 
 
 class SbaTensor(C.Structure):
@@ -34,6 +34,7 @@ class SbaParams(C.Structure):
         ("head_dim", C.c_int32), ("attend_current", C.c_int32), ("scale", C.c_float),
         ("save_for_backward", C.c_int32), ("bwd_phases", C.c_int32),
         ("cu_seqlens", C.c_void_p), ("schedule", C.c_void_p), ("n_schedule", C.c_int32),
+        ("table_cols", C.c_int64),
         ("q", SbaTensor), ("k", SbaTensor), ("v", SbaTensor), ("o", SbaTensor),
         ("rem", SbaVector), ("d_o", SbaTensor), ("d_rem", SbaVector),
         ("dq", SbaTensor), ("dk", SbaTensor), ("dv", SbaTensor),
@@ -69,6 +70,8 @@ def load() -> C.CDLL:
         lib.sba_build_schedule.restype = C.c_int
         lib.sba_build_schedule.argtypes = [C.POINTER(C.c_int32), C.c_int, C.c_int, C.POINTER(C.c_int32), C.c_int]
         lib.sba_row_block.restype = C.c_int
+        lib.sba_table_columns.restype = C.c_int64
+        lib.sba_table_columns.argtypes = [C.POINTER(C.c_int32), C.c_int]
         lib.sba_fwd.restype = C.c_int
         lib.sba_fwd.argtypes = [C.POINTER(SbaParams)]
         lib.sba_bwd.restype = C.c_int
@@ -82,7 +85,8 @@ def load() -> C.CDLL:
 
 
 EXPORTED_SYMBOLS = ("sba_abi_version", "sba_error_string", "sba_workspace_bytes", "sba_bwd_scratch_bytes",
-                    "sba_build_schedule", "sba_row_block", "sba_fwd", "sba_bwd", "sba_bwd_static")
+                    "sba_build_schedule", "sba_row_block", "sba_table_columns", "sba_fwd", "sba_bwd",
+                    "sba_bwd_static")
 
 STATIC_SCRATCH_BYTES = 64 << 20     # SBA_STATIC_SCRATCH_BYTES: what sba_bwd_static() holds per GPU
 
@@ -98,6 +102,15 @@ def dtype_code(dt: torch.dtype) -> int:
     if dt == torch.bfloat16:
         return SBA_DTYPE_BF16
     raise TypeError(f"stick-breaking attention supports float32 and bfloat16, got {dt}")
+
+
+def check_supported(q: torch.Tensor) -> None:
+    """Say up front what the kernels do not cover instead of failing inside the library."""
+    if q.dtype not in (torch.float32, torch.bfloat16):
+        raise TypeError(f"stick-breaking attention supports float32 and bfloat16, got {q.dtype} "
+                        "(float16 is not offered)")
+    if q.shape[-1] > 128:
+        raise ValueError(f"head_dim {q.shape[-1]} is not supported (at most 128)")
 
 
 def tensor4(t: torch.Tensor) -> SbaTensor:
@@ -147,7 +160,7 @@ def cut_head_dim(t: torch.Tensor, D: int) -> torch.Tensor:
     return t if t.shape[-1] == D else t[..., :D].contiguous()
 
 
-SCHEDULE_INTS = 8      # int32 per row: {first_token, doc_len, row_block, doc_index} of job i, then of the i-th job in key-owner order
+SCHEDULE_INTS = 8      # int32 per row: {first_token, doc_len, row_block, first table column of the document} of job i, then of the i-th job in key-owner order
 
 
 DOC_MAJOR_GRID = 8192  # workgroups (jobs x heads) from which the schedule is document-major
@@ -167,18 +180,32 @@ def build_schedule(cu_host: torch.Tensor, n_heads: int = 0) -> torch.Tensor:
     return out[:n]
 
 
-def workspace_upper_bound(n_heads: int, seq_len: int, tab_tokens: int, head_dim: int) -> int:
-    """Pure-Python bounds on sba_workspace_bytes() (one carry table) and sba_bwd_scratch_bytes()
-    (three more tables, or the generic path's fp32 accumulators), usable while torch.compile
-    traces, where no ctypes call can be made.  Always >= what the library asks for."""
-    return _table_bound(n_heads, seq_len, tab_tokens)
+def table_columns(cu_host: torch.Tensor) -> int:
+    """Carry-table columns (of 128 floats, per head) of a packed batch: SbaParams.table_cols."""
+    cu = cu_host.to(torch.int32).contiguous()
+    return int(load().sba_table_columns(C.cast(cu.data_ptr(), C.POINTER(C.c_int32)), cu.numel() - 1))
 
 
-def bwd_scratch_upper_bound(n_heads: int, seq_len: int, tab_tokens: int, head_dim: int) -> int:
+# Pure-Python bounds on the library's sizes, usable while torch.compile traces (no ctypes call,
+# no look at cu_seqlens' values there).  Always >= what the library asks for.
+def dense_columns(n_seq: int, seq_len: int) -> int:
+    n = (seq_len + 127) // 128
+    return n_seq * n * (n + 1)
+
+
+def packed_columns_bound(total_tokens: int, n_docs: int, max_len: int) -> int:
+    """sum over documents of n*(n+1) <= (n_max + 1) * sum n <= (n_max + 1) * (tokens/128 + n_docs)."""
+    n_max = (max_len + 127) // 128
+    return (n_max + 1) * (total_tokens // 128 + n_docs)
+
+
+def workspace_upper_bound(n_heads: int, columns: int) -> int:
+    """One carry table (sba_workspace_bytes)."""
+    return (n_heads * columns * 128 * 4 + 255) & ~255
+
+
+def bwd_scratch_upper_bound(n_heads: int, columns: int, tab_tokens: int, head_dim: int) -> int:
+    """Four tables (the recompute mode's count) or the generic path's fp32 dk|dv accumulators."""
     dp = 32 if head_dim <= 32 else (64 if head_dim <= 64 else 128)
     acc = (2 * tab_tokens * n_heads * dp * 4 + 255) & ~255
-    return max(4 * _table_bound(n_heads, seq_len, tab_tokens), acc)     # four: also covers the recompute mode
-
-
-def _table_bound(n_heads: int, seq_len: int, tab_tokens: int) -> int:
-    return (n_heads * ((seq_len + 63) // 64) * tab_tokens * 4 + 255) & ~255
+    return max(4 * workspace_upper_bound(n_heads, columns), acc)

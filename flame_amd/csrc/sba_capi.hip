@@ -3,6 +3,7 @@
 #include "sba_common.h"
 
 #include <algorithm>
+#include <climits>
 #include <cstdlib>
 #include <cstring>
 #include <mutex>
@@ -41,10 +42,18 @@ int64_t tab_tokens(const SbaParams* p) {
     return p->cu_seqlens ? (int64_t)p->total_tokens : (int64_t)p->n_seq * p->seq_len;
 }
 
-int n_key_blocks(const SbaParams* p) { return (p->seq_len + sba::kKeyBlock - 1) / sba::kKeyBlock; }
-
+// Columns (128 floats) per head of one carry table: a sequence of n row blocks takes n*(n+1)
+// (row block qb holds the 2*qb + 2 key blocks it can see); the packed layout's total comes from
+// the caller (sba_table_columns() of the same cu_seqlens).
+int64_t columns_of(int64_t len) {
+    const int64_t n = (len + sba::kRowBlock - 1) / sba::kRowBlock;
+    return n * (n + 1);
+}
+int64_t table_columns(const SbaParams* p) {
+    return p->cu_seqlens ? p->table_cols : (int64_t)p->n_seq * columns_of(p->seq_len);
+}
 size_t table_bytes(const SbaParams* p) {
-    size_t b = (size_t)p->n_heads * n_key_blocks(p) * tab_tokens(p) * sizeof(float);
+    size_t b = (size_t)p->n_heads * (size_t)table_columns(p) * sba::kRowBlock * sizeof(float);
     return (b + 255) & ~(size_t)255;
 }
 
@@ -64,7 +73,7 @@ int check_common(const SbaParams* p) {
     if (p->head_dim <= 0 || p->head_dim > 128) return SBA_ERR_SHAPE;
     if (!p->q.ptr || !p->k.ptr || !p->v.ptr) return SBA_ERR_NULL;
     if (p->cu_seqlens) {
-        if (!p->schedule || p->n_schedule <= 0) return SBA_ERR_SCHEDULE;
+        if (!p->schedule || p->n_schedule <= 0 || p->table_cols <= 0) return SBA_ERR_SCHEDULE;
     } else if (p->total_tokens != p->seq_len) {
         return SBA_ERR_SHAPE;
     }
@@ -88,7 +97,7 @@ KParams make_kparams(const SbaParams* p) {
     kp.q = cvt(p->q); kp.k = cvt(p->k); kp.v = cvt(p->v); kp.o = cvt(p->o);
     kp.d_o = cvt(p->d_o); kp.dq = cvt(p->dq); kp.dk = cvt(p->dk); kp.dv = cvt(p->dv);
     kp.rem = cvt(p->rem); kp.d_rem = cvt(p->d_rem);
-    kp.n_kb = n_key_blocks(p);
+    kp.tab_head_stride = table_columns(p) * sba::kRowBlock;
     kp.tab_tokens = tab_tokens(p);
     if (p->workspace && use_mfma(p)) kp.rtab = (float*)p->workspace;
     char* bs = (char*)p->bwd_scratch;
@@ -144,26 +153,38 @@ const char* sba_error_string(int code) {
 
 size_t sba_workspace_bytes(const SbaParams* p) {
     if (!p || p->n_heads <= 0 || p->seq_len <= 0 || p->head_dim <= 0 || p->head_dim > 128) return 0;
+    if (p->cu_seqlens && p->table_cols <= 0) return 0;
     return use_mfma(p) ? table_bytes(p) : 0;
 }
 
 size_t sba_bwd_scratch_bytes(const SbaParams* p) {
     if (!p || p->n_heads <= 0 || p->seq_len <= 0 || p->head_dim <= 0 || p->head_dim > 128) return 0;
+    if (p->cu_seqlens && p->table_cols <= 0 && use_mfma_bwd(p)) return 0;
     // without a workspace the backward recomputes the forward's table first, into a fourth slot
     return use_mfma_bwd(p) ? (p->workspace ? 3 : 4) * table_bytes(p) : generic_acc_bytes(p);
 }
 
 int sba_row_block(void) { return sba::kRowBlock; }
 
+int64_t sba_table_columns(const int32_t* cu, int n_seq) {
+    if (!cu || n_seq <= 0) return 0;
+    int64_t cols = 0;
+    for (int s = 0; s < n_seq; ++s) cols += columns_of(std::max(cu[s + 1] - cu[s], 0));
+    return cols;
+}
+
 int sba_build_schedule(const int32_t* cu, int n_seq, int n_heads, int32_t* out, int capacity) {
     if (!cu || n_seq <= 0) return 0;
-    struct J { int32_t tok0, len, rb, doc; };
+    struct J { int32_t tok0, len, rb, doc, tab0; };
     std::vector<J> jobs;
+    int64_t cols = 0;                  // carry-table columns of the documents so far
     for (int s = 0; s < n_seq; ++s) {
         int32_t len = cu[s + 1] - cu[s];
         if (len <= 0) continue;
         int n_rb = (len + sba::kRowBlock - 1) / sba::kRowBlock;
-        for (int rb = 0; rb < n_rb; ++rb) jobs.push_back(J{cu[s], len, rb, s});
+        if (cols + columns_of(len) > INT32_MAX) return 0;       // tables of this size are out of reach anyway
+        for (int rb = 0; rb < n_rb; ++rb) jobs.push_back(J{cu[s], len, rb, s, (int32_t)cols});
+        cols += columns_of(len);
     }
     int n = (int)jobs.size();
     // Longest sweeps first; a stable order keeps the schedule deterministic.  Very large launches
@@ -191,8 +212,8 @@ int sba_build_schedule(const int32_t* cu, int n_seq, int n_heads, int32_t* out, 
         for (int i = 0; i < n; ++i) {
             int32_t* o = out + (size_t)sba::kScheduleInts * i;
             const J& k = jobs[key_order[i]];
-            o[0] = jobs[i].tok0; o[1] = jobs[i].len; o[2] = jobs[i].rb; o[3] = jobs[i].doc;
-            o[4] = k.tok0; o[5] = k.len; o[6] = k.rb; o[7] = k.doc;
+            o[0] = jobs[i].tok0; o[1] = jobs[i].len; o[2] = jobs[i].rb; o[3] = jobs[i].tab0;
+            o[4] = k.tok0; o[5] = k.len; o[6] = k.rb; o[7] = k.tab0;
         }
     }
     return n;

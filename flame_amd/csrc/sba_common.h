@@ -28,16 +28,17 @@ struct KParams {
     const int32_t* schedule;
     TensorArg q, k, v, o, d_o, dq, dk, dv;
     VectorArg rem, d_rem;
-    float* rtab;                   // forward carry table  [H][n_kb][total_tokens] (x n_seq for dense)
+    float* rtab;                   // forward carry table (layout: tab_index() below)
     float* gtab;                   // backward prefix table, same shape
     float* rmid;                   // the same two carries in the MIDDLE of each 64-key block (entering
     float* gmid;                   //   its left / right 32 keys), written by the dQ pass
     float* dkv32;                  // generic path: fp32 dk|dv accumulators
-    int n_kb;                      // carry-table columns = ceil(seq_len / kKeyBlock)
-    int64_t tab_tokens;            // tokens per head in the tables (n_seq*T dense, sumT packed)
+    int64_t tab_head_stride;       // floats per head in each carry table
+    int64_t tab_tokens;            // generic path: tokens per head in the fp32 accumulators (n_seq*T dense, sumT packed)
 };
 
-struct Job { int tok0, len, rb, seq; };
+// tab0: first carry-table column of the job's sequence
+struct Job { int tok0, len, rb, seq, tab0; };
 
 // Workgroup -> (job, head).  blockIdx.x = slot * n_heads + head, so that consecutive
 // workgroups (which the dispatcher deals round-robin to the 8 XCDs) are different heads of
@@ -50,8 +51,8 @@ __device__ inline int order_job(int slot, int n_jobs, bool longest_last) {
 
 // Dense jobs are generated arithmetically (row-blocks in decreasing order); packed jobs
 // come from the host-built schedule, which has the same order.  Row i of the schedule:
-// {first_token, doc_len, row_block, doc_index} of the i-th job, then the same four of the job
-// that comes i-th for the key-owner kernels.
+// {first_token, doc_len, row_block, first table column of the document} of the i-th job, then
+// the same four of the job that comes i-th for the key-owner kernels.
 constexpr int kScheduleInts = 8;
 
 // The schedule is read-only for the kernels and indexed with wave-uniform values: read it
@@ -69,6 +70,7 @@ __device__ inline Job dense_job(const KParams& p, int job) {
     j.seq = job % p.n_seq;
     j.tok0 = 0;
     j.len = p.seq_len;
+    j.tab0 = j.seq * n_rb * (n_rb + 1);
     return j;
 }
 
@@ -76,7 +78,7 @@ __device__ inline Job decode_job(const KParams& p, int job) {
     if (p.cu_seqlens == nullptr) return dense_job(p, job);
     const ScheduleRow s = schedule_row(p, job, 0);
     Job j;
-    j.tok0 = s[0]; j.len = s[1]; j.rb = s[2]; j.seq = 0;
+    j.tok0 = s[0]; j.len = s[1]; j.rb = s[2]; j.seq = 0; j.tab0 = s[3];
     return j;
 }
 
@@ -88,13 +90,24 @@ __device__ inline Job decode_key_job(const KParams& p, int i) {
     if (p.cu_seqlens == nullptr) return dense_job(p, p.n_jobs - 1 - i);
     const ScheduleRow s = schedule_row(p, i, 4);
     Job j;
-    j.tok0 = s[0]; j.len = s[1]; j.rb = s[2]; j.seq = 0;
+    j.tok0 = s[0]; j.len = s[1]; j.rb = s[2]; j.seq = 0; j.tab0 = s[3];
     return j;
 }
 
-// Token index inside the carry tables.
+// Token index inside the generic path's fp32 accumulators.
 __device__ inline int64_t tab_token(const KParams& p, const Job& j, int local) {
     return (p.cu_seqlens == nullptr) ? (int64_t)j.seq * p.seq_len + local : (int64_t)j.tok0 + local;
+}
+
+// Carry tables, compact layout: every sequence has one slab per 128-query row block qb that
+// holds exactly the 2*qb + 2 key blocks (64 keys each) that row block can see, as
+// [key block][128 queries] fp32.  The slabs of a sequence follow each other (row block qb
+// starts qb*(qb+1) columns into the sequence's part, a column being 128 floats), the sequences
+// follow each other (Job::tab0), heads are outermost.  A sequence of n row blocks takes
+// n*(n+1) columns: half of a full [key blocks][tokens] rectangle.
+// Returns the index of (row block qb, key block kb, query 0 of the row block).
+__device__ inline int64_t tab_index(const KParams& p, int head, const Job& j, int qb, int kb) {
+    return (int64_t)head * p.tab_head_stride + ((int64_t)j.tab0 + qb * (qb + 1) + kb) * kRowBlock;
 }
 
 __device__ inline float bf16_to_f32(uint16_t b) { return __uint_as_float(((uint32_t)b) << 16); }

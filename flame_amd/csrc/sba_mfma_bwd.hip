@@ -62,7 +62,6 @@ __global__ __launch_bounds__(kThreads) void mfma_bwd_dq_kernel(KParams p) {
     const int imax = min(m0 + kRowBlock - 1, job.len - 1);
     const int kmax = imax - strict;
     const int n_steps = kmax >= 0 ? kmax / kKeyBlock + 1 : 0;
-    const int64_t tabtok = tab_token(p, job, qi);
 
     TileDma<D> kc, vc;
     kc.init(lane, wave, p.k, kbase);
@@ -75,8 +74,8 @@ __global__ __launch_bounds__(kThreads) void mfma_bwd_dq_kernel(KParams p) {
     // carry-table traffic is kept off the critical path: the value of the NEXT step is loaded
     // while this one is computed, and this step's prefix is stored before the tile loads are
     // issued (vector memory operations retire in order)
-    const int64_t tstride = p.tab_tokens;
-    const int64_t tix0 = (int64_t)head * p.n_kb * p.tab_tokens + tabtok;
+    constexpr int64_t tstride = kRowBlock;
+    const int64_t tix0 = tab_index(p, head, job, job.rb, 0) + 32 * wave + n;
     float Rnext = (row_ok && n_steps > 0) ? p.rtab[tix0] : 1.0f;
     float* mid_table = h == 0 ? p.rmid : p.gmid;
     float mid = 0.f, Genter = 0.f;
@@ -212,7 +211,6 @@ __global__ __launch_bounds__(2 * kThreads, 2) void mfma_bwd_dq2_kernel(KParams p
     const int kmax = imax - strict;
     const int n_steps = kmax >= 0 ? kmax / kKeyBlock + 1 : 0;
     const int n_it = (n_steps + 1) / 2;
-    const int64_t tabtok = tab_token(p, job, qi);
     char* my_tiles = lds + grp * 2 * kTile;          // + buf * 4 * kTile
 
     // each group copies its own tiles (256 threads per tile pair)
@@ -225,8 +223,8 @@ __global__ __launch_bounds__(2 * kThreads, 2) void mfma_bwd_dq2_kernel(KParams p
     }
 
     // the forward's carry for this group's NEXT step is loaded while this one is computed
-    const int64_t tstride = p.tab_tokens;
-    const int64_t tix0 = (int64_t)head * p.n_kb * p.tab_tokens + tabtok;
+    constexpr int64_t tstride = kRowBlock;
+    const int64_t tix0 = tab_index(p, head, job, job.rb, 0) + 32 * qs + n;
     float Rnext = (row_ok && grp < n_steps) ? p.rtab[tix0 + grp * tstride] : 1.0f;
     float* mid_table = h == 0 ? p.rmid : p.gmid;
     float mid = 0.f;
@@ -367,7 +365,6 @@ __global__ __launch_bounds__(kThreads, 2) void mfma_bwd_dkv_kernel(KParams p) {
     const int64_t kbase = (int64_t)job.seq * p.k.sb + (int64_t)head * p.k.sh + (int64_t)job.tok0 * p.k.st;
     const int64_t vbase = (int64_t)job.seq * p.v.sb + (int64_t)head * p.v.sh + (int64_t)job.tok0 * p.v.st;
     const int64_t dobase = (int64_t)job.seq * p.d_o.sb + (int64_t)head * p.d_o.sh + (int64_t)job.tok0 * p.d_o.st;
-    const int64_t trow = ((int64_t)head * p.n_kb + kb) * p.tab_tokens;
     const int n_qb = (job.len + kRowBlock - 1) / kRowBlock;
     const int kh = wave & 1;                   // which 32 keys this wave reduces
     const int dbw = wave >> 1;                 // and which d-blocks: dbw + 2*i
@@ -396,7 +393,7 @@ __global__ __launch_bounds__(kThreads, 2) void mfma_bwd_dkv_kernel(KParams p) {
         const int qi0 = qb0 * kRowBlock + 32 * wave + n;
         load_row_frags<D>(qfn, p.q, qbase, qi0, job.len, lane);
         if (qi0 < job.len) {
-            const int64_t t = trow + tab_token(p, job, qi0);
+            const int64_t t = tab_index(p, head, job, qb0, kb) + 32 * wave + n;
             Rn = p.rtab[t]; Gn = p.gtab[t];
         }
     }
@@ -421,7 +418,7 @@ __global__ __launch_bounds__(kThreads, 2) void mfma_bwd_dkv_kernel(KParams p) {
             load_row_frags<D>(qfn, p.q, qbase, qin, job.len, lane);
             Rn = 1.0f; Gn = 0.0f;
             if (qin < job.len) {
-                const int64_t t = trow + tab_token(p, job, qin);
+                const int64_t t = tab_index(p, head, job, qb + 1, kb) + 32 * wave + n;
                 Rn = p.rtab[t]; Gn = p.gtab[t];
             }
         }
@@ -707,14 +704,14 @@ __global__ __launch_bounds__(2 * kThreads, 2) void mfma_bwd_dkv_stream_kernel(KP
         // the consumers' share of a step is short).
         struct ItemPtrs {
             const char* x;                     // Q or dO: row 0 of the sequence, this head, this thread's chunk
-            const float *rt, *gt;              // carries of this (head, key block), query 0
+            const float *rt, *gt;              // carries of this (head, key block): row block 0, query 0
             int row0, len;                     // first query of the item's sweep; sequence length
         };
         auto item_ptrs = [&](const KeyItem& t) {
             ItemPtrs r;
             const TensorArg& xt = is_dv ? p.d_o : p.q;
             r.x = xt.ptr + 2 * ((int64_t)t.job.seq * xt.sb + (int64_t)t.head * xt.sh + (int64_t)t.job.tok0 * xt.st) + cch * 16;
-            const int64_t tk = ((int64_t)t.head * p.n_kb + t.kb) * p.tab_tokens + tab_token(p, t.job, 0);
+            const int64_t tk = tab_index(p, t.head, t.job, 0, t.kb);
             r.rt = p.rtab + tk;
             r.gt = p.gtab + tk;
             r.row0 = t.job.rb * kRowBlock;
@@ -732,7 +729,9 @@ __global__ __launch_bounds__(2 * kThreads, 2) void mfma_bwd_dkv_stream_kernel(KP
         };
         auto request_carry = [&](const ItemPtrs& t, int row0) {
             const int qi = min(row0 + (ct & (kRowBlock - 1)), t.len - 1);
-            cR = t.rt[qi]; cG = t.gt[qi];
+            const int qb = qi >> 7;            // row block of the query: its slab starts qb*(qb+1) columns in
+            const int64_t ix = (int64_t)qb * (qb + 1) * kRowBlock + (qi & (kRowBlock - 1));
+            cR = t.rt[ix]; cG = t.gt[ix];
         };
         // K and V tiles of an item go straight from global memory into LDS (no registers, and
         // nothing for the wait-count bookkeeping to track): every instruction moves 64 x 16 bytes
@@ -990,17 +989,18 @@ __global__ __launch_bounds__(kThreads, D == 64 ? 2 : 1) void mfma_bwd_dkv_own_ke
 
     // carries of a (query, this wave's 32 keys) pair: the right half of a 64-key block takes the
     // forward's block-edge carry and the mid-block prefix, the left half the other two
-    const int kb64 = min((q_begin + 32 * wave) / kKeyBlock, p.n_kb - 1);   // (waves past the end have no work)
-    const float* rsrc = ((wave & 1) ? p.rtab : p.rmid) + ((int64_t)head * p.n_kb + kb64) * p.tab_tokens;
-    const float* gsrc = ((wave & 1) ? p.gmid : p.gtab) + ((int64_t)head * p.n_kb + kb64) * p.tab_tokens;
+    const int kb64 = (q_begin + 32 * wave) / kKeyBlock;      // 2*rb or 2*rb + 1: a column of every row block's slab from rb on
+    const float* rsrc = ((wave & 1) ? p.rtab : p.rmid) + tab_index(p, head, job, 0, kb64);
+    const float* gsrc = ((wave & 1) ? p.gmid : p.gtab) + tab_index(p, head, job, 0, kb64);
     float Rn[2] = {1.f, 1.f}, Gn[2] = {0.f, 0.f};
     auto request_carries = [&](int q0) {
 #pragma unroll
         for (int t = 0; t < 2; ++t) {
             const int qi = min(q0 + 32 * t + n, job.len - 1);
-            const int64_t tok = tab_token(p, job, qi);
-            Rn[t] = rsrc[tok];
-            Gn[t] = gsrc[tok];
+            const int qb = qi >> 7;
+            const int64_t ix = (int64_t)qb * (qb + 1) * kRowBlock + (qi & (kRowBlock - 1));
+            Rn[t] = rsrc[ix];
+            Gn[t] = gsrc[ix];
         }
     };
     if (n_steps > 0) request_carries(q_begin);

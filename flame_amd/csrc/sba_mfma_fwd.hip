@@ -40,7 +40,7 @@ __global__ __launch_bounds__(kThreads) void mfma_fwd_kernel(KParams p) {
     const int imax = min(m0 + kRowBlock - 1, job.len - 1);
     const int kmax = imax - strict;                       // last key any row of the block sees
     const int n_steps = kmax >= 0 ? kmax / kKeyBlock + 1 : 0;
-    const int64_t tabtok = tab_token(p, job, qi);
+    const int64_t tabq = tab_index(p, head, job, job.rb, 0) + 32 * wave + n;   // + step * kRowBlock
 
     TileDma<D> kc, vc;
     kc.init(lane, wave, p.k, kbase);
@@ -63,7 +63,7 @@ __global__ __launch_bounds__(kThreads) void mfma_fwd_kernel(KParams p) {
         // wait for the tile loads at the end of the step then also covers this store, long
         // after it has completed, instead of stalling the next iteration's loads on it.
         if (!skip && p.save && h == 0 && qi < job.len)
-            p.rtab[((int64_t)head * p.n_kb + step) * p.tab_tokens + tabtok] = R;
+            p.rtab[tabq + step * kRowBlock] = R;
         if (more) {       // next tiles, straight into the other buffer (free since the last barrier)
             kc.issue((step - 1) * kKeyBlock, job.len, lds + (buf ^ 1) * 2 * kTile);
             if (!kCarryOnly) vc.issue((step - 1) * kKeyBlock, job.len, lds + (buf ^ 1) * 2 * kTile + kTile);
@@ -166,7 +166,7 @@ __global__ __launch_bounds__(2 * kThreads) void mfma_fwd2_kernel(KParams p) {
     const int kmax = imax - strict;
     const int n_steps = kmax >= 0 ? kmax / kKeyBlock + 1 : 0;
     const int n_it = (n_steps + 1) / 2;
-    const int64_t tabtok = tab_token(p, job, qi);
+    const int64_t tabq = tab_index(p, head, job, job.rb, 0) + 32 * qs + n;   // + step * kRowBlock
     char* my_tiles = lds + grp * 2 * kTile;          // + buf * 4 * kTile
 
     // each group copies its own tiles (256 threads per tile pair)
@@ -211,7 +211,7 @@ __global__ __launch_bounds__(2 * kThreads) void mfma_fwd2_kernel(KParams p) {
         R = R * total * other;
         if (active) {
             if (p.save && h == 0 && qi < job.len)
-                p.rtab[((int64_t)head * p.n_kb + step) * p.tab_tokens + tabtok] = Rmy;
+                p.rtab[tabq + step * kRowBlock] = Rmy;
             if (!kCarryOnly) {
                 scale_clamped<32>(x, fac * Rmy);
                 bf16x8 pf[4];

@@ -65,7 +65,7 @@ class SBA(nn.Module):
                 raise ValueError("cu_seqlens needs a packed batch of size 1")
             max_len = kwargs.get('max_seqlen', None)
             if max_len is None:
-                max_len = T            # an upper bound is enough: it only sizes the carry tables
+                max_len = T            # an upper bound is enough (the carry tables are sized from the documents)
             q, k, v = (x.view(T, H, D).transpose(0, 1) for x in (q, k, v))     # [H, T, D] views
             o, _ = self.attn_varlen_fn(q, k, v, cu_seqlens, max_len)
             o = o.transpose(0, 1).reshape(1, T, H * D)

@@ -35,7 +35,7 @@ def workspace_bytes(q, inv_temp=1.0) -> int:
     """What lives from the forward to the backward (the forward's carry table)."""
     if torch.compiler.is_compiling():
         B, H, T, D = q.shape
-        return _lib.workspace_upper_bound(H, T, B * T, D)
+        return _lib.workspace_upper_bound(H, _lib.dense_columns(B, T))
     return int(_lib.load().sba_workspace_bytes(C.byref(_params(q, q, q, inv_temp, False))))
 
 
@@ -44,7 +44,7 @@ def bwd_scratch_bytes(q, have_workspace=True) -> int:
     kept none)."""
     if torch.compiler.is_compiling():
         B, H, T, D = q.shape
-        return _lib.bwd_scratch_upper_bound(H, T, B * T, D)
+        return _lib.bwd_scratch_upper_bound(H, _lib.dense_columns(B, T), B * T, D)
     p = _params(q, q, q, 1.0, False)
     p.workspace = 1 if have_workspace else None       # only NULL or not is looked at
     return int(_lib.load().sba_bwd_scratch_bytes(C.byref(p)))
@@ -112,8 +112,11 @@ class StickBreakingAttention(torch.autograd.Function):
                                "there is no CPU path")
         if not (q.dtype == k.dtype == v.dtype):
             raise TypeError("q, k, v must share a dtype")
+        if not (q.device == k.device == v.device):
+            raise ValueError("q, k, v must be on the same device")
         if not (q.shape == k.shape == v.shape) or q.dim() != 4:
             raise ValueError("q, k, v must all be [B, H, T, D]")
+        _lib.check_supported(q)
         no_grad = not any(ctx.needs_input_grad[:3])
         ctx.head_dim = q.shape[-1]
         Dp = _lib.matrix_core_head_dim(q)
@@ -144,4 +147,7 @@ def sb_attn(q, k, v, inv_temp=None, zero_start=True, attend_current=False):
 
 
 def sb_attn_(q, k, v, inv_temp, attend_current):
+    if not torch.is_grad_enabled():
+        # no backward can follow: detached inputs tell the forward to keep no carry table
+        q, k, v = q.detach(), k.detach(), v.detach()
     return StickBreakingAttention.apply(q, k, v, inv_temp, attend_current)

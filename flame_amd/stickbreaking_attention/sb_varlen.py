@@ -25,24 +25,26 @@ from .utils import custom_op
 _SCHEDULES: dict = {}
 
 
-def _schedule_for(cu_seqlens: torch.Tensor, n_heads: int):
-    """(cu int32 on device with leading 0, schedule on device, n_jobs, max_len, total).  The job
-    order depends on the launch size (jobs x heads): one entry per cu_seqlens tensor and order."""
-    hit = _SCHEDULES.get(id(cu_seqlens))
+def _schedule_for(cu_seqlens: torch.Tensor, n_heads: int, device: torch.device):
+    """(cu int32 on `device` with leading 0, schedule on `device`, n_jobs, max_len, total, table
+    columns).  `cu_seqlens` itself may live anywhere (a CPU tensor spares the host sync); what the
+    kernels read is placed on the device of q.  The job order depends on the launch size
+    (jobs x heads): one entry per cu_seqlens tensor, device and order."""
+    key = (id(cu_seqlens), device)
+    hit = _SCHEDULES.get(key)
     if hit is not None and hit[0]() is cu_seqlens and hit[1] == cu_seqlens._version:
         entry = hit[2]
         if (entry[2] * n_heads >= _lib.DOC_MAJOR_GRID) == hit[3]:
             return entry
-    key = id(cu_seqlens)
     cu_host = cu_seqlens.detach().to("cpu", torch.int32)   # one host sync per new packing
-    if cu_host.numel() < 2 or int(cu_host[0]) != 0:
-        raise ValueError("cu_seqlens must start with 0 and hold at least one document")
+    if cu_host.dim() != 1 or cu_host.numel() < 2 or int(cu_host[0]) != 0:
+        raise ValueError("cu_seqlens must be 1-D, start with 0 and hold at least one document")
     lens = cu_host[1:] - cu_host[:-1]
     if bool((lens < 0).any()):
         raise ValueError("cu_seqlens must be non-decreasing")
     sched = _lib.build_schedule(cu_host, n_heads)
-    dev = cu_seqlens.device
-    entry = (cu_host.to(dev), sched.to(dev), sched.shape[0], int(lens.max()), int(cu_host[-1]))
+    entry = (cu_host.to(device), sched.to(device), sched.shape[0], int(lens.max()), int(cu_host[-1]),
+             _lib.table_columns(cu_host))
     ref = weakref.ref(cu_seqlens, lambda _r, key=key: _SCHEDULES.pop(key, None))
     _SCHEDULES[key] = (ref, cu_seqlens._version, entry, sched.shape[0] * n_heads >= _lib.DOC_MAJOR_GRID)
     return entry
@@ -62,33 +64,43 @@ def _params(q, k, v, n_docs, max_seqlens, inv_temp, attend_current):
 
 
 def _bind_schedule(p, q, cu_seqlens, max_seqlens):
-    cu_dev, sched, n_jobs, max_len, total = _schedule_for(cu_seqlens, q.shape[0])
+    cu_dev, sched, n_jobs, max_len, total, cols = _schedule_for(cu_seqlens, q.shape[0], q.device)
     if total != q.shape[1]:
         raise ValueError(f"cu_seqlens ends at {total} but q has {q.shape[1]} tokens")
     if max_len > max_seqlens:
         raise ValueError(f"max_seqlens={max_seqlens} is smaller than the longest document ({max_len})")
-    p.cu_seqlens, p.schedule, p.n_schedule = cu_dev.data_ptr(), sched.data_ptr(), n_jobs
+    p.cu_seqlens, p.schedule, p.n_schedule, p.table_cols = cu_dev.data_ptr(), sched.data_ptr(), n_jobs, cols
     return n_jobs
 
 
-def workspace_bytes(q, max_seqlens: int) -> int:
-    """What lives from the forward to the backward (the forward's carry table)."""
+def _columns(q, cu_seqlens, max_seqlens: int) -> int:
+    """Carry-table columns of this packing: exact from the cached schedule, or, while
+    torch.compile traces (no look at cu_seqlens' values), a bound from the shapes."""
     if torch.compiler.is_compiling():
-        H, N, D = q.shape
-        return _lib.workspace_upper_bound(H, max_seqlens, N, D)
+        return _lib.packed_columns_bound(q.shape[1], cu_seqlens.numel() - 1, max_seqlens)
+    return _schedule_for(cu_seqlens, q.shape[0], q.device)[5]
+
+
+def workspace_bytes(q, cu_seqlens, max_seqlens: int) -> int:
+    """What lives from the forward to the backward (the forward's carry table): one float per
+    query and visible 64-key block of its own document, sized from the actual document lengths."""
+    cols = _columns(q, cu_seqlens, max_seqlens)
+    if torch.compiler.is_compiling():
+        return _lib.workspace_upper_bound(q.shape[0], cols)
     p = _params(q, q, q, 1, max_seqlens, 1.0, False)
-    p.cu_seqlens = 1          # only "packed or not" matters for the size
+    p.cu_seqlens, p.table_cols = 1, cols          # only "packed or not" and the size matter here
     return int(_lib.load().sba_workspace_bytes(C.byref(p)))
 
 
-def bwd_scratch_bytes(q, max_seqlens: int, have_workspace=True) -> int:
+def bwd_scratch_bytes(q, cu_seqlens, max_seqlens: int, have_workspace=True) -> int:
     """What the backward needs for the duration of its call only (one table more when the forward
     kept none)."""
+    cols = _columns(q, cu_seqlens, max_seqlens)
     if torch.compiler.is_compiling():
         H, N, D = q.shape
-        return _lib.bwd_scratch_upper_bound(H, max_seqlens, N, D)
+        return _lib.bwd_scratch_upper_bound(H, cols, N, D)
     p = _params(q, q, q, 1, max_seqlens, 1.0, False)
-    p.cu_seqlens = 1
+    p.cu_seqlens, p.table_cols = 1, cols
     p.workspace = 1 if have_workspace else None       # only NULL or not is looked at
     return int(_lib.load().sba_bwd_scratch_bytes(C.byref(p)))
 
@@ -135,7 +147,7 @@ def varlen_fwd(q, k, v, cu_seqlens, max_seqlens, logit_scale, attend_current=Fal
     o = torch.empty_like(q)
     rem = torch.empty(q.shape[:-1], dtype=q.dtype, device=q.device)
     keep = not (no_grad or _lib.recompute_carries())
-    nbytes = max(workspace_bytes(q, max_seqlens), 16) if keep else 16
+    nbytes = max(workspace_bytes(q, cu_seqlens, max_seqlens), 16) if keep else 16
     ws = torch.empty(nbytes, dtype=torch.uint8, device=q.device)
     _compileable_forward(q, k, v, cu_seqlens, int(max_seqlens), float(logit_scale), bool(attend_current),
                          keep, o, rem, ws)
@@ -145,7 +157,8 @@ def varlen_fwd(q, k, v, cu_seqlens, max_seqlens, logit_scale, attend_current=Fal
 def varlen_bwd(do, dr, q, k, v, cu_seqlens, max_seqlens, ws, logit_scale, attend_current=False):
     dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
     # freed when this call returns: only the forward's table is kept between the two directions
-    scratch = torch.empty(max(bwd_scratch_bytes(q, max_seqlens, ws.numel() > 16), 16), dtype=torch.uint8, device=q.device)
+    scratch = torch.empty(max(bwd_scratch_bytes(q, cu_seqlens, max_seqlens, ws.numel() > 16), 16), dtype=torch.uint8,
+                          device=q.device)
     _compileable_backward(do, dr, q, k, v, cu_seqlens, int(max_seqlens), ws, scratch, float(logit_scale),
                           bool(attend_current), dq, dk, dv)
     return dq, dk, dv
@@ -158,8 +171,13 @@ class StickBreakingAttention(torch.autograd.Function):
         if not q.is_cuda:
             raise RuntimeError("stick-breaking attention runs on the GPU only (HIP kernels); "
                                "there is no CPU path")
+        if not (q.dtype == k.dtype == v.dtype):
+            raise TypeError("q, k, v must share a dtype")
+        if not (q.device == k.device == v.device):
+            raise ValueError("q, k, v must be on the same device")
         if not (q.shape == k.shape == v.shape) or q.dim() != 3:
             raise ValueError("q, k, v must all be [H, total_tokens, D]")
+        _lib.check_supported(q)
         no_grad = not any(ctx.needs_input_grad[:3])
         ctx.head_dim = q.shape[-1]
         Dp = _lib.matrix_core_head_dim(q)
@@ -187,14 +205,26 @@ class StickBreakingAttention(torch.autograd.Function):
 
 def sb_attn_varlen(q, k, v, cu_seqlens, max_seqlens, inv_temp=None, zero_start=True,
                    attend_current=False):
+    """cu_seqlens with its leading 0 when zero_start (the default), document ends only
+    otherwise, as in the reference (sb_varlen/__init__.py:71-78).  The kernels always work from
+    the form with the leading 0, and the schedule is cached per cu_seqlens tensor: pass the
+    same tensor to every layer."""
     if not zero_start:
-        # the reference strips a leading 0 when zero_start; without one we prepend it, so
-        # the kernels always see the same convention
         cu_seqlens = torch.cat([cu_seqlens.new_zeros(1), cu_seqlens])
     if inv_temp is None:
         inv_temp = 1 / math.sqrt(q.size(-1))
-    return sb_attn_varlen_(q, k, v, inv_temp, cu_seqlens, max_seqlens, attend_current)
+    return _apply(q, k, v, cu_seqlens, max_seqlens, inv_temp, attend_current)
+
+
+def _apply(q, k, v, cu_seqlens, max_seqlens, inv_temp, attend_current):
+    if not torch.is_grad_enabled():
+        # no backward can follow: detached inputs tell the forward to keep no carry table
+        q, k, v = q.detach(), k.detach(), v.detach()
+    return StickBreakingAttention.apply(q, k, v, cu_seqlens, max_seqlens, inv_temp, attend_current)
 
 
 def sb_attn_varlen_(q, k, v, inv_temp, cu_seqlens, max_seqlens, attend_current):
-    return StickBreakingAttention.apply(q, k, v, cu_seqlens, max_seqlens, inv_temp, attend_current)
+    """The reference's inner entry point (sb_varlen/__init__.py:81-82): cu_seqlens arrives with
+    the leading 0 already stripped (document ends only)."""
+    cu_seqlens = torch.cat([cu_seqlens.new_zeros(1), cu_seqlens])
+    return _apply(q, k, v, cu_seqlens, max_seqlens, inv_temp, attend_current)

@@ -34,7 +34,7 @@
 extern "C" {
 #endif
 
-#define SBA_ABI_VERSION 4
+#define SBA_ABI_VERSION 5
 #define SBA_SCHEDULE_INTS 8   /* int32 per scheduled job, see sba_build_schedule() */
 #define SBA_DOC_MAJOR_GRID 8192 /* workgroups from which the schedule is document-major */
 
@@ -85,6 +85,7 @@ typedef struct SbaParams {
     const int32_t* cu_seqlens; /* device, n_seq+1 entries, or NULL for dense */
     const int32_t* schedule;   /* device, from sba_build_schedule(); packed layout only */
     int32_t  n_schedule;       /* number of row-block jobs in `schedule` */
+    int64_t  table_cols;       /* packed layout only: sba_table_columns() of the same cu_seqlens */
 
     SbaTensor q, k, v;         /* inputs */
     SbaTensor o;               /* forward output            / backward: unused */
@@ -132,7 +133,8 @@ size_t sba_bwd_scratch_bytes(const SbaParams* p);
  * Row-block schedule for the packed layout, built on the host from host cu_seqlens
  * (n_seq+1 entries, leading 0).  Writes up to `capacity` rows of SBA_SCHEDULE_INTS (8)
  * int32 each into `out` (host memory) and returns the number of jobs: ints 0-3 of row i are
- * {first_token, doc_len, row_block, doc_index} of the i-th job, longest row-blocks first;
+ * {first_token, doc_len, row_block, first carry-table column of the document} of the i-th job,
+ * longest row-blocks first;
  * ints 4-7 are the same four of the job that comes i-th for the dK/dV kernel, whose sweeps
  * run from a row-block to the END of its document (or the number needed when
  * `out` is NULL or capacity is too small).  `n_heads` is the head count the schedule will be
@@ -148,6 +150,17 @@ int sba_build_schedule(const int32_t* cu_seqlens_host, int n_seq, int n_heads, i
 
 /* Rows of queries one scheduled job covers (the kernels' row-block height). */
 int sba_row_block(void);
+
+/*
+ * Size of the carry tables of a packed batch, in columns of sba_row_block() floats per head:
+ * the sum over the documents of n*(n+1), n = ceil(len / sba_row_block()) (a row block keeps one
+ * entry per query for every 64-key block it can see, nothing for the blocks right of the
+ * diagonal).  From host cu_seqlens (n_seq+1 entries); the value goes into SbaParams.table_cols
+ * and sizes sba_workspace_bytes() / sba_bwd_scratch_bytes().  The dense layout needs no call:
+ * the library derives n_seq * n*(n+1) from seq_len.  (The reference keeps one float per query,
+ * sb_fwd.py:146; the tables are what makes the backward atomic-free.)
+ */
+int64_t sba_table_columns(const int32_t* cu_seqlens_host, int n_seq);
 
 /* Forward: o, rem (and the carry table when save_for_backward). */
 int sba_fwd(const SbaParams* p);

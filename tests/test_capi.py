@@ -30,7 +30,7 @@ def test_exports_every_declared_symbol(lib):
 
 
 def test_abi_version_and_struct_size(lib):
-    assert lib.sba_abi_version() == 4
+    assert lib.sba_abi_version() == 5
     p = _lib.SbaParams()
     p.struct_size = C.sizeof(_lib.SbaParams) - 8
     assert lib.sba_fwd(C.byref(p)) == -7          # SBA_ERR_ABI, before anything touches a GPU
@@ -57,7 +57,9 @@ def test_workspace_bytes(lib):
     p.struct_size = C.sizeof(_lib.SbaParams)
     p.dtype = _lib.SBA_DTYPE_BF16
     p.n_seq, p.n_heads, p.seq_len, p.total_tokens, p.head_dim = 1, 16, 4096, 4096, 64
-    table = 16 * 64 * 4096 * 4                      # one carry table [H][T/64][T] fp32
+    # one carry table: per head, row block qb keeps 128 queries x its 2*qb + 2 visible 64-key blocks:
+    # 32 * 33 columns of 128 floats at T = 4096 (half of a full [T/64][T] rectangle, plus the diagonal)
+    table = 16 * 32 * 33 * 128 * 4
     assert lib.sba_workspace_bytes(C.byref(p)) == table          # what the forward hands to the backward
     assert lib.sba_bwd_scratch_bytes(C.byref(p)) == 4 * table    # no workspace: the backward recomputes that table
     p.workspace = 1
@@ -86,9 +88,13 @@ def test_schedule_builder(lib):
     cu = torch.tensor([0, 100, 400, 401, 1000, 1000], dtype=torch.int32)   # last doc empty
     s = _lib.build_schedule(cu)
     jobs = [tuple(r[:4]) for r in s.tolist()]
-    # every (doc, row_block) exactly once, none for the empty document
-    expect = {(0, 100, 0, 0), (100, 300, 0, 1), (100, 300, 1, 1), (100, 300, 2, 1), (400, 1, 0, 2)}
-    expect |= {(401, 599, rb, 3) for rb in range(5)}
+    # every (doc, row_block) exactly once, none for the empty document; the fourth int is the
+    # document's first carry-table column: documents of 1, 3, 1, 5 row blocks take 2, 12, 2, 30 columns
+    doc_of_col = {0: 0, 2: 1, 14: 2, 16: 3}
+    expect = {(0, 100, 0, 0), (100, 300, 0, 2), (100, 300, 1, 2), (100, 300, 2, 2), (400, 1, 0, 14)}
+    expect |= {(401, 599, rb, 16) for rb in range(5)}
+    assert lib.sba_table_columns(C.cast(cu.data_ptr(), C.POINTER(C.c_int32)), 5) == 46
+    assert _lib.table_columns(cu) == 46
     assert set(jobs) == expect and len(jobs) == len(expect)
     rbs = [j[2] for j in jobs]
     assert rbs == sorted(rbs, reverse=True)       # longest sweeps first
@@ -108,9 +114,9 @@ def test_schedule_builder(lib):
     d = _lib.build_schedule(cu, heads)
     assert sorted(tuple(r[:4]) for r in d.tolist()) == sorted(jobs)
     assert sorted(tuple(r[4:8]) for r in d.tolist()) == sorted(jobs)
-    row_order = [(r[3], r[2]) for r in d.tolist()]
+    row_order = [(doc_of_col[r[3]], r[2]) for r in d.tolist()]
     assert row_order == [(3, 4), (3, 3), (3, 2), (3, 1), (3, 0), (1, 2), (1, 1), (1, 0), (0, 0), (2, 0)]
-    key_order = [(r[7], r[6]) for r in d.tolist()]
+    key_order = [(doc_of_col[r[7]], r[6]) for r in d.tolist()]
     assert key_order == [(3, 0), (3, 1), (3, 2), (3, 3), (3, 4), (1, 0), (1, 1), (1, 2), (0, 0), (2, 0)]
     assert _lib.build_schedule(cu, heads - 1).tolist() == s.tolist()      # just below: the usual order
 
@@ -129,5 +135,10 @@ def test_python_workspace_bound_covers_the_library(lib):
             p.struct_size = C.sizeof(_lib.SbaParams)
             p.dtype = dtype
             p.n_seq, p.n_heads, p.seq_len, p.total_tokens, p.head_dim = B, H, T, T, D
-            assert _lib.workspace_upper_bound(H, T, B * T, D) >= lib.sba_workspace_bytes(C.byref(p))
-            assert _lib.bwd_scratch_upper_bound(H, T, B * T, D) >= lib.sba_bwd_scratch_bytes(C.byref(p))
+            cols = _lib.dense_columns(B, T)
+            assert _lib.workspace_upper_bound(H, cols) >= lib.sba_workspace_bytes(C.byref(p))
+            assert _lib.bwd_scratch_upper_bound(H, cols, B * T, D) >= lib.sba_bwd_scratch_bytes(C.byref(p))
+    # packed: the bound from shapes alone (what a torch.compile trace can see) covers the exact count
+    for lens in ([1, 130, 500, 64, 205], [4096] * 3 + [16] * 40, [127, 128, 129], [1]):
+        cu = torch.tensor([0] + list(torch.tensor(lens).cumsum(0)), dtype=torch.int32)
+        assert _lib.packed_columns_bound(sum(lens), len(lens), max(lens)) >= _lib.table_columns(cu)

@@ -26,6 +26,7 @@ def _params(q, k, v, cu=None, max_len=None, sched=None):
         H, N, D = q.shape
         p.n_seq, p.n_heads, p.seq_len, p.total_tokens, p.head_dim = cu.numel() - 1, H, max_len, N, D
         p.cu_seqlens, p.schedule, p.n_schedule = cu.data_ptr(), sched.data_ptr(), sched.shape[0]
+        p.table_cols = _lib.table_columns(cu.cpu())
         desc = _lib.tensor3
     p.scale = 1.0 / math.sqrt(q.shape[-1])
     p.q, p.k, p.v = desc(q), desc(k), desc(v)
