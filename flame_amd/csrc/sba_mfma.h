@@ -327,6 +327,32 @@ __device__ inline void score_tiles_o(float (&x)[32], const char* ktile, const La
     scale_scores(x, raw, scale2);
 }
 
+// Row fragments multiplied by the logit scale once, ahead of the sweep (fp32 product, rounded
+// back to bf16): the score MFMAs then deliver base-2 logits directly and the per-element
+// multiplication disappears from every step.  Costs one more bf16 rounding of q (relative
+// 2^-9 per element, the size of the rounding the inputs already carry).
+template <int NF> __device__ inline void prescale_frags(bf16x8 (&f)[NF], float s) {
+#pragma unroll
+    for (int ks = 0; ks < NF; ++ks)
+#pragma unroll
+        for (int i = 0; i < 8; i += 2) {
+            const f32x2 v = {(float)f[ks][i] * s, (float)f[ks][i + 1] * s};
+            const bf16x2 b = __builtin_convertvector(v, bf16x2);
+            f[ks][i] = b[0]; f[ks][i + 1] = b[1];
+        }
+}
+// Score tiles from pre-scaled fragments: x[16*t + r] = raw accumulator, no vector work.
+template <int D, bool kBatch = (D == 128)>
+__device__ inline void score_tiles_ps(float (&x)[32], const char* ktile, const LaneOffsets<D>& o,
+                                      const bf16x8 (&qf)[D / 16]) {
+    f32x16 raw[2];
+    score_raw_o<D, kBatch>(raw, ktile, o, qf);
+#pragma unroll
+    for (int t = 0; t < 2; ++t)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) x[16 * t + r] = raw[t][r];
+}
+
 // In-place: x[idx] (base-2 logits, idx = key offset inside this lane's 32 keys; invalid
 // pairs already set to -inf) -> stick-breaking weights of this step, given the carry
 // `R` = product of (1 - beta) over all keys right of the step.
@@ -402,6 +428,52 @@ __device__ inline float product_chain_with(float (&x)[N], float (&beta)[kNeedBet
 template <int N> __device__ inline void scale_clamped(float (&x)[N], float f) {
 #pragma unroll
     for (int idx = 0; idx < N; ++idx) x[idx] = clamp01(x[idx] * f);
+}
+
+// Forward weights with ONE reciprocal per lane and step instead of one per key.  With
+// W_j = prod_{k >= j} (1 + e_k) inside the lane's 32 keys, the running products of 1 - beta are
+// L_j = 1 / W_j, and L_{j+1} = L_j (1 + e_j): from the single reciprocal of the lane's total
+// the chain is walked back UP with one fma per key, and the weight of key j is
+//     a_j = L_{j+1} - L_j = L_j e_j                      (no cancellation for small e_j).
+// Starting the walk from  carry / W_0  delivers finished weights, so per key: exp, fma (W),
+// mul (a), fma (L).  The walk needs a finite, not too large W_0 in every lane of the wave
+// (2^96 leaves the reciprocal far from the denormals).  Otherwise - logits so large that the
+// product of 32 factors leaves the fp32 range - the function returns false with R untouched
+// (x then holds e = 2^logit), and the caller does the step with the reciprocal-per-key chain,
+// which handles overflow.  The answer is the same in all lanes of a wave.
+// In: x[idx] base-2 logits (-inf for invisible pairs).  Out: pf[c] = the weights of keys
+// 8c .. 8c+7 packed to bf16 (the B operand of P*V), R advanced.  kWeights = false: only R is
+// advanced (the carry-only forward).
+constexpr float kFastChainLimit = 0x1p96f;
+
+template <bool kWeights>
+__device__ inline bool forward_weights_fast(float (&x)[32], bf16x8 (&pf)[4], float& R, int lane) {
+    float W = 1.0f;
+#pragma unroll
+    for (int idx = 31; idx >= 0; --idx) {
+        x[idx] = __builtin_amdgcn_exp2f(x[idx]);          // e
+        W = __builtin_fmaf(W, x[idx], W);
+    }
+    if (__builtin_amdgcn_ballot_w64(!(W < kFastChainLimit)) != 0) return false;
+    const float Linv = __builtin_amdgcn_rcpf(W);
+    float Llo, Lup;
+    half_values(Linv, Llo, Lup);
+    if (kWeights) {
+        float Lt = ((lane >= 32) ? R : R * Lup) * Linv;       // (carry entering this lane's keys) / W_0
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+            float a[8];
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                const float e = x[8 * c + i];
+                a[i] = Lt * e;
+                Lt = __builtin_fmaf(Lt, e, Lt);
+            }
+            pf[c] = pack8(a);
+        }
+    }
+    R = R * Llo * Lup;
+    return true;
 }
 
 template <bool kNeedBeta>

@@ -1,11 +1,71 @@
-// bf16 MFMA forward kernel (head_dim 64 / 128).
-// Replaces the reference's `_forward_one_row` sweep (sb_varlen/sb_varlen_fwd.py:81-215):
+// bf16 MFMA forward kernels (head_dim 64 / 128).
+// Replace the reference's `_forward_one_row` sweep (sb_varlen/sb_varlen_fwd.py:81-215):
 // one workgroup per (sequence, head, 128-query row-block), keys swept right-to-left from
 // the diagonal in steps of 64, K/V tiles double-buffered in LDS, running product of
 // (1 - beta) per query in a register.  Layout and arithmetic: sba_mfma.h.
 #include "sba_mfma.h"
 
 namespace sba {
+
+// One sweep step of one wave: 32 queries x 64 keys.  Scores (from the pre-scaled Q fragments),
+// mask on the diagonal, weights, O^T += V^T P^T.  kFast: the one-reciprocal chain; it may refuse
+// the step (returns false, nothing changed), see forward_weights_fast().
+template <int D, bool kCarryOnly, bool kFast>
+__device__ inline bool fwd_step(const char* ktile, const char* vtile, const LaneOffsets<D>& lo,
+                                const bf16x8 (&qf)[D / 16], f32x16 (&oacc)[D / 32], float& R, int lane,
+                                int key0, int q0w, int qi, int strict) {
+    const int h = lane >> 5;
+    float x[32];
+    score_tiles_ps<D>(x, ktile, lo, qf);
+    if (key0 + 63 + strict > q0w) mask_step(x, key0 + 32 * h, qi, strict);     // diagonal region
+    bf16x8 pf[4];
+    if (kFast) {
+        if (!forward_weights_fast<!kCarryOnly>(x, pf, R, lane)) return false;
+    } else {
+        float dummy[1];
+        stick_weights<false>(x, dummy, R, lane);
+        if (!kCarryOnly) {
+#pragma unroll
+            for (int c = 0; c < 4; ++c) pf[c] = pack8(&x[8 * c]);
+        }
+    }
+    if (!kCarryOnly) {
+#pragma unroll
+        for (int c2 = 0; c2 < 2; ++c2) {   // operands of two key groups requested together, ahead of their MFMAs
+            bf16x8 vt[2][D / 32];
+#pragma unroll
+            for (int cc = 0; cc < 2; ++cc)
+#pragma unroll
+                for (int db = 0; db < D / 32; ++db) vt[cc][db] = fetch_cols_o<D>(vtile, lo, db, 2 * c2 + cc);
+            if (D == 128) __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int cc = 0; cc < 2; ++cc)
+#pragma unroll
+                for (int db = 0; db < D / 32; ++db) oacc[db] = mfma(vt[cc][db], pf[2 * c2 + cc], oacc[db]);
+        }
+    }
+    return true;
+}
+
+// rows d = 32*db + 8*g + 4*h + 0..3 of O^T, column = this lane's query
+template <int D>
+__device__ inline void store_o_row(const KParams& p, const Job& job, int head, int qi, int lane,
+                                   const f32x16 (&oacc)[D / 32]) {
+    const int h = lane >> 5;
+    const int64_t obase = (int64_t)job.seq * p.o.sb + (int64_t)head * p.o.sh + (int64_t)(job.tok0 + qi) * p.o.st;
+#pragma unroll
+    for (int db = 0; db < D / 32; ++db)
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+            f32x2 a = {oacc[db][4 * g], oacc[db][4 * g + 1]};
+            f32x2 b = {oacc[db][4 * g + 2], oacc[db][4 * g + 3]};
+            bf16x2 pa = __builtin_convertvector(a, bf16x2), pb = __builtin_convertvector(b, bf16x2);
+            uint2 w;
+            w.x = __builtin_bit_cast(uint32_t, pa);
+            w.y = __builtin_bit_cast(uint32_t, pb);
+            *(uint2*)(p.o.ptr + 2 * (obase + 32 * db + 8 * g + 4 * h)) = w;
+        }
+}
 
 // kCarryOnly: write the carry table and nothing else (no P*V, no o / rem): the backward's way of
 // getting the table when the forward kept none.
@@ -31,6 +91,7 @@ __global__ __launch_bounds__(kThreads) void mfma_fwd_kernel(KParams p) {
 
     bf16x8 qf[D / 16];
     load_row_frags<D>(qf, p.q, qbase, qi, job.len, lane);
+    prescale_frags(qf, p.scale2);
 
     f32x16 oacc[D / 32];
 #pragma unroll
@@ -52,92 +113,69 @@ __global__ __launch_bounds__(kThreads) void mfma_fwd_kernel(KParams p) {
     wait_global_memory();
     __syncthreads();
 
-    for (int step = n_steps - 1, buf = 0; step >= 0; --step, buf ^= 1) {
-        const char* ktile = lds + buf * 2 * kTile;
-        const char* vtile = ktile + kTile;
-        const bool more = step > 0;
-        const int key0 = step * kKeyBlock;
-        // whole step right of this wave's last query: nothing visible
-        const bool skip = key0 + strict > q0w + 31;
+    // what a step does before its arithmetic
+    auto open_step = [&](int step, int buf, bool skip) {
         // The carry-table store goes FIRST: vector-memory operations retire in order, so the
         // wait for the tile loads at the end of the step then also covers this store, long
         // after it has completed, instead of stalling the next iteration's loads on it.
-        if (!skip && p.save && h == 0 && qi < job.len)
-            p.rtab[tabq + step * kRowBlock] = R;
-        if (more) {       // next tiles, straight into the other buffer (free since the last barrier)
+        if (!skip && p.save && h == 0 && qi < job.len) p.rtab[tabq + step * kRowBlock] = R;
+        if (step > 0) {   // next tiles, straight into the other buffer (free since the last barrier)
             kc.issue((step - 1) * kKeyBlock, job.len, lds + (buf ^ 1) * 2 * kTile);
             if (!kCarryOnly) vc.issue((step - 1) * kKeyBlock, job.len, lds + (buf ^ 1) * 2 * kTile + kTile);
         }
-        if (!skip) {
-            float x[32];
-            score_tiles_o<D>(x, ktile, lo, qf, p.scale2);
-            if (key0 + 63 + strict > q0w) {     // diagonal region: mask invisible pairs
-mask_step(x, key0 + 32 * h, qi, strict);
-            }
-            float dummy[1];
-            stick_weights<false>(x, dummy, R, lane);
-            if (!kCarryOnly) {
-                bf16x8 pf[4];
-#pragma unroll
-                for (int c = 0; c < 4; ++c) pf[c] = pack8(&x[8 * c]);
-                if (D == 128) {
-#pragma unroll
-                    for (int c = 0; c < 4; ++c) {      // (operands of a key group requested together, see score_raw_o)
-                        bf16x8 vt[D / 32];
-#pragma unroll
-                        for (int db = 0; db < D / 32; ++db) vt[db] = fetch_cols_o<D>(vtile, lo, db, c);
-                        __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-                        for (int db = 0; db < D / 32; ++db) oacc[db] = mfma(vt[db], pf[c], oacc[db]);
-                    }
-                } else {
-#pragma unroll
-                    for (int db = 0; db < D / 32; ++db)
-#pragma unroll
-                        for (int c = 0; c < 4; ++c)
-                            oacc[db] = mfma(fetch_cols_o<D>(vtile, lo, db, c), pf[c], oacc[db]);
-                }
-            }
+    };
+    // The sweep runs with the one-reciprocal chain until a step refuses it (logits too large for
+    // it); from that step on this wave continues with the reciprocal-per-key chain.  Every wave
+    // executes one barrier per step whichever loop it is in.
+    int step = n_steps - 1, buf = 0;
+    bool redo = false;
+    for (; step >= 0; --step, buf ^= 1) {
+        const char* ktile = lds + buf * 2 * kTile;
+        const int key0 = step * kKeyBlock;
+        const bool skip = key0 + strict > q0w + 31;       // whole step right of this wave's last query
+        open_step(step, buf, skip);
+        if (!skip && !fwd_step<D, kCarryOnly, true>(ktile, ktile + kTile, lo, qf, oacc, R, lane, key0, q0w, qi, strict)) {
+            redo = true;
+            break;
         }
         wait_global_memory();                  // the next tiles have landed
         __syncthreads();
     }
+    for (; step >= 0; --step, buf ^= 1) {
+        const char* ktile = lds + buf * 2 * kTile;
+        const int key0 = step * kKeyBlock;
+        const bool skip = key0 + strict > q0w + 31;
+        if (!redo) open_step(step, buf, skip);
+        redo = false;
+        if (!skip) fwd_step<D, kCarryOnly, false>(ktile, ktile + kTile, lo, qf, oacc, R, lane, key0, q0w, qi, strict);
+        wait_global_memory();
+        __syncthreads();
+    }
 
     if (qi < job.len && !kCarryOnly) {
-        const int64_t obase = (int64_t)job.seq * p.o.sb + (int64_t)head * p.o.sh + (int64_t)(job.tok0 + qi) * p.o.st;
-#pragma unroll
-        for (int db = 0; db < D / 32; ++db)
-#pragma unroll
-            for (int g = 0; g < 4; ++g) {
-                // rows d = 32*db + 8*g + 4*h + 0..3 of O^T, column = this query
-                f32x2 a = {oacc[db][4 * g], oacc[db][4 * g + 1]};
-                f32x2 b = {oacc[db][4 * g + 2], oacc[db][4 * g + 3]};
-                bf16x2 pa = __builtin_convertvector(a, bf16x2), pb = __builtin_convertvector(b, bf16x2);
-                uint2 w;
-                w.x = __builtin_bit_cast(uint32_t, pa);
-                w.y = __builtin_bit_cast(uint32_t, pb);
-                *(uint2*)(p.o.ptr + 2 * (obase + 32 * db + 8 * g + 4 * h)) = w;
-            }
+        store_o_row<D>(p, job, head, qi, lane, oacc);
         if (h == 0)
             Elem<uint16_t>::store(p.rem.ptr, (int64_t)job.seq * p.rem.sb + (int64_t)head * p.rem.sh + job.tok0 + qi, R);
     }
 }
 
-// ---------------------------------------------------------------- two steps per iteration
-// Same sweep with 8 waves: wave-group 0 (waves 0-3) and wave-group 1 (waves 4-7) take two
-// CONSECUTIVE 64-key steps of the same 128 queries in every iteration.  All the heavy work of
-// a step (scores, exp/rcp, the in-step product chain, P*V) only needs the step's own keys; what
-// couples neighbouring steps is one number per query, the product of (1 - beta) over the
-// step.  The groups swap those totals through LDS at a barrier, the left group multiplies the
-// right group's total into its carry, and each group accumulates its own partial O, summed once
-// at the end.  The longest dependent chain of a kernel launch (the sweep of the last row-block)
-// is halved, which is what bounds the time when the whole problem is only two waves per SIMD.
-template <int D, bool kCarryOnly>
-__global__ __launch_bounds__(2 * kThreads) void mfma_fwd2_kernel(KParams p) {
+// ---------------------------------------------------------------- small grids: G segments per sweep
+// A launch of a few hundred workgroups cannot fill the SIMDs with one-sweep-per-workgroup work,
+// and lasts as long as its longest sweep.  Here a workgroup has G groups of four waves, and the
+// sweep of its 128 queries is cut into G CONTIGUOUS segments of keys, one per group (group 0 the
+// rightmost, with the diagonal).  Every group runs the ordinary sweep over its segment from a
+// carry of 1 - nothing couples the segments but one number per query, the product of (1 - beta)
+// over a whole segment - and at the end
+//     O = sum_g F_g O_g,   F_g = product of the totals of the segments right of g,
+// is formed through LDS, the carry-table entries that a group wrote relative to its own right
+// edge are multiplied by F_g, and rem is the product of all totals.  No exchange inside the
+// sweep; the groups only share the workgroup barrier that hands over the tiles.
+template <int D, int G, bool kCarryOnly>
+__global__ __launch_bounds__(G * kThreads) void mfma_fwd_seg_kernel(KParams p) {
     constexpr int kTile = 64 * D * 2;
-    // tile(buf, grp, kv) = lds + ((buf * 2 + grp) * 2 + kv) * kTile
-    __shared__ __attribute__((aligned(16))) char lds[8 * kTile];
-    __shared__ float xch[2][kRowBlock];
+    // tile(grp, buf, kv) = lds + ((grp * 2 + buf) * 2 + kv) * kTile
+    __shared__ __attribute__((aligned(16))) char lds[G * 4 * kTile];
+    __shared__ float totals[G][kRowBlock];
 
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -157,6 +195,7 @@ __global__ __launch_bounds__(2 * kThreads) void mfma_fwd2_kernel(KParams p) {
 
     bf16x8 qf[D / 16];
     load_row_frags<D>(qf, p.q, qbase, qi, job.len, lane);
+    prescale_frags(qf, p.scale2);
     f32x16 oacc[D / 32];
 #pragma unroll
     for (int db = 0; db < D / 32; ++db) oacc[db] = f32x16{0};
@@ -165,131 +204,145 @@ __global__ __launch_bounds__(2 * kThreads) void mfma_fwd2_kernel(KParams p) {
     const int imax = min(m0 + kRowBlock - 1, job.len - 1);
     const int kmax = imax - strict;
     const int n_steps = kmax >= 0 ? kmax / kKeyBlock + 1 : 0;
-    const int n_it = (n_steps + 1) / 2;
+    const int chunk = (n_steps + G - 1) / G;              // iterations of every group
+    const int hi = n_steps - grp * chunk;                  // this group sweeps steps hi-1 .. low
+    const int low = max(hi - chunk, 0);
     const int64_t tabq = tab_index(p, head, job, job.rb, 0) + 32 * qs + n;   // + step * kRowBlock
-    char* my_tiles = lds + grp * 2 * kTile;          // + buf * 4 * kTile
+    char* my_tiles = lds + grp * 4 * kTile;                // + buf * 2 * kTile
 
-    // each group copies its own tiles (256 threads per tile pair)
     TileDma<D> kc, vc;
     kc.init(lane, qs, p.k, kbase);
     vc.init(lane, qs, p.v, vbase);
-    {
-        const int s0 = n_steps - 1 - grp;
-        if (s0 >= 0) {
-            kc.issue(s0 * kKeyBlock, job.len, my_tiles);
-            if (!kCarryOnly) vc.issue(s0 * kKeyBlock, job.len, my_tiles + kTile);
-        }
+    if (hi - 1 >= low) {
+        kc.issue((hi - 1) * kKeyBlock, job.len, my_tiles);
+        if (!kCarryOnly) vc.issue((hi - 1) * kKeyBlock, job.len, my_tiles + kTile);
     }
     wait_global_memory();
     __syncthreads();
 
-    for (int it = 0, buf = 0; it < n_it; ++it, buf ^= 1) {
-        const int step = n_steps - 1 - 2 * it - grp;          // -1: this group idles in the last iteration
-        const char* ktile = my_tiles + buf * 4 * kTile;
-        const char* vtile = ktile + kTile;
-        const bool more = step - 2 >= 0;
-        if (more) {       // next tiles, straight into the other buffer (free since the last barrier)
-            kc.issue((step - 2) * kKeyBlock, job.len, my_tiles + (buf ^ 1) * 4 * kTile);
-            if (!kCarryOnly) vc.issue((step - 2) * kKeyBlock, job.len, my_tiles + (buf ^ 1) * 4 * kTile + kTile);
+    auto open_step = [&](int step, int buf, bool skip) {
+        if (!skip && p.save && h == 0 && qi < job.len) p.rtab[tabq + step * kRowBlock] = R;   // relative to the segment's right edge
+        if (step - 1 >= low) {
+            kc.issue((step - 1) * kKeyBlock, job.len, my_tiles + (buf ^ 1) * 2 * kTile);
+            if (!kCarryOnly) vc.issue((step - 1) * kKeyBlock, job.len, my_tiles + (buf ^ 1) * 2 * kTile + kTile);
         }
+    };
+    int it = 0, buf = 0;
+    bool redo = false;
+    for (; it < chunk; ++it, buf ^= 1) {
+        const int step = hi - 1 - it;
+        const char* ktile = my_tiles + buf * 2 * kTile;
         const int key0 = step * kKeyBlock;
-        const bool active = step >= 0 && !(key0 + strict > q0w + 31);
-        float x[32];
-        float total = 1.0f, fac = 1.0f;
-        if (active) {
-            score_tiles_o<D, true>(x, ktile, lo, qf, p.scale2);
-            if (key0 + 63 + strict > q0w) mask_step(x, key0 + 32 * h, qi, strict);
-            float dummy[1];
-            fac = stick_weights_local<false>(x, dummy, total, lane);
+        const bool skip = step < low || key0 + strict > q0w + 31;
+        open_step(step, buf, skip);
+        if (!skip && !fwd_step<D, kCarryOnly, true>(ktile, ktile + kTile, lo, qf, oacc, R, lane, key0, q0w, qi, strict)) {
+            redo = true;
+            break;
         }
-        if (h == 0) xch[grp][32 * qs + n] = total;
+        wait_global_memory();
         __syncthreads();
-        const float other = xch[grp ^ 1][32 * qs + n];
-        // group 0 holds the right step of the pair: its carry is R; group 1's also contains
-        // group 0's total
-        const float Rmy = grp == 0 ? R : R * other;
-        R = R * total * other;
-        if (active) {
-            if (p.save && h == 0 && qi < job.len)
-                p.rtab[tabq + step * kRowBlock] = Rmy;
-            if (!kCarryOnly) {
-                scale_clamped<32>(x, fac * Rmy);
-                bf16x8 pf[4];
+    }
+    for (; it < chunk; ++it, buf ^= 1) {       // reciprocal-per-key chain from the refused step on
+        const int step = hi - 1 - it;
+        const char* ktile = my_tiles + buf * 2 * kTile;
+        const int key0 = step * kKeyBlock;
+        const bool skip = step < low || key0 + strict > q0w + 31;
+        if (!redo) open_step(step, buf, skip);
+        redo = false;
+        if (!skip) fwd_step<D, kCarryOnly, false>(ktile, ktile + kTile, lo, qf, oacc, R, lane, key0, q0w, qi, strict);
+        wait_global_memory();
+        __syncthreads();
+    }
+
+    // ---- segment totals -> F (what this group's results are relative to) and rem
+    if (h == 0) totals[grp][32 * qs + n] = R;
+    __syncthreads();
+    float F = 1.0f, all = 1.0f;
 #pragma unroll
-                for (int c = 0; c < 4; ++c) pf[c] = pack8(&x[8 * c]);
+    for (int g = 0; g < G; ++g) {
+        const float t = totals[g][32 * qs + n];
+        if (g < grp) F *= t;
+        all *= t;
+    }
+    // carry-table entries of this group, written relative to its own right edge: times F.  Both
+    // half-waves take part (alternate steps); the loads go out in batches so that their
+    // latencies overlap.  The entries were written by this wave; its stores have completed
+    // (every iteration ends with a wait for all of the wave's memory traffic).
+    if (p.save && grp > 0 && qi < job.len) {
+        for (int s0 = low + h; s0 < hi; s0 += 8) {
+            float v[4];
 #pragma unroll
-                for (int c2 = 0; c2 < 2; ++c2) {   // operands of two key groups requested together, ahead of their MFMAs
-                    bf16x8 vt[2][D / 32];
+            for (int j = 0; j < 4; ++j)
+                if (s0 + 2 * j < hi) v[j] = p.rtab[tabq + (s0 + 2 * j) * kRowBlock];
 #pragma unroll
-                    for (int cc = 0; cc < 2; ++cc)
-#pragma unroll
-                        for (int db = 0; db < D / 32; ++db) vt[cc][db] = fetch_cols_o<D>(vtile, lo, db, 2 * c2 + cc);
-                    __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-                    for (int cc = 0; cc < 2; ++cc)
-#pragma unroll
-                        for (int db = 0; db < D / 32; ++db) oacc[db] = mfma(vt[cc][db], pf[2 * c2 + cc], oacc[db]);
-                }
-            }
+            for (int j = 0; j < 4; ++j)
+                if (s0 + 2 * j < hi) p.rtab[tabq + (s0 + 2 * j) * kRowBlock] = v[j] * F;
         }
-        wait_global_memory();                  // the next tiles have landed
-        __syncthreads();
     }
     if (kCarryOnly) return;
 
-    // ---- O = O(group 0) + O(group 1): group 1 parks its accumulators in LDS
-    float* park = (float*)lds;                              // [qs][db][r][lane]
-    if (grp == 1) {
+    // ---- O = sum_g F_g O_g: groups 1.. park their scaled accumulators in LDS (the tiles are free
+    // since the last barrier of the sweep), group 0 adds them up
+    float* park = (float*)lds;                              // [grp - 1][qs][db][r][lane]
+    if (grp > 0) {
 #pragma unroll
         for (int db = 0; db < D / 32; ++db)
 #pragma unroll
-            for (int r = 0; r < 16; ++r) park[((qs * (D / 32) + db) * 16 + r) * 64 + lane] = oacc[db][r];
+            for (int r = 0; r < 16; ++r)
+                park[((((grp - 1) * 4 + qs) * (D / 32) + db) * 16 + r) * 64 + lane] = oacc[db][r] * F;
     }
     __syncthreads();
     if (grp == 0 && qi < job.len) {
-        const int64_t obase = (int64_t)job.seq * p.o.sb + (int64_t)head * p.o.sh + (int64_t)(job.tok0 + qi) * p.o.st;
 #pragma unroll
-        for (int db = 0; db < D / 32; ++db) {
+        for (int g = 1; g < G; ++g)
 #pragma unroll
-            for (int r = 0; r < 16; ++r) oacc[db][r] += park[((qs * (D / 32) + db) * 16 + r) * 64 + lane];
+            for (int db = 0; db < D / 32; ++db)
 #pragma unroll
-            for (int g = 0; g < 4; ++g) {
-                f32x2 a = {oacc[db][4 * g], oacc[db][4 * g + 1]};
-                f32x2 b = {oacc[db][4 * g + 2], oacc[db][4 * g + 3]};
-                bf16x2 pa = __builtin_convertvector(a, bf16x2), pb = __builtin_convertvector(b, bf16x2);
-                uint2 w;
-                w.x = __builtin_bit_cast(uint32_t, pa);
-                w.y = __builtin_bit_cast(uint32_t, pb);
-                *(uint2*)(p.o.ptr + 2 * (obase + 32 * db + 8 * g + 4 * h)) = w;
-            }
-        }
+                for (int r = 0; r < 16; ++r)
+                    oacc[db][r] += park[((((g - 1) * 4 + qs) * (D / 32) + db) * 16 + r) * 64 + lane];
+        store_o_row<D>(p, job, head, qi, lane, oacc);
         if (h == 0)
-            Elem<uint16_t>::store(p.rem.ptr, (int64_t)job.seq * p.rem.sb + (int64_t)head * p.rem.sh + job.tok0 + qi, R);
+            Elem<uint16_t>::store(p.rem.ptr, (int64_t)job.seq * p.rem.sb + (int64_t)head * p.rem.sh + job.tok0 + qi, all);
     }
 }
 
 }  // namespace sba
 
+// Groups per workgroup of the segmented forward (SBA_FWD_GROUPS overrides it for experiments;
+// read once per process).
+static int sba_fwd_groups() {
+    static const int v = [] {
+        const char* e = getenv("SBA_FWD_GROUPS");
+        const int g = e ? atoi(e) : 4;
+        return g == 2 || g == 3 || g == 4 ? g : 4;
+    }();
+    return v;
+}
+
+template <bool kCarryOnly>
+static void launch_seg64(int groups, dim3 grid, hipStream_t s, const sba::KParams& kp) {
+    using namespace sba;
+    if (groups == 2) hipLaunchKernelGGL((mfma_fwd_seg_kernel<64, 2, kCarryOnly>), grid, dim3(2 * kThreads), 0, s, kp);
+    else if (groups == 3) hipLaunchKernelGGL((mfma_fwd_seg_kernel<64, 3, kCarryOnly>), grid, dim3(3 * kThreads), 0, s, kp);
+    else hipLaunchKernelGGL((mfma_fwd_seg_kernel<64, 4, kCarryOnly>), grid, dim3(4 * kThreads), 0, s, kp);
+}
+
 int sba_launch_mfma_fwd(const sba::KParams& kp, hipStream_t s) {
     using namespace sba;
     dim3 grid((unsigned)kp.n_jobs * kp.n_heads);
-    // A grid this small cannot give every SIMD more than two waves, and the launch lasts as long
-    // as its longest sweep: take the variant that halves that chain.  Larger grids are bound
-    // by throughput, where the 4-wave kernel (3 waves per SIMD) is ahead (measured: already at
-    // 640 workgroups).
+    // A grid this small cannot fill the SIMDs with one sweep per workgroup, and the launch lasts
+    // as long as its longest sweep: take the kernel that cuts every sweep into segments.  Larger
+    // grids are bound by throughput, where the 4-wave kernel (several workgroups per CU) is ahead.
     const bool small_grid = grid.x <= sba_two_step_max_grid();
-    if (kp.carry_only) {
-        if (kp.head_dim == 64 && small_grid)
-            hipLaunchKernelGGL((mfma_fwd2_kernel<64, true>), grid, dim3(2 * kThreads), 0, s, kp);
-        else if (kp.head_dim == 64)
-            hipLaunchKernelGGL((mfma_fwd_kernel<64, true>), grid, dim3(kThreads), 0, s, kp);
-        else
-            hipLaunchKernelGGL((mfma_fwd_kernel<128, true>), grid, dim3(kThreads), 0, s, kp);
-    } else if (kp.head_dim == 64 && small_grid)
-        hipLaunchKernelGGL((mfma_fwd2_kernel<64, false>), grid, dim3(2 * kThreads), 0, s, kp);
-    else if (kp.head_dim == 64)
-        hipLaunchKernelGGL((mfma_fwd_kernel<64, false>), grid, dim3(kThreads), 0, s, kp);
-    else
-        hipLaunchKernelGGL((mfma_fwd_kernel<128, false>), grid, dim3(kThreads), 0, s, kp);
+    if (kp.head_dim == 64 && small_grid) {
+        if (kp.carry_only) launch_seg64<true>(sba_fwd_groups(), grid, s, kp);
+        else launch_seg64<false>(sba_fwd_groups(), grid, s, kp);
+    } else if (kp.head_dim == 64) {
+        if (kp.carry_only) hipLaunchKernelGGL((mfma_fwd_kernel<64, true>), grid, dim3(kThreads), 0, s, kp);
+        else hipLaunchKernelGGL((mfma_fwd_kernel<64, false>), grid, dim3(kThreads), 0, s, kp);
+    } else {
+        if (kp.carry_only) hipLaunchKernelGGL((mfma_fwd_kernel<128, true>), grid, dim3(kThreads), 0, s, kp);
+        else hipLaunchKernelGGL((mfma_fwd_kernel<128, false>), grid, dim3(kThreads), 0, s, kp);
+    }
     return hipGetLastError() == hipSuccess ? SBA_OK : SBA_ERR_LAUNCH;
 }

@@ -452,12 +452,14 @@ def test_config3_size_packed_invariants():
     assert (o.float() + rem.float()[..., None] - 1).abs().max() <= 2e-2          # row mass
     starts = cu[:-1].long()
     assert rem[:, starts].float().min() == 1 and o[:, starts].abs().max() == 0   # first token of every document
-    # block-diagonal: one document cut out and run alone gives the same rows
+    # block-diagonal: one document cut out and run alone gives the same rows (to a rounding step
+    # of the bf16 outputs: alone, the document is a small launch and takes the segmented kernel,
+    # which adds its partial sums in another order)
     d = max(range(len(lens)), key=lambda i: lens[i])
     a, b = int(cu[d]), int(cu[d + 1])
     o_d, rem_d = sb_attn_varlen(q[:, a:b].contiguous(), k[:, a:b].contiguous(), ones[:, a:b].contiguous(),
                                 torch.tensor([0, b - a], dtype=torch.int32, device="cuda"), b - a)
-    assert torch.equal(o_d, o[:, a:b]) and torch.equal(rem_d, rem[:, a:b])
+    assert max_abs(o_d.float(), o[:, a:b].float()) <= 2 ** -7 and max_abs(rem_d.float(), rem[:, a:b].float()) <= 2 ** -7
     v = randn((H, N, D), 142, 0.5, torch.bfloat16).cuda()
     ups = [randn((H, N, D), 143 + i, 1.0, torch.bfloat16).cuda() for i in range(2)] + \
           [randn((H, N), 145 + i, 1.0, torch.bfloat16).cuda() for i in range(2)]
