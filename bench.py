@@ -19,12 +19,32 @@ if ROOT not in sys.path:
 BF16_MFMA_PEAK_TFLOPS = 2516.6     # 256 CU x 2.4 GHz x 4096 FLOP/clk/CU (dense bf16)
 
 KERNEL_TIMING_SAMPLES = 5      # steps of the timed region whose kernels are timed with events
-# HBM bytes per launch (read + write) from the rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs
-# summarised in profiles/sba_cfg{2,3,4}_hbm_traffic.txt (counters cannot be read from inside this
-# process).
-PROFILED_HBM_BYTES = {("cfg2", "fwd"): 42339771, ("cfg2", "bwd_dq"): 63414370, ("cfg2", "bwd_dkv"): 68069661,
-                      ("cfg3", "fwd"): 865755241, ("cfg3", "bwd_dq"): 990492784, ("cfg3", "bwd_dkv"): 1126127762,
-                      ("cfg4", "fwd"): 754136986, ("cfg4", "bwd_dq"): 1344713737, ("cfg4", "bwd_dkv"): 1401608381}
+# Counters cannot be read from inside this process: the figures below are copied from the rocprofv3
+# runs summarised under profiles/ (sba_cfg{2,3,4}_hbm_traffic.txt, sba_cfg{2,3,4}_shader_counters.txt) and
+# are reported with that source next to what this run measures itself.
+# HBM bytes per launch (FETCH_SIZE + WRITE_SIZE, scaled by a copy kernel of known size):
+PROFILED_HBM_BYTES = {("cfg2", "fwd"): 54341416, ("cfg2", "bwd_dq"): 62276476, ("cfg2", "bwd_dkv"): 68003005,
+                      ("cfg3", "fwd"): 909894854, ("cfg3", "bwd_dq"): 980533123, ("cfg3", "bwd_dkv"): 1121534757,
+                      ("cfg4", "fwd"): 639594244, ("cfg4", "bwd_dq"): 1381842591, ("cfg4", "bwd_dkv"): 1402182615}
+# wave instructions per launch: (vector incl. transcendental, transcendental, MFMA)
+PROFILED_INSTRUCTIONS = {("cfg2", "fwd"): (16467648, 2196480, 1064960), ("cfg2", "bwd_dq"): (30978048, 4259840, 1597440), ("cfg2", "bwd_dkv"): (37096628, 4292608, 2146304),
+                   ("cfg3", "fwd"): (125639104, 18584544, 9010688), ("cfg3", "bwd_dq"): (258147184, 36042752, 13516032), ("cfg3", "bwd_dkv"): (304725344, 35128320, 17564160),
+                   ("cfg4", "fwd"): (258899968, 34738176, 33685504), ("cfg4", "bwd_dq"): (530288640, 67371008, 50528256), ("cfg4", "bwd_dkv"): (631058432, 67371008, 67371008)}
+# issue time of one SIMD per instruction, ns, four waves per SIMD (profiles/gfx950_issue_rates.txt): plain vector,
+# transcendental issued while MFMAs are in flight, MFMA 32x32x16 bf16.  MFMAs and plain vector instructions do not
+# overlap on gfx950, so their times add up.
+ISSUE_NS = {"vector": 0.98, "transcendental": 0.97, "mfma": 17.0}
+N_SIMDS = 1024
+
+
+def issue_floor(workload, kernel):
+    """Secondary ceiling: the time the kernel's own instruction mix needs at the measured issue rates."""
+    c = PROFILED_INSTRUCTIONS.get((workload, kernel))
+    if c is None:
+        return None
+    valu, trans, mfma = c
+    ns = ((valu - trans) * ISSUE_NS["vector"] + trans * ISSUE_NS["transcendental"] + mfma * ISSUE_NS["mfma"]) / N_SIMDS
+    return ns * 1e-6      # ms
 
 
 def _lognormal_lengths(total, seed, median=600.0, sigma=1.0, lo=16, hi=4096):
@@ -89,29 +109,60 @@ def make_workload(name, device):
     raise SystemExit(f"unknown workload {name}")
 
 
-def cpu_baseline(name, budget_heads=16, reps=3):
-    """The oracle (a PyTorch restatement of the reference formula) timed on the host cores:
-    fwd+bwd of `budget_heads` heads of the cfg2 problem, scaled to TFLOP/s."""
+def cpu_baseline(name, reps=3):
+    """The oracle (a PyTorch restatement of the reference formula, oracle/sb_oracle.py) timed on
+    the host cores on a bounded sample of workload `name`, scaled to the metric's unit through
+    the same 12*d*P FLOP count.  cfg2: every head, full size.  cfg3: one head of the same packed
+    batch (all documents).  cfg4: one head of a 4096-token prefix at d=128 (the full 16384-token
+    head needs a 1 GiB score matrix per temporary)."""
     import torch
     from oracle import sb_oracle as O
+    # the GPU box gives one GPU's job 16 cores, whatever os.cpu_count() shows there
     torch.set_num_threads(min(os.cpu_count() or 1, 16))
-    T, D = 4096, 64
     g = torch.Generator().manual_seed(1)
-    q, k, v = ((torch.randn(1, budget_heads, T, D, generator=g) * 0.5).to(torch.bfloat16) for _ in range(3))
-    do = torch.randn(1, budget_heads, T, D, generator=g).to(torch.bfloat16)
-    O.sb_attn_grads_oracle(q[:, :1, :512], k[:, :1, :512], v[:, :1, :512], do[:, :1, :512])   # warm-up
+
+    def rn(shape, scale=0.5):
+        return (torch.randn(shape, generator=g) * scale).to(torch.bfloat16)
+
+    if name == "cfg3":
+        D, N = 64, 65536
+        lens = _lognormal_lengths(N, seed=0)
+        cu = [0]
+        for L in lens:
+            cu.append(cu[-1] + L)
+        q, k, v, do = rn((1, N, D)), rn((1, N, D)), rn((1, N, D)), rn((1, N, D), 1.0)
+        run = lambda: O.sb_attn_grads_oracle(q, k, v, do, None, cu_seqlens=cu)
+        pairs, full_pairs, tokens = sum(L * (L - 1) // 2 for L in lens), 16 * sum(L * (L - 1) // 2 for L in lens), N
+        what = f"1 of 16 heads of the cfg3 pack ({len(lens)} documents, 65536 tokens, d=64), document by document"
+    elif name == "cfg4":
+        T, D, Hs = 4096, 128, 8
+        q, k, v, do = rn((1, Hs, T, D)), rn((1, Hs, T, D)), rn((1, Hs, T, D), 1.0), rn((1, Hs, T, D), 1.0)
+
+        def run():
+            for h in range(Hs):
+                O.sb_attn_grads_oracle(q[:, h:h + 1], k[:, h:h + 1], v[:, h:h + 1], do[:, h:h + 1])
+        pairs, full_pairs, tokens = Hs * T * (T - 1) // 2, 16 * 16384 * 16383 // 2, 16384
+        what = "8 heads of a 4096-token prefix at d=128 (1/32 of cfg4's pairs: T=16384 needs 1 GiB per score matrix)"
+    else:
+        T, D, H = 4096, 64, 16
+        q, k, v, do = rn((1, H, T, D)), rn((1, H, T, D)), rn((1, H, T, D)), rn((1, H, T, D), 1.0)
+
+        def run():
+            for h in range(H):
+                O.sb_attn_grads_oracle(q[:, h:h + 1], k[:, h:h + 1], v[:, h:h + 1], do[:, h:h + 1])
+        pairs, full_pairs, tokens = H * T * (T - 1) // 2, H * T * (T - 1) // 2, T
+        what = "all 16 heads of cfg2 (T=4096, d=64), one head at a time"
+    D = q.shape[-1]
+    O.sb_attn_grads_oracle(rn((1, 1, 256, D)), rn((1, 1, 256, D)), rn((1, 1, 256, D)), rn((1, 1, 256, D)))   # warm-up
     t0 = time.perf_counter()
     for _ in range(reps):
-        for h in range(budget_heads):
-            O.sb_attn_grads_oracle(q[:, h:h + 1], k[:, h:h + 1], v[:, h:h + 1], do[:, h:h + 1])
+        run()
     dt = (time.perf_counter() - t0) / reps
-    pairs = budget_heads * T * (T - 1) // 2
     return {"value": round(12 * D * pairs / dt / 1e12, 5), "unit": "TFLOP/s", "cores": torch.get_num_threads(),
-            "kind": "port",
-            "sample": f"oracle/sb_oracle.py (torch fp32) fwd+bwd of {budget_heads} of 16 heads of cfg2 "
-                      f"(T=4096, d=64), one head at a time, {reps} repetitions, {dt:.2f} s each; "
+            "kind": "port", "workload": name,
+            "sample": f"oracle/sb_oracle.py (torch fp32) fwd+bwd of {what}, {reps} repetitions, {dt:.2f} s each; "
                       f"same 12*d*P FLOP count",
-            "tokens_per_s": round(T / (dt * 16 / budget_heads), 1)}
+            "tokens_per_s": round(tokens / (dt * full_pairs / pairs), 1)}
 
 
 def settle_clocks(step, seconds=0.3):
@@ -248,8 +299,19 @@ def main():
         "roofline": {"bound": "mfma", "kernel": dom, "achieved": round(achieved, 2),
                      "peak": BF16_MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
                      "frac": round(achieved / BF16_MFMA_PEAK_TFLOPS, 4),
-                     "traffic": PROFILED_HBM_BYTES.get((args.workload, dom))},
+                     "traffic": PROFILED_HBM_BYTES.get((args.workload, dom)),
+                     "traffic_source": f"profiles/sba_{args.workload}_hbm_traffic.txt (rocprofv3 --pmc, not measured by this run)"},
     }
+    fl = issue_floor(args.workload, dom)
+    if fl is not None:
+        # what the dominant kernel could reach if only instruction issue limited it: MFMA time + vector time
+        out["issue_floor"] = {"kernel": dom, "floor_ms": round(fl, 4), "measured_ms": round(kern[dom], 4),
+                              "frac_of_floor_rate": round(fl / kern[dom], 3),
+                              "tflops_at_floor": round(per_kernel_flops / (fl * 1e-3) / 1e12, 1),
+                              "frac_of_mfma_peak_at_floor": round(per_kernel_flops / (fl * 1e-3) / 1e12 / BF16_MFMA_PEAK_TFLOPS, 4),
+                              "ns_per_instruction": ISSUE_NS,
+                              "source": f"instruction counts from profiles/sba_{args.workload}_shader_counters.txt, "
+                                        "issue rates from profiles/gfx950_issue_rates.txt"}
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(args.workload)
     print(json.dumps(out))
