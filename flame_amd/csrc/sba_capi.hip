@@ -62,6 +62,8 @@ size_t generic_acc_bytes(const SbaParams* p) {
     return (b + 255) & ~(size_t)255;
 }
 
+constexpr size_t kErrorWordBytes = 256;     // tail of the MFMA backward's scratch: the error word
+
 sba::TensorArg cvt(const SbaTensor& t) { return sba::TensorArg{(char*)t.ptr, t.stride_b, t.stride_h, t.stride_t}; }
 sba::VectorArg cvt(const SbaVector& t) { return sba::VectorArg{(char*)t.ptr, t.stride_b, t.stride_h}; }
 
@@ -76,6 +78,13 @@ int check_common(const SbaParams* p) {
         if (!p->schedule || p->n_schedule <= 0 || p->table_cols <= 0) return SBA_ERR_SCHEDULE;
     } else if (p->total_tokens != p->seq_len) {
         return SBA_ERR_SHAPE;
+    }
+    if (use_mfma(p)) {
+        // the matrix-core kernels move 16-byte chunks: aligned rows, outer strides in whole chunks
+        for (const SbaTensor* t : {&p->q, &p->k, &p->v, &p->o, &p->d_o, &p->dq, &p->dk, &p->dv}) {
+            if (!t->ptr) continue;          // presence is checked per direction
+            if (((uintptr_t)t->ptr & 15) || (t->stride_b & 7) || (t->stride_h & 7) || (t->stride_t & 7)) return SBA_ERR_SHAPE;
+        }
     }
     return SBA_OK;
 }
@@ -106,6 +115,7 @@ KParams make_kparams(const SbaParams* p) {
         kp.rmid = (float*)(bs + table_bytes(p));
         kp.gmid = (float*)(bs + 2 * table_bytes(p));
         if (!p->workspace) kp.rtab = (float*)(bs + 3 * table_bytes(p));   // recomputed by sba_bwd
+        kp.gave_up = (int*)(bs + (p->workspace ? 3 : 4) * table_bytes(p));
     } else if (bs) {
         kp.dkv32 = (float*)bs;
     }
@@ -140,7 +150,7 @@ const char* sba_error_string(int code) {
     switch (code) {
         case SBA_OK: return "ok";
         case SBA_ERR_NULL: return "a required pointer is NULL";
-        case SBA_ERR_SHAPE: return "bad shape: sizes must be positive, head_dim <= 128, dense total_tokens == seq_len";
+        case SBA_ERR_SHAPE: return "bad shape: sizes must be positive, head_dim <= 128, dense total_tokens == seq_len; bf16 at head_dim 64 / 128 needs 16-byte aligned pointers and strides that are multiples of 8 elements";
         case SBA_ERR_DTYPE: return "unsupported dtype (float32 and bfloat16 only)";
         case SBA_ERR_WORKSPACE: return "workspace / bwd_scratch missing or smaller than sba_workspace_bytes() / sba_bwd_scratch_bytes()";
         case SBA_ERR_SCHEDULE: return "packed layout needs a row-block schedule from sba_build_schedule()";
@@ -161,7 +171,7 @@ size_t sba_bwd_scratch_bytes(const SbaParams* p) {
     if (!p || p->n_heads <= 0 || p->seq_len <= 0 || p->head_dim <= 0 || p->head_dim > 128) return 0;
     if (p->cu_seqlens && p->table_cols <= 0 && use_mfma_bwd(p)) return 0;
     // without a workspace the backward recomputes the forward's table first, into a fourth slot
-    return use_mfma_bwd(p) ? (p->workspace ? 3 : 4) * table_bytes(p) : generic_acc_bytes(p);
+    return use_mfma_bwd(p) ? (p->workspace ? 3 : 4) * table_bytes(p) + kErrorWordBytes : generic_acc_bytes(p);
 }
 
 int sba_row_block(void) { return sba::kRowBlock; }

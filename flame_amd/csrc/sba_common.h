@@ -10,8 +10,10 @@ namespace sba {
 constexpr int kRowBlock = 128;   // query rows per scheduled job (one workgroup)
 constexpr int kKeyBlock = 64;    // keys per sweep step of the MFMA kernels / carry-table column
 
-// Logits above this (in base-2 units) are clamped: sigmoid(z) differs from 1 by < 2^-30
-// there, so outputs move by < 1e-9, and exp2 of the clamped value cannot overflow.
+// Generic (fp32 / any head dim) kernels only: logits above this (in base-2 units) are clamped;
+// sigmoid(z) differs from 1 by < 2^-30 there, so outputs move by < 1e-9, and exp2 of the clamped
+// value cannot overflow.  The matrix-core kernels do not clamp: their product chains let
+// 1 + e^z overflow to +inf (see sba_mfma.h).
 constexpr float kMaxLogit2 = 30.0f;
 constexpr float kLog2e = 1.4426950408889634f;
 
@@ -33,6 +35,7 @@ struct KParams {
     float* rmid;                   // the same two carries in the MIDDLE of each 64-key block (entering
     float* gmid;                   //   its left / right 32 keys), written by the dQ pass
     float* dkv32;                  // generic path: fp32 dk|dv accumulators
+    int* gave_up;                  // backward error word (set if a kernel abandoned a bounded internal wait)
     int64_t tab_head_stride;       // floats per head in each carry table
     int64_t tab_tokens;            // generic path: tokens per head in the fp32 accumulators (n_seq*T dense, sumT packed)
 };

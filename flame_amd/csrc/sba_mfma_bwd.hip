@@ -47,6 +47,7 @@ __global__ __launch_bounds__(kThreads) void mfma_bwd_dq_kernel(KParams p) {
     const int64_t vbase = (int64_t)job.seq * p.v.sb + (int64_t)head * p.v.sh + (int64_t)job.tok0 * p.v.st;
     const int64_t dobase = (int64_t)job.seq * p.d_o.sb + (int64_t)head * p.d_o.sh + (int64_t)job.tok0 * p.d_o.st;
 
+    if (blockIdx.x == 0 && threadIdx.x == 0 && p.gave_up) *p.gave_up = 0;     // error word of the launch pair, see wait_for_count()
     bf16x8 qf[D / 16], dof[D / 16];
     load_row_frags<D>(qf, p.q, qbase, qi, job.len, lane);
     load_row_frags<D>(dof, p.d_o, dobase, qi, job.len, lane);
@@ -195,6 +196,7 @@ __global__ __launch_bounds__(2 * kThreads, 2) void mfma_bwd_dq2_kernel(KParams p
     const int64_t vbase = (int64_t)job.seq * p.v.sb + (int64_t)head * p.v.sh + (int64_t)job.tok0 * p.v.st;
     const int64_t dobase = (int64_t)job.seq * p.d_o.sb + (int64_t)head * p.d_o.sh + (int64_t)job.tok0 * p.d_o.st;
 
+    if (blockIdx.x == 0 && threadIdx.x == 0 && p.gave_up) *p.gave_up = 0;     // error word of the launch pair, see wait_for_count()
     bf16x8 qf[D / 16], dof[D / 16];
     load_row_frags<D>(qf, p.q, qbase, qi, job.len, lane);
     load_row_frags<D>(dof, p.d_o, dobase, qi, job.len, lane);
@@ -511,6 +513,20 @@ __global__ __launch_bounds__(kThreads, 2) void mfma_bwd_dkv_kernel(KParams p) {
 // the current item's K fragments.
 // An item's accumulators are complete after the reduction that follows its last step; they are
 // staged after that iteration's B and written to global memory before the next iteration's B.
+// The stream kernel's two internal waits are on counters in LDS that waves of the same
+// (resident) workgroup bump, so they end within microseconds.  They are bounded all the same: a
+// wave that has slept through kSpinLimit polls stops waiting, raises the launch's error word
+// (KParams::gave_up, the last 256 bytes of the backward scratch) and runs on, so that the kernel
+// always drains; its results are then meaningless.
+constexpr int kSpinLimit = 1 << 22;            // polls of 64+ clocks each: more than 0.1 s
+__device__ inline void wait_for_count(int* counter, int target, int* gave_up) {
+    for (int i = 0; i < kSpinLimit; ++i) {
+        if (__hip_atomic_load(counter, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) >= target) return;
+        __builtin_amdgcn_s_sleep(1);
+    }
+    if (gave_up && (threadIdx.x & 63) == 0) *gave_up = 1;
+}
+
 struct KeyItem {
     Job job;
     int head, kb, key0, n_steps;
@@ -818,14 +834,13 @@ __global__ __launch_bounds__(2 * kThreads, 2) void mfma_bwd_dkv_stream_kernel(KP
         int fin_stage = cur_idx, fin_store = cur_idx;
         // B, a barrier of the four consumer waves only (the producers have no part in what it
         // protects and must not be held up by it): a running count in LDS, bumped by each wave,
-        // and a short spin.  All four waves are resident, so it terminates.
+        // and a short, bounded spin (all four waves are resident).
         int sync_target = 0;
         auto consumer_sync = [&]() {
             sync_target += 4;
             __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
             if (lane == 0) __hip_atomic_fetch_add(&consumers_done, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
-            while (__hip_atomic_load(&consumers_done, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) < sync_target)
-                __builtin_amdgcn_s_sleep(1);
+            wait_for_count(&consumers_done, sync_target, p.gave_up);
             __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
         };
         // One iteration of the stream; `rq`, `rq_row0` say what the stream's next step needs.
@@ -848,8 +863,7 @@ __global__ __launch_bounds__(2 * kThreads, 2) void mfma_bwd_dkv_stream_kernel(KP
             if (finish_after_reduce) consumer_sync();
             if (keys_now) {
                 // the K tile is free once every producer holds this item's fragments
-                while (__hip_atomic_load(&producers_took_k, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) < 4 * (item + 1))
-                    __builtin_amdgcn_s_sleep(1);
+                wait_for_count(&producers_took_k, 4 * (item + 1), p.gave_up);
                 __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
                 request_keys(decode_item(p, nxt_idx), vtiles + ((item + 1) & 1) * kTile);
             }

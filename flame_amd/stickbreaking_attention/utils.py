@@ -5,14 +5,11 @@ registered form is taken only while ``torch.compile`` is tracing, so that the ct
 into the HIP library is an opaque node of the graph."""
 from __future__ import annotations
 
-import math
 from typing import Callable, Iterable
 
 import torch
 
 PACKAGE_NAME = "stickbreaking_attention"
-log2 = math.log(2)
-inv_log2 = 1 / log2
 
 
 def _dispatch(func: Callable, compileable_fn: Callable, *args, **kwargs):

@@ -2,9 +2,12 @@
  * C ABI of libsba_mi355x.so: stick-breaking attention for AMD MI355X (gfx950).
  *
  * Plain pointers and sizes only; no torch types.  All tensor pointers are device
- * pointers (HIP), all launches are asynchronous on `stream`, nothing is allocated,
- * nothing synchronises, and no global state is kept, so every entry point may be called
- * from any thread.  Return value: 0 on success, a negative SBA_ERR_* code otherwise
+ * pointers (HIP), all launches are asynchronous on `stream`, nothing is allocated and
+ * nothing synchronises, so every entry point may be called from any thread.  Process-wide
+ * state: the compute-unit count of each device and the address of sba_bwd_static()'s array are
+ * looked up once and kept; the SBA_* environment switches (experiments and tests only) are read
+ * when a call dispatches, so they must not change between an sba_fwd and the sba_bwd that
+ * consumes its workspace.  Return value: 0 on success, a negative SBA_ERR_* code otherwise
  * (sba_error_string() gives the text).
  *
  * The reference has no native code; what each entry point replaces is the Python host
@@ -22,7 +25,9 @@
  *   packed [H, sumT, D]  : n_seq = number of documents, cu_seqlens = device int32[n_seq+1]
  *                          with cu_seqlens[0] == 0, stride_b = 0,
  *                          element (h,t,d) at    base + h*stride_h + t*stride_t + d
- * Strides are in elements; the innermost (D) stride is 1.
+ * Strides are in elements; the innermost (D) stride is 1.  bf16 problems at head_dim 64 / 128
+ * (the matrix-core kernels) need 16-byte aligned tensor pointers and outer strides that are
+ * multiples of 8 elements (SBA_ERR_SHAPE otherwise); rem / d_rem are contiguous along tokens.
  */
 #ifndef SBA_MI355X_H
 #define SBA_MI355X_H
@@ -120,7 +125,9 @@ size_t sba_workspace_bytes(const SbaParams* p);
  * Bytes of device memory sba_bwd needs for the duration of the call only (three more
  * tables between its two kernels, or the generic path's fp32 accumulators): allocate before
  * the call, free after it has run.  With bwd_phases 1 and 2 issued as two calls, the same
- * buffer goes to both.
+ * buffer goes to both.  For bf16 at head_dim 64 / 128 the last 256 bytes hold an error word
+ * (int32): the backward clears it and sets it to 1 if a kernel abandoned one of its bounded
+ * internal waits (the results are then invalid); a caller may read it after synchronising.
  *
  * Memory-lean mode: a forward run WITHOUT save_for_backward keeps nothing, and sba_bwd called
  * with workspace = NULL first repeats the forward's sweep for the carries alone (about 0.7 of

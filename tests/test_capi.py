@@ -52,6 +52,36 @@ def test_argument_checks_without_gpu(lib):
     assert lib.sba_row_block() == 128
 
 
+def test_error_codes_of_the_call_sequence_without_gpu(lib):
+    # every check below fails before anything is launched
+    p = _lib.SbaParams()
+    p.struct_size = C.sizeof(_lib.SbaParams)
+    p.dtype = _lib.SBA_DTYPE_BF16
+    p.n_seq, p.n_heads, p.seq_len, p.total_tokens, p.head_dim = 1, 2, 256, 256, 64
+    for t in ("q", "k", "v", "o", "d_o", "dq", "dk", "dv"):
+        getattr(p, t).ptr = 256
+        getattr(p, t).stride_h, getattr(p, t).stride_t = 256 * 64, 64
+    p.rem.ptr = 256
+    p.save_for_backward = 1
+    assert lib.sba_fwd(C.byref(p)) == -4                      # SBA_ERR_WORKSPACE: no workspace given
+    p.workspace, p.workspace_bytes = 256, lib.sba_workspace_bytes(C.byref(p)) - 1
+    assert lib.sba_fwd(C.byref(p)) == -4                      # one byte short
+    assert lib.sba_bwd(C.byref(p)) == -4                      # the backward checks it too
+    p.workspace_bytes += 1
+    assert lib.sba_bwd(C.byref(p)) == -4                      # and its own scratch
+    assert b"sba_bwd_scratch_bytes" in lib.sba_error_string(-4)
+    p.q.ptr = 264                                             # not 16-byte aligned
+    assert lib.sba_fwd(C.byref(p)) == -2
+    p.q.ptr, p.k.stride_t = 256, 68                           # stride not a multiple of 8 elements
+    assert lib.sba_fwd(C.byref(p)) == -2
+    p.k.stride_t = 64
+    p.cu_seqlens = 256                                        # packed layout ...
+    assert lib.sba_fwd(C.byref(p)) == -5                      # ... without a schedule: SBA_ERR_SCHEDULE
+    p.schedule, p.n_schedule = 256, 2
+    assert lib.sba_fwd(C.byref(p)) == -5                      # ... without the table size
+    assert b"sba_build_schedule" in lib.sba_error_string(-5)
+
+
 def test_workspace_bytes(lib):
     p = _lib.SbaParams()
     p.struct_size = C.sizeof(_lib.SbaParams)
@@ -61,9 +91,9 @@ def test_workspace_bytes(lib):
     # 32 * 33 columns of 128 floats at T = 4096 (half of a full [T/64][T] rectangle, plus the diagonal)
     table = 16 * 32 * 33 * 128 * 4
     assert lib.sba_workspace_bytes(C.byref(p)) == table          # what the forward hands to the backward
-    assert lib.sba_bwd_scratch_bytes(C.byref(p)) == 4 * table    # no workspace: the backward recomputes that table
+    assert lib.sba_bwd_scratch_bytes(C.byref(p)) == 4 * table + 256    # no workspace: the backward recomputes that table (+ error word)
     p.workspace = 1
-    assert lib.sba_bwd_scratch_bytes(C.byref(p)) == 3 * table    # what the backward needs for itself
+    assert lib.sba_bwd_scratch_bytes(C.byref(p)) == 3 * table + 256    # what the backward needs for itself
     p.workspace = None
     p.dtype = _lib.SBA_DTYPE_F32                    # generic kernels: nothing kept, fp32 dk|dv accumulators
     assert lib.sba_workspace_bytes(C.byref(p)) == 0

@@ -121,3 +121,31 @@ def test_torch_compile_fullgraph_on_the_layer_dense_and_packed():
         kw_ref = {k_: (v_.cpu() if torch.is_tensor(v_) else v_) for k_, v_ in kw.items()}
         o_ref = ref(x.float().cpu(), **kw_ref)[0]
         assert max_abs(comp[0].float().cpu(), o_ref) <= 3e-2
+
+
+def test_hf_auto_model_from_config_trains_one_step_on_the_gpu():
+    # the route flame's trainer takes for a custom model: AutoModelForCausalLM.from_config on the
+    # registered 'sba' config (flame/train.py:66-67, custom_models/sba/__init__.py:7-9)
+    from transformers import AutoModelForCausalLM
+    import flame_amd.hf as hf
+    torch.manual_seed(0)
+    cfg = hf.SBAConfig(hidden_size=256, num_hidden_layers=2, num_heads=4, vocab_size=512)
+    model = AutoModelForCausalLM.from_config(cfg).cuda()
+    assert isinstance(model, hf.SBAForCausalLM)
+    opt = torch.optim.AdamW(model.parameters(), lr=1e-3)
+    ids = torch.randint(0, 512, (1, 384), device="cuda")
+    cu = torch.tensor([0, 100, 101, 300, 384], dtype=torch.int32, device="cuda")
+    losses = []
+    for _ in range(3):
+        with torch.autocast("cuda", dtype=torch.bfloat16):
+            out = model(input_ids=ids, labels=ids, cu_seqlens=cu, max_seqlen=199)
+        opt.zero_grad()
+        out.loss.backward()
+        assert all(torch.isfinite(p.grad).all() for p in model.parameters())
+        opt.step()
+        losses.append(float(out.loss))
+    print("hf losses", losses, flush=True)
+    assert losses[-1] < losses[0]
+    # and the dense route
+    with torch.autocast("cuda", dtype=torch.bfloat16):
+        assert torch.isfinite(model(input_ids=ids.view(2, 192), labels=ids.view(2, 192)).loss)

@@ -82,3 +82,35 @@ def test_context_len_rechunking():
     cu = torch.tensor([0, 10, 13, 30], dtype=torch.int32)
     assert split_by_context_len(cu, 8).tolist() == [0, 8, 10, 13, 21, 29, 30]
     assert cu_seqlens_from_tokens(torch.tensor([1] + [3] * 19), bos_token_id=1, context_len=8).tolist() == [0, 8, 16, 20]
+
+
+def test_hf_registration_and_340m_config_values():
+    # custom_models/sba/__init__.py:7-9: importing the package registers model_type 'sba'
+    import json
+    from transformers import AutoConfig, AutoModel, AutoModelForCausalLM
+    import flame_amd.hf as hf
+    # the values of the reference's configs/sba_340m.json (the file itself is not part of this tree)
+    sba_340m = {"attention_bias": False, "bos_token_id": 1, "eos_token_id": 2, "fuse_cross_entropy": True,
+                "fuse_norm": True, "hidden_act": "swish", "hidden_size": 1024, "initializer_range": 0.006,
+                "max_position_embeddings": 8192, "model_type": "sba", "num_heads": 16, "num_hidden_layers": 24,
+                "norm_eps": 1e-06, "tie_word_embeddings": False, "use_cache": True, "vocab_size": 32000}
+    cfg = AutoConfig.for_model(**json.loads(json.dumps(sba_340m)))
+    assert isinstance(cfg, hf.SBAConfig) and cfg.model_type == "sba"
+    assert (cfg.hidden_size, cfg.num_heads, cfg.num_hidden_layers, cfg.vocab_size) == (1024, 16, 24, 32000)
+    assert cfg.mlp_width() == 2816 and cfg.hidden_ratio == 4 and cfg.norm_eps == 1e-6
+    small = hf.SBAConfig(hidden_size=64, num_hidden_layers=2, num_heads=2, vocab_size=97)
+    lm = AutoModelForCausalLM.from_config(small)
+    assert isinstance(lm, hf.SBAForCausalLM) and isinstance(AutoModel.from_config(small), hf.SBAModel)
+    # weights are N(0, initializer_range)
+    assert abs(float(lm.model.layers[0].attn.q_proj.weight.std()) - 0.006) < 1e-3
+    # same wiring as the plain model: the oracle attention in both, equal losses for equal weights
+    for layer in lm.model.layers:
+        layer.attn.attn_fn = lambda q, k, v, t: O.sb_attn_oracle(q, k, v)
+        layer.attn.attn_varlen_fn = lambda q, k, v, cu, ml: O.sb_attn_varlen_oracle(q, k, v, cu)
+    plain = _oracle_model(SBAConfig(hidden_size=64, num_hidden_layers=2, num_heads=2, vocab_size=97))
+    plain.load_state_dict(lm.state_dict())
+    ids = torch.randint(0, 97, (1, 40))
+    cu = torch.tensor([0, 17, 40])
+    out = lm(input_ids=ids, labels=ids, cu_seqlens=cu)
+    loss_plain, logits_plain = plain(ids, labels=ids, cu_seqlens=cu)
+    assert torch.allclose(out.logits, logits_plain, atol=1e-5) and torch.allclose(out.loss, loss_plain, atol=1e-6)
