@@ -31,6 +31,21 @@ typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
 
 constexpr int kThreads = 256;
 
+// Row fragments multiplied by the logit scale once, ahead of the sweep (fp32 product, rounded
+// back to bf16): the score MFMAs then deliver base-2 logits directly and the per-element
+// multiplication disappears from every step.  Costs one more bf16 rounding of q (relative
+// 2^-9 per element, the size of the rounding the inputs already carry).
+template <int NF> __device__ inline void prescale_frags(bf16x8 (&f)[NF], float s) {
+#pragma unroll
+    for (int ks = 0; ks < NF; ++ks)
+#pragma unroll
+        for (int i = 0; i < 8; i += 2) {
+            const f32x2 v = {(float)f[ks][i] * s, (float)f[ks][i + 1] * s};
+            const bf16x2 b = __builtin_convertvector(v, bf16x2);
+            f[ks][i] = b[0]; f[ks][i + 1] = b[1];
+        }
+}
+
 __device__ inline int mfma_row_of_key(int kl) {   // key_local -> LDS row
     return ((kl >> 4) & 1) * 32 + ((kl >> 2) & 3) * 8 + (kl >> 5) * 4 + (kl & 3);
 }
@@ -161,6 +176,14 @@ template <int D> struct TileCopy {
                 if (row0 + kl + r * kRowStep < len) v = *(const u32x4*)(tile_base + (size_t)(lane_off + r * step_off));
                 regs[r] = v;
             }
+        }
+    }
+    __device__ inline void scale(float f) {      // every bf16 of the tile times f (fp32 product, rounded back)
+#pragma unroll
+        for (int r = 0; r < kPerThread; ++r) {
+            bf16x8 b[1] = {__builtin_bit_cast(bf16x8, regs[r])};
+            prescale_frags(b, f);
+            regs[r] = __builtin_bit_cast(u32x4, b[0]);
         }
     }
     __device__ inline void store(char* tile) const {
@@ -327,20 +350,6 @@ __device__ inline void score_tiles_o(float (&x)[32], const char* ktile, const La
     scale_scores(x, raw, scale2);
 }
 
-// Row fragments multiplied by the logit scale once, ahead of the sweep (fp32 product, rounded
-// back to bf16): the score MFMAs then deliver base-2 logits directly and the per-element
-// multiplication disappears from every step.  Costs one more bf16 rounding of q (relative
-// 2^-9 per element, the size of the rounding the inputs already carry).
-template <int NF> __device__ inline void prescale_frags(bf16x8 (&f)[NF], float s) {
-#pragma unroll
-    for (int ks = 0; ks < NF; ++ks)
-#pragma unroll
-        for (int i = 0; i < 8; i += 2) {
-            const f32x2 v = {(float)f[ks][i] * s, (float)f[ks][i + 1] * s};
-            const bf16x2 b = __builtin_convertvector(v, bf16x2);
-            f[ks][i] = b[0]; f[ks][i + 1] = b[1];
-        }
-}
 // Score tiles from pre-scaled fragments: x[16*t + r] = raw accumulator, no vector work.
 template <int D, bool kBatch = (D == 128)>
 __device__ inline void score_tiles_ps(float (&x)[32], const char* ktile, const LaneOffsets<D>& o,

@@ -50,6 +50,7 @@ __global__ __launch_bounds__(kThreads) void mfma_bwd_dq_kernel(KParams p) {
     if (blockIdx.x == 0 && threadIdx.x == 0 && p.gave_up) *p.gave_up = 0;     // error word of the launch pair, see wait_for_count()
     bf16x8 qf[D / 16], dof[D / 16];
     load_row_frags<D>(qf, p.q, qbase, qi, job.len, lane);
+    prescale_frags(qf, p.scale2);          // the score MFMAs then deliver base-2 logits
     load_row_frags<D>(dof, p.d_o, dobase, qi, job.len, lane);
     float dr = 0.f;
     if (row_ok && p.d_rem.ptr)
@@ -106,7 +107,7 @@ __global__ __launch_bounds__(kThreads) void mfma_bwd_dq_kernel(KParams p) {
         if (!skip) {
             float x[32], beta[32], dp[32];
             float Rlane, Glane;
-            score_tiles_o<D>(x, ktile, lo, qf, p.scale2);
+            score_tiles_ps<D>(x, ktile, lo, qf);
             if (key0 + 63 + strict > q0w) {
 mask_step(x, key0 + 32 * h, qi, strict);
             }
@@ -199,6 +200,7 @@ __global__ __launch_bounds__(2 * kThreads, 2) void mfma_bwd_dq2_kernel(KParams p
     if (blockIdx.x == 0 && threadIdx.x == 0 && p.gave_up) *p.gave_up = 0;     // error word of the launch pair, see wait_for_count()
     bf16x8 qf[D / 16], dof[D / 16];
     load_row_frags<D>(qf, p.q, qbase, qi, job.len, lane);
+    prescale_frags(qf, p.scale2);          // the score MFMAs then deliver base-2 logits
     load_row_frags<D>(dof, p.d_o, dobase, qi, job.len, lane);
     float dr = 0.f;
     if (row_ok && p.d_rem.ptr)
@@ -253,7 +255,7 @@ __global__ __launch_bounds__(2 * kThreads, 2) void mfma_bwd_dq2_kernel(KParams p
         float x[32], beta[32], dp[32];
         float total = 0.f, start = 0.f, Rlane = 1.f;
         if (active) {
-            score_tiles_o<D, true>(x, ktile, lo, qf, p.scale2);
+            score_tiles_ps<D, true>(x, ktile, lo, qf);
             if (key0 + 63 + strict > q0w) mask_step(x, key0 + 32 * h, qi, strict);
             float Rc = R;
             stick_weights_and_dp<D>(x, beta, dp, Rc, lane, &Rlane, vtile, lo, dof);
@@ -380,6 +382,7 @@ __global__ __launch_bounds__(kThreads, 2) void mfma_bwd_dkv_kernel(KParams p) {
         TileCopy<D> kc, vc;
         kc.load(p.k, kbase, key0, job.len);
         vc.load(p.v, vbase, key0, job.len);
+        kc.scale(p.scale2);                    // K times the logit scale: the score MFMAs deliver base-2 logits
         kc.store(ktile);
         vc.store(vtile);
     }
@@ -434,7 +437,7 @@ __global__ __launch_bounds__(kThreads, 2) void mfma_bwd_dkv_kernel(KParams p) {
         const bool skip = key0 + strict > q0w + 31 || q0w >= job.len;
         if (!skip) {
             float beta[32];
-            score_tiles_o<D>(x, ktile, lo, qf, p.scale2);
+            score_tiles_ps<D>(x, ktile, lo, qf);
             if (key0 + 63 + strict > q0w) mask_step(x, key0 + 32 * h, qi, strict);
             stick_weights<true>(x, beta, R, lane);
 #pragma unroll
@@ -604,6 +607,7 @@ __global__ __launch_bounds__(2 * kThreads, 2) void mfma_bwd_dkv_stream_kernel(KP
                     kfr[t][ks] = fetch_rows_o<D>(ktile, lo, t, ks);
                     vfr[t][ks] = fetch_rows_o<D>(vtile, lo, t, ks);
                 }
+
             // tell the consumers that the K tile may be refilled
             __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
             if (lane == 0) __hip_atomic_fetch_add(&producers_took_k, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
@@ -643,7 +647,10 @@ __global__ __launch_bounds__(2 * kThreads, 2) void mfma_bwd_dkv_stream_kernel(KP
                         for (int ks = 0; ks < D / 16; ++ks) acc = mfma(kfr[t][ks], qf[ks], acc);
                         raw[t] = acc;
                     }
-                    scale_scores(x, raw, p.scale2);
+#pragma unroll
+                    for (int t = 0; t < 2; ++t)
+#pragma unroll
+                        for (int r = 0; r < 16; ++r) x[16 * t + r] = raw[t][r] * p.scale2;
                     if (key0 + 63 + strict > q0w) mask_step(x, key0 + 32 * h, qi, strict);
                     // dP = dO V^T does not depend on the weights: its eight MFMAs go between the
                     // segments of the chain, where the chain's exp/rcp overlap them
@@ -985,6 +992,7 @@ __global__ __launch_bounds__(kThreads, D == 64 ? 2 : 1) void mfma_bwd_dkv_own_ke
         const int key = kb0 + 16 * ((m >> 2) & 1) + 4 * (m >> 3) + (m & 3);
         load_row_frags<D>(kfr, p.k, kbase, key, job.len, lane);
         load_row_frags<D>(vfr, p.v, vbase, key, job.len, lane);
+        prescale_frags(kfr, p.scale2);         // K times the logit scale: the score MFMAs deliver base-2 logits
     }
 
     f32x16 dkacc[D / 32], dvacc[D / 32];
@@ -1075,7 +1083,7 @@ __global__ __launch_bounds__(kThreads, D == 64 ? 2 : 1) void mfma_bwd_dkv_own_ke
 #pragma unroll
                     for (int ks = 0; ks < D / 16; ++ks) acc = mfma(kfr[ks], bq[ks], acc);
 #pragma unroll
-                    for (int r = 0; r < 16; ++r) x[r] = acc[r] * p.scale2;
+                    for (int r = 0; r < 16; ++r) x[r] = acc[r];
                 }
                 if (kb0 + 31 + strict > qt0 || qt0 + 31 >= job.len) {     // diagonal or ragged tile
 #pragma unroll
