@@ -640,6 +640,45 @@ __device__ inline void logit_grads(const float (&a)[32], const float (&beta)[32]
     }
 }
 
+// Register-lean form of the backward's per-step arithmetic for the row-owner kernel at head_dim
+// 128, where registers decide between one and two waves per SIMD: two arrays of 32 instead of
+// four.  Part 1 runs the reciprocal-per-key chain right-to-left and leaves, in place of the
+// logits, beta, and in place of dP, g' = a' * dP with a' the weight relative to the right edge of
+// the lane's 32 keys (the finished weight is F * a', F the carry entering the lane's keys, which
+// only the exchange after the chain supplies).  Returns the lane's product of (1 - beta) (clamped,
+// see product_chain) and in `gsum` the lane's sum of g'.  Part 2 walks left-to-right from the
+// prefix `G` entering the lane's keys:  t = F g',  G += t,  dz = t - beta G,  packed as it goes.
+__device__ inline float chain_beta_gprime(float (&x)[32], float (&dp)[32], float& gsum) {
+    float W = 1.0f, L = 1.0f, c = 0.f;
+#pragma unroll
+    for (int idx = 31; idx >= 0; --idx) {
+        const float e = __builtin_amdgcn_exp2f(x[idx]);
+        const float Wn = __builtin_fmaf(W, e, W);
+        const float Ln = __builtin_amdgcn_rcpf(Wn);
+        x[idx] = clamp01(__builtin_fmaf(-W, Ln, 1.0f));       // beta
+        dp[idx] = clamp01(L - Ln) * dp[idx];                  // g' (the clamps map the NaN of an overflowed chain to 0)
+        c += dp[idx];
+        W = Wn;
+        L = Ln;
+    }
+    gsum = c;
+    return clamp01(L);
+}
+// Out: zf[c] = dz of keys 8c .. 8c+7 packed to bf16 (the B operand of dQ^T += K^T dZ^T).
+__device__ inline void walk_logit_grads(const float (&beta)[32], const float (&g)[32], float F, float G, bf16x8 (&zf)[4]) {
+#pragma unroll
+    for (int c = 0; c < 4; ++c) {
+        float dz[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const float t = F * g[8 * c + i];
+            G += t;
+            dz[i] = __builtin_fmaf(-beta[8 * c + i], G, t);
+        }
+        zf[c] = pack8(dz);
+    }
+}
+
 // logit_grads in two parts (see stick_weights_local): part 1 forms g in place of dp and
 // returns this lane's offset inside the step (0 for the lower half-wave, the lower half's
 // sum for the upper) and, in `total`, the step's sum of g; part 2 applies the prefix.

@@ -26,7 +26,7 @@ namespace sba {
 
 // ---------------------------------------------------------------- pass 1: dQ + prefix table
 template <int D>
-__global__ __launch_bounds__(kThreads) void mfma_bwd_dq_kernel(KParams p) {
+__global__ __launch_bounds__(kThreads, 2) void mfma_bwd_dq_kernel(KParams p) {
     constexpr int kTile = 64 * D * 2;
     __shared__ __attribute__((aligned(16))) char lds[4 * kTile];   // K0 V0 K1 V1
 
@@ -105,30 +105,55 @@ __global__ __launch_bounds__(kThreads) void mfma_bwd_dq_kernel(KParams p) {
             vc.issue((step + 1) * kKeyBlock, job.len, lds + (buf ^ 1) * 2 * kTile + kTile);
         }
         if (!skip) {
-            float x[32], beta[32], dp[32];
-            float Rlane, Glane;
-            score_tiles_ps<D>(x, ktile, lo, qf);
-            if (key0 + 63 + strict > q0w) {
-mask_step(x, key0 + 32 * h, qi, strict);
-            }
-            // dP does not depend on the weights: its MFMAs go between the segments of the chain,
-            // where the chain's exp/rcp overlap them
-            stick_weights_and_dp<D>(x, beta, dp, R, lane, &Rlane, vtile, lo, dof);
-            // The gradient of rem rides in the prefix: g is formed from the plain dP, and the term
-            // -beta_ik * d_rem_i * rem_i that d_rem adds to dz_ik is a constant d_rem_i * rem_i in
-            // the running prefix.  After the leftmost block R is the product over all keys, rem_i.
-            if (step == 0) Gc = dr * R;
-            Genter = Gc;
-            g_pending = true;
-            logit_grads<false>(x, beta, dp, Gc, lane, &Glane);
-            // carries in the middle of the block, for the key-owner pass whose waves own 32 keys:
-            // the left half-wave holds the product entering the left 32 keys, the right half-wave
-            // the prefix entering the right 32 (stored at the top of the next iteration)
-            mid = h == 0 ? Rlane : Glane;
-            mid_pending = true;
             bf16x8 zf[4];
+            if constexpr (D == 128) {
+                // Register-lean arrangement (two arrays of 32 live instead of four: two waves per SIMD
+                // instead of one): scores and dP first, then the chain over both in place.
+                float x[32], dp[32];
+                score_tiles_ps<D>(x, ktile, lo, qf);
+                dp_tiles_o<D>(dp, vtile, lo, dof);
+                if (key0 + 63 + strict > q0w) mask_step(x, key0 + 32 * h, qi, strict);
+                float gsum;
+                const float L = chain_beta_gprime(x, dp, gsum);
+                float Llo, Lup;
+                half_values(L, Llo, Lup);
+                const float F = h ? R : R * Lup;         // the carry entering this lane's 32 keys
+                R = R * Llo * Lup;
+                if (step == 0) Gc = dr * R;              // the gradient of rem rides in the prefix, see below
+                Genter = Gc;
+                g_pending = true;
+                float clo, cup;
+                half_values(F * gsum, clo, cup);
+                const float Glane = h ? Gc + clo : Gc;   // the prefix entering this lane's 32 keys
+                Gc = Gc + clo + cup;
+                mid = h == 0 ? F : Glane;                // carries in the middle of the block, see below
+                mid_pending = true;
+                walk_logit_grads(x, dp, F, Glane, zf);
+            } else {
+                float x[32], beta[32], dp[32];
+                float Rlane, Glane;
+                score_tiles_ps<D>(x, ktile, lo, qf);
+                if (key0 + 63 + strict > q0w) {
+    mask_step(x, key0 + 32 * h, qi, strict);
+                }
+                // dP does not depend on the weights: its MFMAs go between the segments of the chain,
+                // where the chain's exp/rcp overlap them
+                stick_weights_and_dp<D>(x, beta, dp, R, lane, &Rlane, vtile, lo, dof);
+                // The gradient of rem rides in the prefix: g is formed from the plain dP, and the term
+                // -beta_ik * d_rem_i * rem_i that d_rem adds to dz_ik is a constant d_rem_i * rem_i in
+                // the running prefix.  After the leftmost block R is the product over all keys, rem_i.
+                if (step == 0) Gc = dr * R;
+                Genter = Gc;
+                g_pending = true;
+                logit_grads<false>(x, beta, dp, Gc, lane, &Glane);
+                // carries in the middle of the block, for the key-owner pass whose waves own 32 keys:
+                // the left half-wave holds the product entering the left 32 keys, the right half-wave
+                // the prefix entering the right 32 (stored at the top of the next iteration)
+                mid = h == 0 ? Rlane : Glane;
+                mid_pending = true;
 #pragma unroll
-            for (int c = 0; c < 4; ++c) zf[c] = pack8(&dp[8 * c]);
+                for (int c = 0; c < 4; ++c) zf[c] = pack8(&dp[8 * c]);
+            }
 #pragma unroll
             for (int c = 0; c < 4; ++c) {      // (operands of a key group requested together, see score_raw_o)
                 bf16x8 kt[D / 32];
