@@ -1256,7 +1256,10 @@ int sba_launch_mfma_bwd(const sba::KParams& kp_in, int phases, hipStream_t s) {
         // small grids last as long as their longest sweep: take the variant that halves it
         if (p1 && grid.x <= sba_two_step_max_grid()) hipLaunchKernelGGL((mfma_bwd_dq2_kernel<64>), grid, dim3(2 * kThreads), 0, s, kp);
         else if (p1) hipLaunchKernelGGL((mfma_bwd_dq_kernel<64>), grid, dim3(kThreads), 0, s, kp);
-        if (p2 && own) {
+        const char* e = getenv("SBA_DKV_KERNEL");
+        if (p2 && e && !strcmp(e, "plain")) {
+            hipLaunchKernelGGL((mfma_bwd_dkv_kernel<64>), dim3(2 * grid.x), dim3(kThreads), 0, s, kp);
+        } else if (p2 && own) {
             hipLaunchKernelGGL((mfma_bwd_dkv_own_kernel<64>), grid, dim3(kThreads), 0, s, kp);
         } else if (p2) {
             // one resident workgroup per CU, in whole rounds of the 8 XCDs (surplus workgroups
