@@ -23,13 +23,13 @@ KERNEL_TIMING_SAMPLES = 5      # steps of the timed region whose kernels are tim
 # runs summarised under profiles/ (sba_cfg{2,3,4}_hbm_traffic.txt, sba_cfg{2,3,4}_shader_counters.txt) and
 # are reported with that source next to what this run measures itself.
 # HBM bytes per launch (FETCH_SIZE + WRITE_SIZE, scaled by a copy kernel of known size):
-PROFILED_HBM_BYTES = {("cfg2", "fwd"): 54341416, ("cfg2", "bwd_dq"): 62276476, ("cfg2", "bwd_dkv"): 68003005,
-                      ("cfg3", "fwd"): 909894854, ("cfg3", "bwd_dq"): 980533123, ("cfg3", "bwd_dkv"): 1121534757,
-                      ("cfg4", "fwd"): 639594244, ("cfg4", "bwd_dq"): 1381842591, ("cfg4", "bwd_dkv"): 1402182615}
+PROFILED_HBM_BYTES = {("cfg2", "fwd"): 54520951, ("cfg2", "bwd_dq"): 62559004, ("cfg2", "bwd_dkv"): 68049117,
+                      ("cfg3", "fwd"): 877430953, ("cfg3", "bwd_dq"): 976620654, ("cfg3", "bwd_dkv"): 1120507593,
+                      ("cfg4", "fwd"): 638883430, ("cfg4", "bwd_dq"): 1562850522, ("cfg4", "bwd_dkv"): 1401645330}
 # wave instructions per launch: (vector incl. transcendental, transcendental, MFMA)
-PROFILED_INSTRUCTIONS = {("cfg2", "fwd"): (16467648, 2196480, 1064960), ("cfg2", "bwd_dq"): (30978048, 4259840, 1597440), ("cfg2", "bwd_dkv"): (37096628, 4292608, 2146304),
-                   ("cfg3", "fwd"): (125639104, 18584544, 9010688), ("cfg3", "bwd_dq"): (258147184, 36042752, 13516032), ("cfg3", "bwd_dkv"): (304725344, 35128320, 17564160),
-                   ("cfg4", "fwd"): (258899968, 34738176, 33685504), ("cfg4", "bwd_dq"): (530288640, 67371008, 50528256), ("cfg4", "bwd_dkv"): (631058432, 67371008, 67371008)}
+PROFILED_INSTRUCTIONS = {("cfg2", "fwd"): (16467648, 2196480, 1064960), ("cfg2", "bwd_dq"): (29192193, 4259840, 1597440), ("cfg2", "bwd_dkv"): (37204161, 4292608, 2146304),
+                   ("cfg3", "fwd"): (125639104, 18584544, 9010688), ("cfg3", "bwd_dq"): (242991217, 36042752, 13516032), ("cfg3", "bwd_dkv"): (289956704, 35128320, 17564160),
+                   ("cfg4", "fwd"): (258899968, 34738176, 33685504), ("cfg4", "bwd_dq"): (465956865, 67371008, 50528256), ("cfg4", "bwd_dkv"): (623136768, 67371008, 67371008)}
 # issue time of one SIMD per instruction, ns, four waves per SIMD (profiles/gfx950_issue_rates.txt): plain vector,
 # transcendental issued while MFMAs are in flight, MFMA 32x32x16 bf16.  MFMAs and plain vector instructions do not
 # overlap on gfx950, so their times add up.

@@ -1,4 +1,5 @@
 """Writes the golden vectors of this folder (``sb_*.npz``).  Run: python tests/golden/make_vectors.py
+(``python tests/golden/make_vectors.py overflow`` writes only ``sb_packed_overflow.npz``)
 
 The reference ships no fixtures for stick-breaking attention, so these come from the
 mathematics alone, evaluated with 50-digit arithmetic (mpmath) and sharing no code with the
@@ -154,7 +155,50 @@ def run_directional_case(name, rng, lens, D, scale, attend_current, in_scale, pa
     print(name, "written", flush=True)
 
 
+def run_overflow_case(name):
+    """A packed batch whose second document holds, inside the 32 keys that one lane of the
+    matrix-core kernels chains over, logits of +90 (the running product of 1 + e^z leaves the
+    fp32 range) followed further left by logits of -200 (e^z is exactly 0 in fp32) and by the keys
+    of the previous document and of the diagonal, which are masked: a chain kept as that product
+    meets inf * 0 there.  Own random stream, so that adding it does not move the other cases."""
+    rng = np.random.default_rng(20250117)
+    lens, D, H = [5, 40], 4, 1
+    total = sum(lens)
+    q, k, v, do = (rng.standard_normal((H, total, D)) * s for s in (0.5, 0.5, 1.0, 1.0))
+    q[0, 25:, :] = 0.0
+    q[0, 25:, 1] = 4.0                     # queries 20.. of the second document look along one coordinate
+    k[0, 17:21, :] = 0.0
+    k[0, 17:21, 1] = 45.0                  # logit +90 at scale 0.5
+    k[0, 9:13, :] = 0.0
+    k[0, 9:13, 1] = -100.0                 # logit -200
+    q, k, v, do, drem = (bf16_exact(x) for x in (q, k, v, do, rng.standard_normal((H, total))))
+    scale, attend_current = 0.5, False
+    res = {n: np.zeros((H, total, D)) for n in ("o", "dq", "dk", "dv")}
+    rem = np.zeros((H, total))
+    start = 0
+    for L in lens:
+        sl = slice(start, start + L)
+        args = [to_mp(x[0, sl]) for x in (q, k, v, do)] + [[mpf(float(x)) for x in drem[0, sl]]]
+        o_, rem_ = forward_one(args[0], args[1], args[2], mpf(scale), attend_current)
+        dq_, dk_, dv_ = grads_one(*args, mpf(scale), attend_current)
+        res["o"][0, sl] = np.array(o_, dtype=np.float64).reshape(L, D)
+        rem[0, sl] = np.array(rem_, dtype=np.float64)
+        for n, g in (("dq", dq_), ("dk", dk_), ("dv", dv_)):
+            res[n][0, sl] = np.array(g, dtype=np.float64).reshape(L, D)
+        start += L
+    arrays = dict(q=q, k=k, v=v, do=do, drem=drem, rem=rem, **res)
+    arrays["cu_seqlens"] = np.cumsum([0] + list(lens)).astype(np.int32)
+    arrays["scale"] = np.float64(scale)
+    arrays["attend_current"] = np.bool_(attend_current)
+    np.savez(os.path.join(HERE, name + ".npz"), **arrays)
+    print(name, "written", flush=True)
+
+
 if __name__ == "__main__":
+    import sys
+    if sys.argv[1:] == ["overflow"]:       # only the case added last
+        run_overflow_case("sb_packed_overflow")
+        sys.exit(0)
     rng = np.random.default_rng(20240607)
     run_case("sb_dense_strict", rng, H=2, lens=[9], D=4, scale=0.7, attend_current=False, in_scale=1.0, packed=False)
     run_case("sb_dense_current", rng, H=2, lens=[6], D=3, scale=3 ** -0.5, attend_current=True, in_scale=1.0, packed=False)
@@ -166,3 +210,4 @@ if __name__ == "__main__":
     run_directional_case("sbdir_dense_d64", rng, lens=[150], D=64, scale=0.125, attend_current=False, in_scale=1.0, packed=False)
     run_directional_case("sbdir_packed_d64", rng, lens=[40, 136], D=64, scale=0.125, attend_current=True, in_scale=1.0, packed=True)
     run_directional_case("sbdir_dense_d128", rng, lens=[130], D=128, scale=128 ** -0.5, attend_current=True, in_scale=1.0, packed=False)
+    run_overflow_case("sb_packed_overflow")

@@ -25,7 +25,7 @@ def _load(path):
 
 
 def test_all_fixtures_present():
-    assert len(GOLDEN) == 5
+    assert len(GOLDEN) == 6
 
 
 @pytest.mark.parametrize("path", GOLDEN, ids=os.path.basename)
