@@ -23,10 +23,11 @@ bool force_generic() {
     return e && e[0] == '1';
 }
 
-// The MFMA kernels cover bf16 with head_dim 64 or 128; everything else takes the
-// generic vector-ALU kernels.
+// The matrix-core kernels cover bf16 with head_dim 64 or 128 and fp32 with head_dim 64;
+// everything else takes the generic vector-ALU kernels.
 bool use_mfma(const SbaParams* p) {
     if (force_generic()) return false;
+    if (p->dtype == SBA_DTYPE_F32) return p->head_dim == 64;
     return p->dtype == SBA_DTYPE_BF16 && (p->head_dim == 64 || p->head_dim == 128);
 }
 
@@ -81,9 +82,10 @@ int check_common(const SbaParams* p) {
     }
     if (use_mfma(p)) {
         // the matrix-core kernels move 16-byte chunks: aligned rows, outer strides in whole chunks
+        const int64_t per16 = p->dtype == SBA_DTYPE_F32 ? 3 : 7;
         for (const SbaTensor* t : {&p->q, &p->k, &p->v, &p->o, &p->d_o, &p->dq, &p->dk, &p->dv}) {
             if (!t->ptr) continue;          // presence is checked per direction
-            if (((uintptr_t)t->ptr & 15) || (t->stride_b & 7) || (t->stride_h & 7) || (t->stride_t & 7)) return SBA_ERR_SHAPE;
+            if (((uintptr_t)t->ptr & 15) || (t->stride_b & per16) || (t->stride_h & per16) || (t->stride_t & per16)) return SBA_ERR_SHAPE;
         }
     }
     return SBA_OK;
@@ -150,7 +152,7 @@ const char* sba_error_string(int code) {
     switch (code) {
         case SBA_OK: return "ok";
         case SBA_ERR_NULL: return "a required pointer is NULL";
-        case SBA_ERR_SHAPE: return "bad shape: sizes must be positive, head_dim <= 128, dense total_tokens == seq_len; bf16 at head_dim 64 / 128 needs 16-byte aligned pointers and strides that are multiples of 8 elements";
+        case SBA_ERR_SHAPE: return "bad shape: sizes must be positive, head_dim <= 128, dense total_tokens == seq_len; bf16 at head_dim 64 / 128 and fp32 at head_dim 64 need 16-byte aligned pointers and strides that are multiples of 16 bytes";
         case SBA_ERR_DTYPE: return "unsupported dtype (float32 and bfloat16 only)";
         case SBA_ERR_WORKSPACE: return "workspace / bwd_scratch missing or smaller than sba_workspace_bytes() / sba_bwd_scratch_bytes()";
         case SBA_ERR_SCHEDULE: return "packed layout needs a row-block schedule from sba_build_schedule()";
@@ -239,6 +241,7 @@ int sba_fwd(const SbaParams* p) {
     }
     KParams kp = make_kparams(p);
     hipStream_t s = (hipStream_t)p->stream;
+    if (mfma && p->dtype == SBA_DTYPE_F32) return sba_launch_mfma_f32_fwd(kp, s);
     return mfma ? sba_launch_mfma_fwd(kp, s) : sba_launch_generic_fwd(kp, p->dtype, s);
 }
 
@@ -256,11 +259,12 @@ int sba_bwd(const SbaParams* p) {
         KParams carry = kp;
         carry.save = 1;
         carry.carry_only = 1;
-        rc = sba_launch_mfma_fwd(carry, s);
+        rc = p->dtype == SBA_DTYPE_F32 ? sba_launch_mfma_f32_fwd(carry, s) : sba_launch_mfma_fwd(carry, s);
         if (rc) return rc;
     }
     // the generic backward is one piece: it all runs in phase 1
     if (!use_mfma_bwd(p) && p->bwd_phases == 2) return SBA_OK;
+    if (use_mfma_bwd(p) && p->dtype == SBA_DTYPE_F32) return sba_launch_mfma_f32_bwd(kp, p->bwd_phases, s);
     return use_mfma_bwd(p) ? sba_launch_mfma_bwd(kp, p->bwd_phases, s) : sba_launch_generic_bwd(kp, p->dtype, s);
 }
 

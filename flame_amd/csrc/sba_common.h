@@ -149,4 +149,6 @@ int sba_launch_generic_fwd(const sba::KParams& kp, int dtype, hipStream_t s);
 int sba_launch_generic_bwd(const sba::KParams& kp, int dtype, hipStream_t s);
 int sba_launch_mfma_fwd(const sba::KParams& kp, hipStream_t s);
 int sba_launch_mfma_bwd(const sba::KParams& kp, int phases, hipStream_t s);
+int sba_launch_mfma_f32_fwd(const sba::KParams& kp, hipStream_t s);
+int sba_launch_mfma_f32_bwd(const sba::KParams& kp, int phases, hipStream_t s);
 bool sba_mfma_bwd_available();

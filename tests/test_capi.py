@@ -95,9 +95,11 @@ def test_workspace_bytes(lib):
     p.workspace = 1
     assert lib.sba_bwd_scratch_bytes(C.byref(p)) == 3 * table + 256    # what the backward needs for itself
     p.workspace = None
-    p.dtype = _lib.SBA_DTYPE_F32                    # generic kernels: nothing kept, fp32 dk|dv accumulators
+    p.dtype = _lib.SBA_DTYPE_F32                    # fp32 at head_dim 64 runs on the matrix cores too: same tables
+    assert lib.sba_workspace_bytes(C.byref(p)) == table
+    p.head_dim = 128                                # generic kernels: nothing kept, fp32 dk|dv accumulators
     assert lib.sba_workspace_bytes(C.byref(p)) == 0
-    assert lib.sba_bwd_scratch_bytes(C.byref(p)) == 2 * 4096 * 16 * 64 * 4
+    assert lib.sba_bwd_scratch_bytes(C.byref(p)) == 2 * 4096 * 16 * 128 * 4
 
 
 def test_static_backward_refuses_oversize_without_gpu(lib):

@@ -603,3 +603,42 @@ def test_recomputing_the_carries_in_the_backward_gives_the_same_bits(D, monkeypa
     for a, b in zip(kept, again):
         for x, y in zip(a, b):
             assert torch.equal(x, y)
+
+
+def test_fp32_runs_on_the_matrix_cores_bit_reproducibly_and_agrees_with_the_generic_kernels(monkeypatch):
+    # fp32 at head_dim <= 64 takes the fp32 MFMA kernels (no atomics): two runs give identical bits,
+    # dense and packed; the generic vector-ALU kernels (a separate implementation) agree to fp32 accuracy
+    sb_attn, sb_attn_varlen = _ops()
+    q, k, v, do = (randn((2, 3, 333, 64), 500 + i, 1.0 if i < 3 else 1.0).cuda() for i in range(4))
+    drem = randn((2, 3, 333), 505).cuda()
+    lens = [70, 1, 200, 129, 266]
+    cu = cu_from_lengths(lens).cuda()
+    qp, kp, vp, dop = (x.reshape(6, 333, 64)[:, :, :].reshape(3, 666, 64).contiguous() for x in (q, k, v, do))
+
+    def dense():
+        qq, kk, vv = (x.clone().requires_grad_(True) for x in (q, k, v))
+        o, rem = sb_attn(qq, kk, vv)
+        torch.autograd.backward([o, rem], [do, drem])
+        return o, rem, qq.grad, kk.grad, vv.grad
+
+    def packed():
+        qq, kk, vv = (x.clone().requires_grad_(True) for x in (qp, kp, vp))
+        o, rem = sb_attn_varlen(qq, kk, vv, cu, max(lens))
+        torch.autograd.backward([o], [dop])
+        return o, rem, qq.grad, kk.grad, vv.grad
+
+    for fn in (dense, packed):
+        a, b = fn(), fn()
+        assert all(torch.equal(x, y) for x, y in zip(a, b))
+        monkeypatch.setenv("SBA_FORCE_GENERIC", "1")
+        c = fn()
+        monkeypatch.delenv("SBA_FORCE_GENERIC")
+        assert max_abs(a[0], c[0]) <= 1e-4 and max_abs(a[1], c[1]) <= 1e-4
+        for x, y in zip(a[2:], c[2:]):
+            assert rel_l2(x, y) <= 2e-3
+
+
+def test_fp32_config1_in_memory_lean_mode(monkeypatch):
+    # benchmark configuration 1 once more with the backward recomputing the carry table (fp32 MFMA kernels)
+    monkeypatch.setenv("SBA_RECOMPUTE_CARRIES", "1")
+    _check_dense(2, 4, 512, 64, torch.float32, seed=0)
