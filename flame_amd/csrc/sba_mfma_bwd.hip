@@ -20,6 +20,7 @@
 // Every element of the score matrix is therefore evaluated twice in the backward (once per
 // pass); in exchange nothing is reduced through memory.
 #include <string.h>
+#include <type_traits>
 #include "sba_mfma.h"
 
 namespace sba {
@@ -555,6 +556,31 @@ __device__ inline void wait_for_count(int* counter, int target, int* gave_up) {
     if (gave_up && (threadIdx.x & 63) == 0) *gave_up = 1;
 }
 
+// Weights and logit gradients of ONE [32 keys x 32 queries] tile whose lanes hold 16 consecutive keys
+// (the own-keys kernel and the eight-producer stream): the carries enter per 32 keys.
+template <class Between>
+__device__ inline void own_tile_weights(float (&x)[16], float (&beta)[16], float Rin, int lane, Between&& between) {
+    const float L = product_chain_with<true, 16>(x, beta, between);
+    float Llo, Lup;
+    half_values(L, Llo, Lup);
+    scale_clamped<16>(x, (lane >= 32) ? Rin : Rin * Lup);         // upper half-wave: the right 16 keys
+}
+__device__ inline void own_tile_grads(const float (&a)[16], const float (&beta)[16], float (&dp)[16], float Gin,
+                                      int lane) {
+    float c = 0.f, pre[16];
+#pragma unroll
+    for (int idx = 0; idx < 16; ++idx) {
+        dp[idx] = a[idx] * dp[idx];     // g
+        c += dp[idx];
+        pre[idx] = c;
+    }
+    float clo, cup;
+    half_values(c, clo, cup);
+    const float F = (lane >= 32) ? Gin + clo : Gin;
+#pragma unroll
+    for (int idx = 0; idx < 16; ++idx) dp[idx] = __builtin_fmaf(-beta[idx], pre[idx] + F, dp[idx]);
+}
+
 struct KeyItem {
     Job job;
     int head, kb, key0, n_steps;
@@ -574,13 +600,18 @@ __device__ inline KeyItem decode_item(const KParams& p, int idx) {
     return r;
 }
 
-template <int D>
-__global__ __launch_bounds__(2 * kThreads, 2) void mfma_bwd_dkv_stream_kernel(KParams p) {
+// NP = number of producer waves.  4: producer w does queries 32w.. of the step against all 64 keys
+// (one wave per SIMD computes weights).  8: producer w does queries 32(w%4).. against the 32 keys
+// 32(w/4).. of the block - two producers per SIMD, which is what lets a SIMD issue their vector
+// instructions back to back (one wave alone issues one every 2.2-2.7 ns, two together one every
+// 1.1-1.2 ns); the half blocks take the mid-block carries of the dQ pass, like the own-keys kernel.
+template <int D, int NP>
+__global__ __launch_bounds__((NP + 4) * 64, NP == 4 ? 2 : 3) void mfma_bwd_dkv_stream_kernel(KParams p) {
     constexpr int kTile = 64 * D * 2;          // K or V tile (64 keys)
     constexpr int kQTile = 128 * D * 2;        // Q or dO tile (128 queries)
     constexpr int kZTile = 128 * 64 * 2;       // weights of one step, [query][key] bf16
     constexpr int kBuf = 2 * kZTile + 2 * kQTile;
-    constexpr int kCarry = kRowBlock * 8;      // {R, G} per query
+    constexpr int kCarry = kRowBlock * (NP == 4 ? 8 : 16);   // {R, G} per query; NP = 8: {R, G, R mid-block, G mid-block}
     __shared__ __attribute__((aligned(1024))) char lds[3 * kTile + 2 * kCarry + 2 * kBuf];
     __shared__ int consumers_done;             // consumer waves that have finished a reduction, running total
     __shared__ int producers_took_k;           // producer waves that hold an item's K fragments, running total
@@ -591,7 +622,7 @@ __global__ __launch_bounds__(2 * kThreads, 2) void mfma_bwd_dkv_stream_kernel(KP
 
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const bool producer = wave < 4;
+    const bool producer = wave < NP;
     const int w4 = wave & 3;
     const int n = lane & 31, h = lane >> 5;
     const int strict = p.attend_current ? 0 : 1;
@@ -621,6 +652,90 @@ __global__ __launch_bounds__(2 * kThreads, 2) void mfma_bwd_dkv_stream_kernel(KP
         __syncthreads();                       // first item's tiles and carries visible
         int s = 0;
         bool staged_prev = false;              // the consumers staged a dK/dV in the previous iteration
+        if constexpr (NP == 8) {
+        const int kh = wave >> 2;              // this wave's half of the 64-key block
+        for (int item = 0;; ++item) {
+            const char* vtile = vtiles + (item & 1) * kTile;
+            // rows 32kh.. of the K and V tiles are this wave's keys, in the order that puts 16
+            // consecutive keys into a lane's accumulator registers (see request_keys)
+            bf16x8 kfr[D / 16], vfr[D / 16];
+#pragma unroll
+            for (int ks = 0; ks < D / 16; ++ks) {
+                kfr[ks] = fetch_rows_o<D>(ktile, lo, kh, ks);
+                vfr[ks] = fetch_rows_o<D>(vtile, lo, kh, ks);
+            }
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+            if (lane == 0) __hip_atomic_fetch_add(&producers_took_k, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+            const int key0 = cur.key0 + 32 * kh;
+            const int len = cur.job.len;
+            for (int it = 0; it < cur.n_steps; ++it, ++s) {
+                const bool x_now = staged_prev;
+                staged_prev = it == 0 && item > 0;
+                char* zp = bufs + (s & 1) * kBuf;
+                char* zd = zp + kZTile;
+                const char* qtile = zd + kZTile;
+                const char* dotile = qtile + kQTile;
+                const int q0w = (cur.job.rb + it) * kRowBlock + 32 * w4;
+                const int qi = q0w + n;
+#ifdef SBA_EXP_IDLE_PRODUCERS
+                const bool skip = true;
+#else
+                const bool skip = key0 + strict > q0w + 31 || q0w >= len || key0 >= len;
+#endif
+                float x[16], beta[16], dp[16];
+                float Gt = 0.f;
+                if (!skip) {
+                    const float4 cv = *(const float4*)(carry + (s & 1) * kCarry + (32 * w4 + n) * 16);
+                    // table entries of pairs that no query of the row sees are not written
+                    const bool sees = qi < len && qi - strict - key0 + 1 > 0;
+                    const float Rt = sees ? (kh ? cv.x : cv.z) : 1.0f;
+                    Gt = sees ? (kh ? cv.w : cv.y) : 0.0f;
+                    bf16x8 qf[D / 16], dof[D / 16];
+#pragma unroll
+                    for (int ks = 0; ks < D / 16; ++ks) {
+                        qf[ks] = fetch_rows_o<D>(qtile, lo, w4, ks);
+                        dof[ks] = fetch_rows_o<D>(dotile, lo, w4, ks);
+                    }
+                    f32x16 acc = {0};
+#pragma unroll
+                    for (int ks = 0; ks < D / 16; ++ks) acc = mfma(kfr[ks], qf[ks], acc);
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) x[r] = acc[r] * p.scale2;
+                    if (key0 + 31 + strict > q0w || q0w + 31 >= len) {        // diagonal or ragged tile
+                        const int nvis = qi < len ? qi - strict - (key0 + 16 * h) + 1 : 0;
+#pragma unroll
+                        for (int idx = 0; idx < 16; ++idx)
+                            if (idx >= nvis) x[idx] = -INFINITY;
+                    }
+                    // dP = dO V^T: one MFMA behind each of the chain's four segments
+                    static_assert(D == 64, "one dP MFMA per chain segment");
+                    f32x16 dacc;
+                    own_tile_weights(x, beta, Rt, lane, [&](int seg) {
+                        dacc = mfma(vfr[seg], dof[seg], seg == 0 ? f32x16{0} : dacc);
+                    });
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) dp[r] = dacc[r];
+                }
+                if (x_now) __syncthreads();    // X
+                if (!skip) {
+                    own_tile_grads(x, beta, dp, Gt, lane);
+                } else {
+#pragma unroll
+                    for (int idx = 0; idx < 16; ++idx) { x[idx] = 0.f; dp[idx] = 0.f; }
+                }
+#pragma unroll
+                for (int c = 0; c < 2; ++c) {
+                    *(bf16x8*)(zp + tile_offset<64>(32 * w4 + n, 4 * kh + 2 * h + c)) = pack8(&x[8 * c]);
+                    *(bf16x8*)(zd + tile_offset<64>(32 * w4 + n, 4 * kh + 2 * h + c)) = pack8(&dp[8 * c]);
+                }
+                __syncthreads();               // A
+            }
+            if (!nxt.valid) break;
+            cur = nxt;
+            nxt = decode_item(p, static_item(ring));
+            ++ring;
+        }
+        } else {
         for (int item = 0;; ++item) {
             const char* vtile = vtiles + (item & 1) * kTile;
             // the key block of an item never changes: its score and dP operands stay in registers
@@ -709,6 +824,7 @@ __global__ __launch_bounds__(2 * kThreads, 2) void mfma_bwd_dkv_stream_kernel(KP
             nxt = decode_item(p, static_item(ring));
             ++ring;
         }
+        }
         __syncthreads();                       // A of the draining iteration
     } else {
         LaneOffsets<D> lo;
@@ -738,7 +854,7 @@ __global__ __launch_bounds__(2 * kThreads, 2) void mfma_bwd_dkv_stream_kernel(KP
         // iteration consumes what it requested: no register is "perhaps still being loaded" on
         // some path, so the compiler's wait-count bookkeeping stays exact.
         u32x4 tx[8];
-        float cR, cG;
+        float cR, cG, cRm = 1.f, cGm = 0.f;
         // Four lanes fill the 64 bytes of a row that this wave reduces; an LDS write cycle takes eight
         // lanes, i.e. two rows, whose swizzles must differ in the bit that selects the other half of the
         // row's banks: rows r and r + 2 do (r and r + 1 would collide), hence the order 0 2 1 3 ...
@@ -753,6 +869,7 @@ __global__ __launch_bounds__(2 * kThreads, 2) void mfma_bwd_dkv_stream_kernel(KP
         struct ItemPtrs {
             const char* x;                     // Q or dO: row 0 of the sequence, this head, this thread's chunk
             const float *rt, *gt;              // carries of this (head, key block): row block 0, query 0
+            const float *rm, *gm;              // NP = 8: the mid-block carries
             int row0, len;                     // first query of the item's sweep; sequence length
         };
         auto item_ptrs = [&](const KeyItem& t) {
@@ -762,25 +879,28 @@ __global__ __launch_bounds__(2 * kThreads, 2) void mfma_bwd_dkv_stream_kernel(KP
             const int64_t tk = tab_index(p, t.head, t.job, 0, t.kb);
             r.rt = p.rtab + tk;
             r.gt = p.gtab + tk;
+            r.rm = p.rmid + tk;
+            r.gm = p.gmid + tk;
             r.row0 = t.job.rb * kRowBlock;
             r.len = t.job.len;
             asm volatile("" : "+v"(r.x), "+v"(r.rt), "+v"(r.gt));
+            if (NP == 8) asm volatile("" : "+v"(r.rm), "+v"(r.gm));
             return r;
         };
         const uint32_t x_st2 = 2u * (uint32_t)(is_dv ? p.d_o.st : p.q.st);
-        auto request_tile = [&](const ItemPtrs& t, int row0, int part) {       // part 0..3: two loads each
-#pragma unroll
-            for (int i = 2 * part; i < 2 * part + 2; ++i) {
-                const uint32_t row = (uint32_t)min(row0 + crow + 16 * i, t.len - 1);
-                tx[i] = *(const u32x4*)(t.x + (size_t)row * x_st2);
-            }
-        };
-        auto request_carry = [&](const ItemPtrs& t, int row0) {
+        auto request_step = [&](const ItemPtrs& t, int row0) {
             const int qi = min(row0 + (ct & (kRowBlock - 1)), t.len - 1);
             const int qb = qi >> 7;            // row block of the query: its slab starts qb*(qb+1) columns in
             const int64_t ix = (int64_t)qb * (qb + 1) * kRowBlock + (qi & (kRowBlock - 1));
             cR = t.rt[ix]; cG = t.gt[ix];
+            if (NP == 8) { cRm = t.rm[ix]; cGm = t.gm[ix]; }
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                const uint32_t row = (uint32_t)min(row0 + crow + 16 * i, t.len - 1);
+                tx[i] = *(const u32x4*)(t.x + (size_t)row * x_st2);
+            }
         };
+        constexpr int kLoadsPerStep = 8 + (NP == 8 ? 4 : 2);      // per lane: what request_step issues
         // K and V tiles of an item go straight from global memory into LDS (no registers, and
         // nothing for the wait-count bookkeeping to track): every instruction moves 64 x 16 bytes
         // into 1 KB of consecutive LDS, the lane picks the global chunk that belongs at its LDS
@@ -795,7 +915,10 @@ __global__ __launch_bounds__(2 * kThreads, 2) void mfma_bwd_dkv_stream_kernel(KP
                 const int pos = inst * 64 + lane;          // LDS chunk position
                 const int r = pos / (D / 8), pc = pos % (D / 8);
                 const int c = pc ^ swz<D>(r);
-                const int kl = (((r >> 2) & 1) << 5) | (((r >> 5) & 1) << 4) | (((r >> 3) & 3) << 2) | (r & 3);
+                // NP = 4: the accumulator registers of a producer lane are 32 consecutive keys over its two
+                // tiles; NP = 8: 16 consecutive keys of the one tile (rows 32kh..) of producer half kh
+                const int kl = NP == 4 ? (((r >> 2) & 1) << 5) | (((r >> 5) & 1) << 4) | (((r >> 3) & 3) << 2) | (r & 3)
+                                       : (((r >> 5) & 1) << 5) | (((r >> 2) & 1) << 4) | (((r >> 3) & 3) << 2) | (r & 3);
                 const int row = min(t.key0 + kl, t.job.len - 1);
                 __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(p.k.ptr + 2 * (kbase + (int64_t)row * p.k.st + c * 8)),
                                                  (__attribute__((address_space(3))) void*)(uintptr_t)(uint32_t)(uintptr_t)(ktile + inst * 1024),
@@ -809,8 +932,10 @@ __global__ __launch_bounds__(2 * kThreads, 2) void mfma_bwd_dkv_stream_kernel(KP
             char* xtile = bufs + (s & 1) * kBuf + 2 * kZTile + (is_dv ? kQTile : 0);
 #pragma unroll
             for (int i = 0; i < 8; ++i) *(u32x4*)(xtile + tile_offset<D>(crow + 16 * i, cch)) = tx[i];
-            if (ct < kRowBlock)
-                *(float2*)(carry + (s & 1) * kCarry + ct * 8) = float2{cR, cG};
+            if (ct < kRowBlock) {
+                if (NP == 8) *(float4*)(carry + (s & 1) * kCarry + ct * 16) = float4{cR, cG, cRm, cGm};
+                else *(float2*)(carry + (s & 1) * kCarry + ct * 8) = float2{cR, cG};
+            }
         };
         auto store_staged = [&](int idx, const char* staging) {
             const KeyItem t = decode_item(p, idx);
@@ -833,31 +958,58 @@ __global__ __launch_bounds__(2 * kThreads, 2) void mfma_bwd_dkv_stream_kernel(KP
         auto reduce = [&](int s_done) {
             const char* zt = bufs + (s_done & 1) * kBuf + (is_dv ? 0 : kZTile);            // a or dz
             const char* xt = bufs + (s_done & 1) * kBuf + 2 * kZTile + (is_dv ? kQTile : 0); // dO or Q
+            constexpr int kBatch = NP == 8 ? 2 : 4;        // NP = 8: three waves per SIMD, fewer registers
 #pragma unroll
-            for (int b = 0; b < 2; ++b) {
-                bf16x8 aw[4][2], bx[4];
+            for (int b = 0; b < 8 / kBatch; ++b) {
+                bf16x8 aw[kBatch][2], bx[kBatch];
 #pragma unroll
-                for (int j = 0; j < 4; ++j) {
-                    const int c2 = 4 * b + j;
+                for (int j = 0; j < kBatch; ++j) {
+                    const int c2 = kBatch * b + j;
                     aw[j][0] = fetch_nat_2<64>(zt, za[0][0], za[0][1], 16 * c2);
                     aw[j][1] = fetch_nat_2<64>(zt, za[1][0], za[1][1], 16 * c2);
                     bx[j] = fetch_nat_2<D>(xt, qb0o, qb1o, 16 * c2);
                 }
 #pragma unroll
-                for (int j = 0; j < 4; ++j) {
+                for (int j = 0; j < kBatch; ++j) {
                     acc[0] = mfma(aw[j][0], bx[j], acc[0]);
                     acc[1] = mfma(aw[j][1], bx[j], acc[1]);
                 }
+                if (NP == 8) __builtin_amdgcn_sched_barrier(0);
             }
         };
 
-        ItemPtrs cp = item_ptrs(cur), np = item_ptrs(nxt);
+        // A step's tiles and carries are requested right after the previous step's have been
+        // deposited, almost a whole iteration before their own deposit (an iteration is shorter than
+        // a round trip to memory plus the reduction: requested at the start of the iteration that
+        // deposits them, as an earlier version did, they were waited for).  `front` is the position of
+        // the next request in the stream of (item, step) pairs; past the end of the stream it stays on
+        // the last step (a harmless repeat).
+        struct Front {
+            ItemPtrs ptrs;
+            int it, n_steps, ring;
+            bool done;
+        } front;
+        front.ptrs = item_ptrs(cur);
+        front.it = 0; front.n_steps = cur.n_steps; front.ring = 1; front.done = false;
+        auto request_front = [&]() {
+            request_step(front.ptrs, front.ptrs.row0 + front.it * kRowBlock);
+            if (front.done) return;
+            if (front.it + 1 < front.n_steps) { ++front.it; return; }
+            const int idx = static_item(front.ring);
+            if (idx < 0) { front.done = true; return; }
+            const KeyItem t = decode_item(p, idx);
+            front.ptrs = item_ptrs(t);
+            front.it = 0; front.n_steps = t.n_steps; ++front.ring;
+        };
+        // Memory operations complete in order: with one step's requests in flight, everything issued
+        // before them (a deposited step, K / V tiles, stores) has landed.
+        static_assert(kLoadsPerStep < 16, "wait-count immediate");
+        auto wait_all_but_requests = [&]() { __builtin_amdgcn_s_waitcnt(0x0F70 | kLoadsPerStep); };
         request_keys(cur, vtiles);
-#pragma unroll
-        for (int part = 0; part < 4; ++part) request_tile(cp, cp.row0, part);
-        request_carry(cp, cp.row0);
+        request_front();
         deposit(0);
-        wait_global_memory();
+        request_front();
+        wait_all_but_requests();
         __syncthreads();                       // first item's tiles and carries visible
 
         int s = 0;
@@ -875,63 +1027,56 @@ __global__ __launch_bounds__(2 * kThreads, 2) void mfma_bwd_dkv_stream_kernel(KP
             wait_for_count(&consumers_done, sync_target, p.gave_up);
             __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
         };
-        // One iteration of the stream; `rq`, `rq_row0` say what the stream's next step needs.
-        auto iteration = [&](const ItemPtrs& rq, int rq_row0, bool last, bool keys_now, int item) {
+        // One iteration of the stream: the producers work on step s meanwhile.
+        auto iteration = [&](bool last, bool keys_now, int item) {
             if (store_pending) {               // staged in the previous iteration
                 store_staged(fin_store, bufs + (s & 1) * kBuf);
                 store_pending = false;
                 __syncthreads();               // X: the producers may overwrite the staging
             }
-            // The next step's carries and tiles are requested in one go ahead of the reduction: the
-            // answers are only needed at this iteration's deposit, a whole reduction away.  (Spread
-            // between the reduction's MFMAs, as an earlier version had them, the last requests were
-            // still in flight when the deposit came: 4 % of the kernel.)
-            request_carry(rq, rq_row0);
-#pragma unroll
-            for (int part = 0; part < 4; ++part) request_tile(rq, rq_row0, part);
-            if (s > 0) reduce(s - 1);
-            // B, only where a finished dK/dV is staged into the Z buffer just reduced: every
-            // consumer must be through with it
-            if (finish_after_reduce) consumer_sync();
             if (keys_now) {
-                // the K tile is free once every producer holds this item's fragments
-                wait_for_count(&producers_took_k, 4 * (item + 1), p.gave_up);
+                // the K tile is free once every producer holds this item's fragments; V goes to the
+                // tile of the other parity
+                wait_for_count(&producers_took_k, NP * (item + 1), p.gave_up);
                 __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
                 request_keys(decode_item(p, nxt_idx), vtiles + ((item + 1) & 1) * kTile);
             }
+#ifndef SBA_EXP_IDLE_REDUCE
+            if (s > 0) reduce(s - 1);
+#endif
+            // B, only where a finished dK/dV is staged into the Z buffer just reduced: every
+            // consumer must be through with it
             if (finish_after_reduce) {
+                consumer_sync();
                 stage(bufs + ((s - 1) & 1) * kBuf);
                 fin_store = fin_stage;
                 store_pending = true;
             }
-            deposit(s + 1);
+#ifndef SBA_EXP_NO_REQUEST
+            deposit(s + 1);                    // requested at the end of the previous iteration
+#endif
             finish_after_reduce = last;
             if (last) fin_stage = cur_idx;
-            wait_global_memory();              // nothing in flight across the back edge
+            __builtin_amdgcn_sched_barrier(0);
+#ifndef SBA_EXP_NO_REQUEST
+            request_front();                   // step s + 2
+#endif
+            wait_all_but_requests();
             __syncthreads();                   // A
             ++s;
         };
         for (int item = 0;; ++item) {
-            // The next item's K and V are requested after B of the second-to-last step: K's tile
-            // is free once the producers have taken their fragments (before the item's first B),
-            // V goes to the tile of the other parity.
+            // The next item's K and V are requested in the second-to-last step
             const int n_steps = cur.n_steps;
             const bool has_next = nxt.valid;
             const int keys_at = n_steps >= 2 ? n_steps - 2 : 0;
-            for (int it = 0; it + 1 < n_steps; ++it)
-                iteration(cp, cp.row0 + (it + 1) * kRowBlock, false, has_next && it == keys_at, item);
-            // the item's last step: the request is the next item's first step, or at the very end
-            // of the stream a harmless repeat
-            if (has_next) iteration(np, np.row0, true, n_steps - 1 == keys_at, item);
-            else iteration(cp, cp.row0, true, false, item);
+            for (int it = 0; it < n_steps; ++it) iteration(it + 1 == n_steps, has_next && it == keys_at, item);
             if (!has_next) break;
             cur_idx = nxt_idx;
             cur = nxt;
             nxt_idx = static_item(ring);
             nxt = decode_item(p, nxt_idx);
             ++ring;
-            cp = np;
-            np = item_ptrs(nxt);
         }
         // draining iteration: the last step of the last item
         if (store_pending) store_staged(fin_store, bufs + (s & 1) * kBuf);
@@ -954,29 +1099,6 @@ __global__ __launch_bounds__(2 * kThreads, 2) void mfma_bwd_dkv_stream_kernel(KP
 // a 64-key block that touches the edge, the mid-block ones for the other half.  Weights and
 // logit gradients go as bf16 [query][32 a | 32 dz] rows into a tile private to the wave and
 // come back transposed as the A operands of  dV += A^T dO  and  dK += dZ^T Q.
-template <class Between>
-__device__ inline void own_tile_weights(float (&x)[16], float (&beta)[16], float Rin, int lane, Between&& between) {
-    const float L = product_chain_with<true, 16>(x, beta, between);
-    float Llo, Lup;
-    half_values(L, Llo, Lup);
-    scale_clamped<16>(x, (lane >= 32) ? Rin : Rin * Lup);         // upper half-wave: the right 16 keys
-}
-__device__ inline void own_tile_grads(const float (&a)[16], const float (&beta)[16], float (&dp)[16], float Gin,
-                                      int lane) {
-    float c = 0.f, pre[16];
-#pragma unroll
-    for (int idx = 0; idx < 16; ++idx) {
-        dp[idx] = a[idx] * dp[idx];     // g
-        c += dp[idx];
-        pre[idx] = c;
-    }
-    float clo, cup;
-    half_values(c, clo, cup);
-    const float F = (lane >= 32) ? Gin + clo : Gin;
-#pragma unroll
-    for (int idx = 0; idx < 16; ++idx) dp[idx] = __builtin_fmaf(-beta[idx], pre[idx] + F, dp[idx]);
-}
-
 template <int D>
 __global__ __launch_bounds__(kThreads, D == 64 ? 2 : 1) void mfma_bwd_dkv_own_kernel(KParams p) {
     constexpr int kQTile = 64 * D * 2;           // Q or dO tile of one step (64 queries)
@@ -1251,13 +1373,19 @@ int sba_launch_mfma_bwd(const sba::KParams& kp_in, int phases, hipStream_t s) {
     // 64-key blocks, which has twice as many workgroups.
     const unsigned cus = (unsigned)sba_cu_count();
     const bool own = own_keys_kernel(kp.head_dim == 64 ? grid.x >= 3u * cus : grid.x > cus);
-    if (!own) kp.rmid = kp.gmid = nullptr;     // only the own-keys kernel reads the mid-block carries: dQ skips them
+    const char* which = getenv("SBA_DKV_KERNEL");
+    const bool plain = which && !strcmp(which, "plain");
+    // the stream with eight half-block producers (12 waves): measured within 1 % of the one with four
+    // full-block producers (109.1 against 110.3 us at B=1 H=16 T=4096), which stays the default
+    const bool stream8 = which && !strcmp(which, "stream8");
+    // the mid-block carries are read by the own-keys kernel and by the stream's half-block producers:
+    // otherwise the dQ pass skips them
+    if (!own && !(kp.head_dim == 64 && stream8 && !plain)) kp.rmid = kp.gmid = nullptr;
     if (kp.head_dim == 64) {
         // small grids last as long as their longest sweep: take the variant that halves it
         if (p1 && grid.x <= sba_two_step_max_grid()) hipLaunchKernelGGL((mfma_bwd_dq2_kernel<64>), grid, dim3(2 * kThreads), 0, s, kp);
         else if (p1) hipLaunchKernelGGL((mfma_bwd_dq_kernel<64>), grid, dim3(kThreads), 0, s, kp);
-        const char* e = getenv("SBA_DKV_KERNEL");
-        if (p2 && e && !strcmp(e, "plain")) {
+        if (p2 && plain) {
             hipLaunchKernelGGL((mfma_bwd_dkv_kernel<64>), dim3(2 * grid.x), dim3(kThreads), 0, s, kp);
         } else if (p2 && own) {
             hipLaunchKernelGGL((mfma_bwd_dkv_own_kernel<64>), grid, dim3(kThreads), 0, s, kp);
@@ -1267,7 +1395,8 @@ int sba_launch_mfma_bwd(const sba::KParams& kp_in, int phases, hipStream_t s) {
             const unsigned n_items = 2 * grid.x;
             unsigned n_wg = n_items < cus ? n_items : cus;
             n_wg = (n_wg + 7) & ~7u;
-            hipLaunchKernelGGL((mfma_bwd_dkv_stream_kernel<64>), dim3(n_wg), dim3(2 * kThreads), 0, s, kp);
+            if (stream8) hipLaunchKernelGGL((mfma_bwd_dkv_stream_kernel<64, 8>), dim3(n_wg), dim3(12 * 64), 0, s, kp);
+            else hipLaunchKernelGGL((mfma_bwd_dkv_stream_kernel<64, 4>), dim3(n_wg), dim3(8 * 64), 0, s, kp);
         }
     } else {
         if (p1) hipLaunchKernelGGL((mfma_bwd_dq_kernel<128>), grid, dim3(kThreads), 0, s, kp);

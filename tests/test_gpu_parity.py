@@ -498,12 +498,14 @@ def test_config4_size_invariants():
     _full_size_properties(fwd_bwd, ups)
 
 
-@pytest.mark.parametrize("dkv_kernel,D", [("", 64), ("own", 64), ("other", 64), ("own", 128), ("other", 128)])
+@pytest.mark.parametrize("dkv_kernel,D", [("", 64), ("own", 64), ("other", 64), ("stream8", 64), ("plain", 64),
+                                          ("own", 128), ("other", 128)])
 def test_randomized_packed_batches_mfma_vs_generic_backward(dkv_kernel, D, monkeypatch):
     # Seeded random packed batches (document counts, lengths around the 64/128 block edges,
     # head counts that are and are not multiples of 8, both masks): the MFMA kernels against the
     # generic vector-ALU kernels, an independent implementation, forward and all three gradients.
-    # Either key-owner kernel is forced in turn (the library picks between them by grid size).
+    # Every key-owner kernel is forced in turn (the library picks between them by grid size; the
+    # stream with eight half-block producers and the plain 64-key-block kernel are selectable only).
     _, sb_attn_varlen = _ops()
     if dkv_kernel:
         monkeypatch.setenv("SBA_DKV_KERNEL", dkv_kernel)
