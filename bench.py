@@ -17,6 +17,7 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 BF16_MFMA_PEAK_TFLOPS = 2516.6     # 256 CU x 2.4 GHz x 4096 FLOP/clk/CU (dense bf16)
+HBM_PEAK_GBS = 8000.0               # MI355X HBM3E
 
 KERNEL_TIMING_SAMPLES = 5      # steps of the timed region whose kernels are timed with events
 # Counters cannot be read from inside this process: the figures below are copied from the rocprofv3
@@ -104,6 +105,25 @@ def make_workload(name, device):
         pairs = H * sum(L * (L - 1) // 2 for L in lens)
         cu_t = torch.tensor(cu, dtype=torch.int32, device=device)
         desc = {"workload": "cfg3: packed varlen fwd+bwd H=16 d=64 bf16, 65536 tokens, lognormal docs",
+                "H": H, "tokens": N, "d": D, "n_docs": len(lens), "max_len": max(lens)}
+        return desc, (q, k, v, do, cu_t, max(lens)), pairs, N, D, H
+    if name == "short":
+        # the short-document regime of a packed batch: too few pairs per token for the matrix cores to
+        # matter, every tensor is read once -> priced against the HBM roofline
+        H, N, D = 16, 65536, 64
+        lens, s_ = [], 0
+        while s_ < N:
+            L = min(int(torch.randint(16, 129, (1,), generator=g)), N - s_)
+            lens.append(L)
+            s_ += L
+        cu = [0]
+        for L in lens:
+            cu.append(cu[-1] + L)
+        q, k, v = rn((H, N, D), 0.5), rn((H, N, D), 0.5), rn((H, N, D), 0.5)
+        do = rn((H, N, D), 1.0)
+        pairs = H * sum(L * (L - 1) // 2 for L in lens)
+        cu_t = torch.tensor(cu, dtype=torch.int32, device=device)
+        desc = {"workload": "short: packed varlen fwd+bwd H=16 d=64 bf16, 65536 tokens in documents of 16..128 tokens",
                 "H": H, "tokens": N, "d": D, "n_docs": len(lens), "max_len": max(lens)}
         return desc, (q, k, v, do, cu_t, max(lens)), pairs, N, D, H
     raise SystemExit(f"unknown workload {name}")
@@ -229,7 +249,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--workload", default="cfg2", choices=["cfg2", "cfg3", "cfg4", "cfg5", "copy"])
+    ap.add_argument("--workload", default="cfg2", choices=["cfg2", "cfg3", "cfg4", "cfg5", "short", "copy"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--compile", action="store_true",
                     help="cfg5 only: torch.compile every block, as flame does with --training.compile")
@@ -310,6 +330,16 @@ def main():
                      "traffic": PROFILED_HBM_BYTES.get((args.workload, dom)),
                      "traffic_source": f"profiles/sba_{args.workload}_hbm_traffic.txt (rocprofv3 --pmc, not measured by this run)"},
     }
+    if args.workload == "short":
+        # algorithmic bytes per launch: q, k, v (+ dO) read once, the outputs written once (bf16), rem and the
+        # carries not counted: forward 4 tensors, dQ pass 5, dK/dV pass 6
+        unit = tokens * H * D * 2
+        nbytes = {"fwd": 4 * unit, "bwd_dq": 5 * unit, "bwd_dkv": 6 * unit}
+        gbs = {n: nbytes[n] / (kern[n] * 1e-3) / 1e9 for n in kern if n in nbytes}
+        out["roofline"] = {"bound": "hbm", "kernel": dom, "achieved": round(gbs[dom], 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                           "frac": round(gbs[dom] / HBM_PEAK_GBS, 4), "traffic": None,
+                           "per_kernel_GBps": {n: round(x, 1) for n, x in gbs.items()},
+                           "step_GBps": round(15 * unit / (ms * 1e-3) / 1e9, 1)}
     fl = issue_floor(args.workload, dom)
     if fl is not None:
         # what the dominant kernel could reach if only instruction issue limited it: MFMA time + vector time
@@ -320,7 +350,7 @@ def main():
                               "ns_per_instruction": ISSUE_NS,
                               "source": f"instruction counts from profiles/sba_{args.workload}_shader_counters.txt, "
                                         "issue rates from profiles/gfx950_issue_rates.txt"}
-    if not args.no_cpu_baseline:
+    if not args.no_cpu_baseline and args.workload != "short":     # (the CPU leg is defined for BASELINE's configurations)
         out["cpu_baseline"] = cpu_baseline(args.workload)
     print(json.dumps(out))
 
