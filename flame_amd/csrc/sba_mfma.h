@@ -640,6 +640,18 @@ __device__ inline void logit_grads(const float (&a)[32], const float (&beta)[32]
     }
 }
 
+// The same when the prefix entering this lane's keys is known up front (from the tables of the dQ pass):
+// one pass, no exchange.  Out: dp[idx] <- dz.
+template <int N>
+__device__ inline void logit_grads_from(const float (&a)[N], const float (&beta)[N], float (&dp)[N], float run) {
+#pragma unroll
+    for (int idx = 0; idx < N; ++idx) {
+        const float g = a[idx] * dp[idx];
+        run += g;
+        dp[idx] = __builtin_fmaf(-beta[idx], run, g);
+    }
+}
+
 // Register-lean form of the backward's per-step arithmetic for the row-owner kernel at head_dim
 // 128, where registers decide between one and two waves per SIMD: two arrays of 32 instead of
 // four.  Part 1 runs the reciprocal-per-key chain right-to-left and leaves, in place of the

@@ -611,7 +611,7 @@ __global__ __launch_bounds__((NP + 4) * 64, NP == 4 ? 2 : 3) void mfma_bwd_dkv_s
     constexpr int kQTile = 128 * D * 2;        // Q or dO tile (128 queries)
     constexpr int kZTile = 128 * 64 * 2;       // weights of one step, [query][key] bf16
     constexpr int kBuf = 2 * kZTile + 2 * kQTile;
-    constexpr int kCarry = kRowBlock * (NP == 4 ? 8 : 16);   // {R, G} per query; NP = 8: {R, G, R mid-block, G mid-block}
+    constexpr int kCarry = kRowBlock * 16;      // {R, G, R mid-block, G mid-block} per query
     __shared__ __attribute__((aligned(1024))) char lds[3 * kTile + 2 * kCarry + 2 * kBuf];
     __shared__ int consumers_done;             // consumer waves that have finished a reduction, running total
     __shared__ int producers_took_k;           // producer waves that hold an item's K fragments, running total
@@ -768,11 +768,17 @@ __global__ __launch_bounds__((NP + 4) * 64, NP == 4 ? 2 : 3) void mfma_bwd_dkv_s
                 float x[32], beta[32], dp[32];
                 float Gc = 0.f;
                 if (!skip) {
-                    const float2 cv = *(const float2*)(carry + (s & 1) * kCarry + (32 * w4 + n) * 8);
-                    // rows past the end of the sequence hold copies of its last row: a zero carry
-                    // makes their weights and gradients exactly zero
-                    float R = qi < len ? cv.x : 0.f;
-                    Gc = qi < len ? cv.y : 0.f;
+                    // Both carries that enter this LANE's 32 keys come from the tables: the right half-wave
+                    // takes the forward's block-edge product and the mid-block prefix, the left one the
+                    // mid-block product and the block-edge prefix - no exchange between the halves, and the
+                    // prefix sums run in one pass.  Entries of (query, half block) pairs that the query does not
+                    // see are not written: their weights are zero whatever the carry.  Rows past the end of
+                    // the sequence hold copies of its last row: a zero carry makes their weights and
+                    // gradients exactly zero.
+                    const float4 cv = *(const float4*)(carry + (s & 1) * kCarry + (32 * w4 + n) * 16);
+                    const bool sees = qi < len && qi - strict - (key0 + 32 * h) + 1 > 0;
+                    const float R = sees ? (h ? cv.x : cv.z) : (qi < len ? 1.0f : 0.0f);
+                    Gc = sees ? (h ? cv.w : cv.y) : 0.0f;
                     bf16x8 qf[D / 16], dof[D / 16];
 #pragma unroll
                     for (int ks = 0; ks < D / 16; ++ks) {
@@ -796,10 +802,11 @@ __global__ __launch_bounds__((NP + 4) * 64, NP == 4 ? 2 : 3) void mfma_bwd_dkv_s
                     // segments of the chain, where the chain's exp/rcp overlap them
                     static_assert(D == 64, "one dP MFMA per chain segment");
                     f32x16 dacc[2];
-                    stick_weights_hooked(x, beta, R, lane, nullptr, [&](int seg) {
+                    product_chain_with<true, 32>(x, beta, [&](int seg) {
                         const int t = seg & 1, ks = seg >> 1;
                         dacc[t] = mfma(vfr[t][ks], dof[ks], ks == 0 ? f32x16{0} : dacc[t]);
                     });
+                    scale_clamped<32>(x, R);
 #pragma unroll
                     for (int t = 0; t < 2; ++t)
 #pragma unroll
@@ -807,7 +814,7 @@ __global__ __launch_bounds__((NP + 4) * 64, NP == 4 ? 2 : 3) void mfma_bwd_dkv_s
                 }
                 if (x_now) __syncthreads();    // X
                 if (!skip) {
-                    logit_grads<true>(x, beta, dp, Gc, lane);
+                    logit_grads_from<32>(x, beta, dp, Gc);
                 } else {
 #pragma unroll
                     for (int idx = 0; idx < 32; ++idx) { x[idx] = 0.f; dp[idx] = 0.f; }
@@ -869,7 +876,7 @@ __global__ __launch_bounds__((NP + 4) * 64, NP == 4 ? 2 : 3) void mfma_bwd_dkv_s
         struct ItemPtrs {
             const char* x;                     // Q or dO: row 0 of the sequence, this head, this thread's chunk
             const float *rt, *gt;              // carries of this (head, key block): row block 0, query 0
-            const float *rm, *gm;              // NP = 8: the mid-block carries
+            const float *rm, *gm;              // the mid-block carries
             int row0, len;                     // first query of the item's sweep; sequence length
         };
         auto item_ptrs = [&](const KeyItem& t) {
@@ -884,7 +891,7 @@ __global__ __launch_bounds__((NP + 4) * 64, NP == 4 ? 2 : 3) void mfma_bwd_dkv_s
             r.row0 = t.job.rb * kRowBlock;
             r.len = t.job.len;
             asm volatile("" : "+v"(r.x), "+v"(r.rt), "+v"(r.gt));
-            if (NP == 8) asm volatile("" : "+v"(r.rm), "+v"(r.gm));
+            asm volatile("" : "+v"(r.rm), "+v"(r.gm));
             return r;
         };
         const uint32_t x_st2 = 2u * (uint32_t)(is_dv ? p.d_o.st : p.q.st);
@@ -893,14 +900,14 @@ __global__ __launch_bounds__((NP + 4) * 64, NP == 4 ? 2 : 3) void mfma_bwd_dkv_s
             const int qb = qi >> 7;            // row block of the query: its slab starts qb*(qb+1) columns in
             const int64_t ix = (int64_t)qb * (qb + 1) * kRowBlock + (qi & (kRowBlock - 1));
             cR = t.rt[ix]; cG = t.gt[ix];
-            if (NP == 8) { cRm = t.rm[ix]; cGm = t.gm[ix]; }
+            cRm = t.rm[ix]; cGm = t.gm[ix];
 #pragma unroll
             for (int i = 0; i < 8; ++i) {
                 const uint32_t row = (uint32_t)min(row0 + crow + 16 * i, t.len - 1);
                 tx[i] = *(const u32x4*)(t.x + (size_t)row * x_st2);
             }
         };
-        constexpr int kLoadsPerStep = 8 + (NP == 8 ? 4 : 2);      // per lane: what request_step issues
+        constexpr int kLoadsPerStep = 8 + 4;        // per lane: what request_step issues
         // K and V tiles of an item go straight from global memory into LDS (no registers, and
         // nothing for the wait-count bookkeeping to track): every instruction moves 64 x 16 bytes
         // into 1 KB of consecutive LDS, the lane picks the global chunk that belongs at its LDS
@@ -933,8 +940,7 @@ __global__ __launch_bounds__((NP + 4) * 64, NP == 4 ? 2 : 3) void mfma_bwd_dkv_s
 #pragma unroll
             for (int i = 0; i < 8; ++i) *(u32x4*)(xtile + tile_offset<D>(crow + 16 * i, cch)) = tx[i];
             if (ct < kRowBlock) {
-                if (NP == 8) *(float4*)(carry + (s & 1) * kCarry + ct * 16) = float4{cR, cG, cRm, cGm};
-                else *(float2*)(carry + (s & 1) * kCarry + ct * 8) = float2{cR, cG};
+                *(float4*)(carry + (s & 1) * kCarry + ct * 16) = float4{cR, cG, cRm, cGm};
             }
         };
         auto store_staged = [&](int idx, const char* staging) {
@@ -1378,9 +1384,9 @@ int sba_launch_mfma_bwd(const sba::KParams& kp_in, int phases, hipStream_t s) {
     // the stream with eight half-block producers (12 waves): measured within 1 % of the one with four
     // full-block producers (109.1 against 110.3 us at B=1 H=16 T=4096), which stays the default
     const bool stream8 = which && !strcmp(which, "stream8");
-    // the mid-block carries are read by the own-keys kernel and by the stream's half-block producers:
-    // otherwise the dQ pass skips them
-    if (!own && !(kp.head_dim == 64 && stream8 && !plain)) kp.rmid = kp.gmid = nullptr;
+    // the mid-block carries are read by the own-keys kernel and by the stream: otherwise the dQ pass
+    // skips them
+    if (!own && (kp.head_dim != 64 || plain)) kp.rmid = kp.gmid = nullptr;
     if (kp.head_dim == 64) {
         // small grids last as long as their longest sweep: take the variant that halves it
         if (p1 && grid.x <= sba_two_step_max_grid()) hipLaunchKernelGGL((mfma_bwd_dq2_kernel<64>), grid, dim3(2 * kThreads), 0, s, kp);
