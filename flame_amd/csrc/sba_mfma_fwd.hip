@@ -10,7 +10,7 @@ namespace sba {
 // One sweep step of one wave: 32 queries x 64 keys.  Scores (from the pre-scaled Q fragments),
 // mask on the diagonal, weights, O^T += V^T P^T.  kFast: the one-reciprocal chain; it may refuse
 // the step (returns false, nothing changed), see forward_weights_fast().
-template <int D, bool kCarryOnly, bool kFast>
+template <int D, bool kCarryOnly, bool kFast, bool kPinBase>
 __device__ inline bool fwd_step(const char* ktile, const char* vtile, const LaneOffsets<D>& lo,
                                 const bf16x8 (&qf)[D / 16], f32x16 (&oacc)[D / 32], float& R, int lane,
                                 int key0, int q0w, int qi, int strict) {
@@ -36,7 +36,7 @@ __device__ inline bool fwd_step(const char* ktile, const char* vtile, const Lane
 #pragma unroll
             for (int cc = 0; cc < 2; ++cc)
 #pragma unroll
-                for (int db = 0; db < D / 32; ++db) vt[cc][db] = fetch_cols_o<D>(vtile, lo, db, 2 * c2 + cc);
+                for (int db = 0; db < D / 32; ++db) vt[cc][db] = fetch_cols_o<D, kPinBase>(vtile, lo, db, 2 * c2 + cc);
             if (D == 128) __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
             for (int cc = 0; cc < 2; ++cc)
@@ -134,7 +134,7 @@ __global__ __launch_bounds__(kThreads) void mfma_fwd_kernel(KParams p) {
         const int key0 = step * kKeyBlock;
         const bool skip = key0 + strict > q0w + 31;       // whole step right of this wave's last query
         open_step(step, buf, skip);
-        if (!skip && !fwd_step<D, kCarryOnly, true>(ktile, ktile + kTile, lo, qf, oacc, R, lane, key0, q0w, qi, strict)) {
+        if (!skip && !fwd_step<D, kCarryOnly, true, D == 128>(ktile, ktile + kTile, lo, qf, oacc, R, lane, key0, q0w, qi, strict)) {
             redo = true;
             break;
         }
@@ -147,7 +147,7 @@ __global__ __launch_bounds__(kThreads) void mfma_fwd_kernel(KParams p) {
         const bool skip = key0 + strict > q0w + 31;
         if (!redo) open_step(step, buf, skip);
         redo = false;
-        if (!skip) fwd_step<D, kCarryOnly, false>(ktile, ktile + kTile, lo, qf, oacc, R, lane, key0, q0w, qi, strict);
+        if (!skip) fwd_step<D, kCarryOnly, false, D == 128>(ktile, ktile + kTile, lo, qf, oacc, R, lane, key0, q0w, qi, strict);
         wait_global_memory();
         __syncthreads();
     }
@@ -235,7 +235,7 @@ __global__ __launch_bounds__(G * kThreads) void mfma_fwd_seg_kernel(KParams p) {
         const int key0 = step * kKeyBlock;
         const bool skip = step < low || key0 + strict > q0w + 31;
         open_step(step, buf, skip);
-        if (!skip && !fwd_step<D, kCarryOnly, true>(ktile, ktile + kTile, lo, qf, oacc, R, lane, key0, q0w, qi, strict)) {
+        if (!skip && !fwd_step<D, kCarryOnly, true, true>(ktile, ktile + kTile, lo, qf, oacc, R, lane, key0, q0w, qi, strict)) {
             redo = true;
             break;
         }
@@ -249,7 +249,7 @@ __global__ __launch_bounds__(G * kThreads) void mfma_fwd_seg_kernel(KParams p) {
         const bool skip = step < low || key0 + strict > q0w + 31;
         if (!redo) open_step(step, buf, skip);
         redo = false;
-        if (!skip) fwd_step<D, kCarryOnly, false>(ktile, ktile + kTile, lo, qf, oacc, R, lane, key0, q0w, qi, strict);
+        if (!skip) fwd_step<D, kCarryOnly, false, true>(ktile, ktile + kTile, lo, qf, oacc, R, lane, key0, q0w, qi, strict);
         wait_global_memory();
         __syncthreads();
     }
