@@ -249,8 +249,20 @@ template <int D, bool kNatural = false> struct TileDma {      // kNatural: rows 
             off[i] = 2u * (uint32_t)(kl * st + c * 8);
         }
     }
+    // a tile known to lie inside the sequence (every key tile of a sweep but the rightmost)
+    __device__ inline void issue_full(int row0, char* tile) const {
+        const char* tile_base = origin + (((uint64_t)(uint32_t)row0 * (uint32_t)st) << 1);
+#pragma unroll
+        for (int i = 0; i < kPerWave; ++i)
+            __builtin_amdgcn_global_load_lds(
+                (const __attribute__((address_space(1))) void*)(tile_base + (size_t)off[i]),
+                (__attribute__((address_space(3))) void*)(uintptr_t)(uint32_t)(uintptr_t)(tile + (w4 + 4 * i) * 1024),
+                16, 0, 0);
+    }
     __device__ inline void issue(int row0, int len, char* tile) const {
-        const char* tile_base = origin + 2 * ((int64_t)row0 * st);          // uniform
+        // uniform; row0 and the stride are non-negative: the unsigned product is two scalar instructions, the
+        // signed 64-bit one about ten
+        const char* tile_base = origin + (((uint64_t)(uint32_t)row0 * (uint32_t)st) << 1);
         if (row0 + 64 <= len) {
 #pragma unroll
             for (int i = 0; i < kPerWave; ++i)

@@ -85,6 +85,7 @@ __global__ __launch_bounds__(kThreads) void mfma_fwd_kernel(KParams p) {
     const int m0 = job.rb * kRowBlock;
     const int q0w = m0 + 32 * wave;              // first query of this wave
     const int qi = q0w + n;                      // this lane's query
+    const bool rows_full = q0w + 31 < job.len;   // wave-uniform
     const int64_t qbase = (int64_t)job.seq * p.q.sb + (int64_t)head * p.q.sh + (int64_t)job.tok0 * p.q.st;
     const int64_t kbase = (int64_t)job.seq * p.k.sb + (int64_t)head * p.k.sh + (int64_t)job.tok0 * p.k.st;
     const int64_t vbase = (int64_t)job.seq * p.v.sb + (int64_t)head * p.v.sh + (int64_t)job.tok0 * p.v.st;
@@ -118,10 +119,16 @@ __global__ __launch_bounds__(kThreads) void mfma_fwd_kernel(KParams p) {
         // The carry-table store goes FIRST: vector-memory operations retire in order, so the
         // wait for the tile loads at the end of the step then also covers this store, long
         // after it has completed, instead of stalling the next iteration's loads on it.
-        if (!skip && p.save && h == 0 && qi < job.len) p.rtab[tabq + step * kRowBlock] = R;
-        if (step > 0) {   // next tiles, straight into the other buffer (free since the last barrier)
-            kc.issue((step - 1) * kKeyBlock, job.len, lds + (buf ^ 1) * 2 * kTile);
-            if (!kCarryOnly) vc.issue((step - 1) * kKeyBlock, job.len, lds + (buf ^ 1) * 2 * kTile + kTile);
+        // (A wave whose 32 rows all exist stores with every lane - both half-waves hold the same carry and
+        // write it to the same entry -, which spares the lane mask per step.)
+        if (!skip && p.save) {
+            if (rows_full) p.rtab[tabq + step * kRowBlock] = R;
+            else if (h == 0 && qi < job.len) p.rtab[tabq + step * kRowBlock] = R;
+        }
+        if (step > 0) {   // next tiles, straight into the other buffer (free since the last barrier);
+                          // every tile left of the sweep's first lies inside the sequence
+            kc.issue_full((step - 1) * kKeyBlock, lds + (buf ^ 1) * 2 * kTile);
+            if (!kCarryOnly) vc.issue_full((step - 1) * kKeyBlock, lds + (buf ^ 1) * 2 * kTile + kTile);
         }
     };
     // The sweep runs with the one-reciprocal chain until a step refuses it (logits too large for
@@ -189,6 +196,7 @@ __global__ __launch_bounds__(G * kThreads) void mfma_fwd_seg_kernel(KParams p) {
     const int m0 = job.rb * kRowBlock;
     const int q0w = m0 + 32 * qs;
     const int qi = q0w + n;
+    const bool rows_full = q0w + 31 < job.len;      // wave-uniform
     const int64_t qbase = (int64_t)job.seq * p.q.sb + (int64_t)head * p.q.sh + (int64_t)job.tok0 * p.q.st;
     const int64_t kbase = (int64_t)job.seq * p.k.sb + (int64_t)head * p.k.sh + (int64_t)job.tok0 * p.k.st;
     const int64_t vbase = (int64_t)job.seq * p.v.sb + (int64_t)head * p.v.sh + (int64_t)job.tok0 * p.v.st;
@@ -221,10 +229,13 @@ __global__ __launch_bounds__(G * kThreads) void mfma_fwd_seg_kernel(KParams p) {
     __syncthreads();
 
     auto open_step = [&](int step, int buf, bool skip) {
-        if (!skip && p.save && h == 0 && qi < job.len) p.rtab[tabq + step * kRowBlock] = R;   // relative to the segment's right edge
+        if (!skip && p.save) {                 // relative to the segment's right edge
+            if (rows_full) p.rtab[tabq + step * kRowBlock] = R;          // every lane stores: no lane mask per step
+            else if (h == 0 && qi < job.len) p.rtab[tabq + step * kRowBlock] = R;
+        }
         if (step - 1 >= low) {
-            kc.issue((step - 1) * kKeyBlock, job.len, my_tiles + (buf ^ 1) * 2 * kTile);
-            if (!kCarryOnly) vc.issue((step - 1) * kKeyBlock, job.len, my_tiles + (buf ^ 1) * 2 * kTile + kTile);
+            kc.issue_full((step - 1) * kKeyBlock, my_tiles + (buf ^ 1) * 2 * kTile);
+            if (!kCarryOnly) vc.issue_full((step - 1) * kKeyBlock, my_tiles + (buf ^ 1) * 2 * kTile + kTile);
         }
     };
     int it = 0, buf = 0;
