@@ -150,11 +150,21 @@ __device__ inline bf16x8 fetch_cols_o(const char* tile, const LaneOffsets<D>& o,
     }
     return u.b;
 }
-template <int D> __device__ inline bf16x8 fetch_nat_o(const char* tile, const LaneOffsets<D>& o, int row0, int cb) {
+template <int D, bool kPinBase = false>
+__device__ inline bf16x8 fetch_nat_o(const char* tile, const LaneOffsets<D>& o, int row0, int cb) {
     union { s16x4 v[2]; bf16x8 b; } u;
-    u.v[0] = lds_read_tr(tile + o.nat[0][cb] + row0 * D * 2);
-    u.v[1] = lds_read_tr(tile + o.nat[1][cb] + row0 * D * 2);
+    if (kPinBase) {
+        u.v[0] = lds_read_tr_at(lds_lane_base(tile, o.nat[0][cb]), row0 * D * 2);
+        u.v[1] = lds_read_tr_at(lds_lane_base(tile, o.nat[1][cb]), row0 * D * 2);
+    } else {
+        u.v[0] = lds_read_tr(tile + o.nat[0][cb] + row0 * D * 2);
+        u.v[1] = lds_read_tr(tile + o.nat[1][cb] + row0 * D * 2);
+    }
     return u.b;
+}
+// fetch_rows_o with the pinned base (see fetch_cols_o): row 32*t + lane%32 of a tile in natural or MFMA order
+template <int D> __device__ inline bf16x8 fetch_rows_p(const char* tile, const LaneOffsets<D>& o, int t, int ks) {
+    return *(const __attribute__((address_space(3))) bf16x8*)((__attribute__((address_space(3))) char*)(uintptr_t)lds_lane_base(tile, o.rows[ks]) + t * 32 * D * 2);
 }
 // The same with the two lane offsets already picked (column block chosen at run time:
 // indexing the offset table with a run-time value would push it into scratch memory).

@@ -1115,6 +1115,8 @@ __global__ __launch_bounds__(kThreads, D == 64 ? 2 : 1) void mfma_bwd_dkv_own_ke
     // and goes between the segments of that step's first chain.  The Q / dO tiles of a step then
     // have to outlive it by one step: three tile buffers instead of two.
     constexpr bool kDefer = D == 128;
+    // LDS fetches with the pinned base (see fetch_cols_o): -1.6 % at head_dim 64, +2.5 % at 128 (registers)
+    constexpr bool kOwnPin = D == 64;
     constexpr int kNBuf = kDefer ? 3 : 2;
     __shared__ __attribute__((aligned(16))) char lds[2 * kNBuf * kQTile + 4 * kZTile];   // Q, dO per buffer | one Z tile per wave
 
@@ -1185,12 +1187,12 @@ __global__ __launch_bounds__(kThreads, D == 64 ? 2 : 1) void mfma_bwd_dkv_own_ke
     auto second_tile_reduction = [&](const char* qt, const char* dot) {
 #pragma unroll
         for (int kk = 2; kk < 4; ++kk) {
-            const bf16x8 af = fetch_nat_o<64>(ztile, lz, 16 * kk, 0);
-            const bf16x8 zf = fetch_nat_o<64>(ztile, lz, 16 * kk, 1);
+            const bf16x8 af = fetch_nat_o<64, kOwnPin>(ztile, lz, 16 * kk, 0);
+            const bf16x8 zf = fetch_nat_o<64, kOwnPin>(ztile, lz, 16 * kk, 1);
 #pragma unroll
             for (int db = 0; db < D / 32; ++db) {
-                dvacc[db] = mfma(af, fetch_nat_o<D>(dot, lo, 16 * kk, db), dvacc[db]);
-                dkacc[db] = mfma(zf, fetch_nat_o<D>(qt, lo, 16 * kk, db), dkacc[db]);
+                dvacc[db] = mfma(af, fetch_nat_o<D, kOwnPin>(dot, lo, 16 * kk, db), dvacc[db]);
+                dkacc[db] = mfma(zf, fetch_nat_o<D, kOwnPin>(qt, lo, 16 * kk, db), dkacc[db]);
             }
         }
     };
@@ -1230,7 +1232,7 @@ __global__ __launch_bounds__(kThreads, D == 64 ? 2 : 1) void mfma_bwd_dkv_own_ke
                     // each MFMA: all operands of the tile are requested first
                     bf16x8 bq[D / 16];
 #pragma unroll
-                    for (int ks = 0; ks < D / 16; ++ks) bq[ks] = fetch_row_nat<D>(qtile, 32 * t + n, ks, lane);
+                    for (int ks = 0; ks < D / 16; ++ks) bq[ks] = kOwnPin ? fetch_rows_p<D>(qtile, lo, t, ks) : fetch_row_nat<D>(qtile, 32 * t + n, ks, lane);
                     if (D == 128) __builtin_amdgcn_sched_barrier(0);
                     f32x16 acc = {0};
 #pragma unroll
@@ -1246,8 +1248,8 @@ __global__ __launch_bounds__(kThreads, D == 64 ? 2 : 1) void mfma_bwd_dkv_own_ke
                 if (t == 0 && kDefer && pending) {
                     // the previous step's second tile: rows 32.. of the wave's weight tile (not yet
                     // overwritten: this step's second tile comes later) and of the previous Q / dO tiles
-                    auto red_a = [&](int seg) { return fetch_nat_o<64>(ztile, lz, 32 + 16 * (seg >> 1), seg & 1); };
-                    auto red_b = [&](int seg, int db) { return fetch_nat_o<D>((seg & 1) ? pqtile : pdotile, lo, 32 + 16 * (seg >> 1), db); };
+                    auto red_a = [&](int seg) { return fetch_nat_o<64, kOwnPin>(ztile, lz, 32 + 16 * (seg >> 1), seg & 1); };
+                    auto red_b = [&](int seg, int db) { return fetch_nat_o<D, kOwnPin>((seg & 1) ? pqtile : pdotile, lo, 32 + 16 * (seg >> 1), db); };
                     bf16x8 na = red_a(0), nb[D / 32];
 #pragma unroll
                     for (int db = 0; db < D / 32; ++db) nb[db] = red_b(0, db);
@@ -1273,8 +1275,8 @@ __global__ __launch_bounds__(kThreads, D == 64 ? 2 : 1) void mfma_bwd_dkv_own_ke
                     // The reduction over the first tile's 32 queries only needs that tile's weights, which
                     // this wave wrote above: its MFMAs go between the segments of the second tile's chain,
                     // whose exp/rcp overlap them.  Segment 2kk: dV += A^T dO, segment 2kk + 1: dK += dZ^T Q.
-                    auto red_a = [&](int seg) { return fetch_nat_o<64>(ztile, lz, 16 * (seg >> 1), seg & 1); };
-                    auto red_b = [&](int seg, int db) { return fetch_nat_o<D>((seg & 1) ? qtile : dotile, lo, 16 * (seg >> 1), db); };
+                    auto red_a = [&](int seg) { return fetch_nat_o<64, kOwnPin>(ztile, lz, 16 * (seg >> 1), seg & 1); };
+                    auto red_b = [&](int seg, int db) { return fetch_nat_o<D, kOwnPin>((seg & 1) ? qtile : dotile, lo, 16 * (seg >> 1), db); };
                     bf16x8 na = red_a(0), nb[D / 32];
 #pragma unroll
                     for (int db = 0; db < D / 32; ++db) nb[db] = red_b(0, db);
@@ -1298,7 +1300,7 @@ __global__ __launch_bounds__(kThreads, D == 64 ? 2 : 1) void mfma_bwd_dkv_own_ke
                 {
                     bf16x8 bd[D / 16];
 #pragma unroll
-                    for (int ks = 0; ks < D / 16; ++ks) bd[ks] = fetch_row_nat<D>(dotile, 32 * t + n, ks, lane);
+                    for (int ks = 0; ks < D / 16; ++ks) bd[ks] = kOwnPin ? fetch_rows_p<D>(dotile, lo, t, ks) : fetch_row_nat<D>(dotile, 32 * t + n, ks, lane);
                     if (D == 128) __builtin_amdgcn_sched_barrier(0);
                     f32x16 acc = {0};
 #pragma unroll
