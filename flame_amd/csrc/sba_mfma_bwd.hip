@@ -652,6 +652,10 @@ __global__ __launch_bounds__((NP + 4) * 64, NP == 4 ? 2 : 3) void mfma_bwd_dkv_s
         __syncthreads();                       // first item's tiles and carries visible
         int s = 0;
         bool staged_prev = false;              // the consumers staged a dK/dV in the previous iteration
+        // the logit scale in a VECTOR register: a multiply with a scalar-register operand takes a whole
+        // quad-cycle, one on vector registers half of that
+        float scale2v = p.scale2;
+        asm volatile("" : "+v"(scale2v));
         if constexpr (NP == 8) {
         const int kh = wave >> 2;              // this wave's half of the 64-key block
         for (int item = 0;; ++item) {
@@ -700,7 +704,7 @@ __global__ __launch_bounds__((NP + 4) * 64, NP == 4 ? 2 : 3) void mfma_bwd_dkv_s
 #pragma unroll
                     for (int ks = 0; ks < D / 16; ++ks) acc = mfma(kfr[ks], qf[ks], acc);
 #pragma unroll
-                    for (int r = 0; r < 16; ++r) x[r] = acc[r] * p.scale2;
+                    for (int r = 0; r < 16; ++r) x[r] = acc[r] * scale2v;
                     if (key0 + 31 + strict > q0w || q0w + 31 >= len) {        // diagonal or ragged tile
                         const int nvis = qi < len ? qi - strict - (key0 + 16 * h) + 1 : 0;
 #pragma unroll
@@ -796,7 +800,7 @@ __global__ __launch_bounds__((NP + 4) * 64, NP == 4 ? 2 : 3) void mfma_bwd_dkv_s
 #pragma unroll
                     for (int t = 0; t < 2; ++t)
 #pragma unroll
-                        for (int r = 0; r < 16; ++r) x[16 * t + r] = raw[t][r] * p.scale2;
+                        for (int r = 0; r < 16; ++r) x[16 * t + r] = raw[t][r] * scale2v;
                     if (key0 + 63 + strict > q0w) mask_step(x, key0 + 32 * h, qi, strict);
                     // dP = dO V^T does not depend on the weights: its eight MFMAs go between the
                     // segments of the chain, where the chain's exp/rcp overlap them
