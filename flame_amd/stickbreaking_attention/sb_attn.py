@@ -147,6 +147,9 @@ def sb_attn(q, k, v, inv_temp=None, zero_start=True, attend_current=False):
 
 
 def sb_attn_(q, k, v, inv_temp, attend_current):
+    if q.numel() == 0:
+        # nothing to launch (an empty batch or a zero-length sequence): empty results that stay in the graph
+        return q * 0, q.sum(-1) * 0
     if not torch.is_grad_enabled():
         # no backward can follow: detached inputs tell the forward to keep no carry table
         q, k, v = q.detach(), k.detach(), v.detach()

@@ -217,6 +217,9 @@ def sb_attn_varlen(q, k, v, cu_seqlens, max_seqlens, inv_temp=None, zero_start=T
 
 
 def _apply(q, k, v, cu_seqlens, max_seqlens, inv_temp, attend_current):
+    if q.numel() == 0:
+        # no tokens (or no heads): nothing to launch; empty results that stay in the graph
+        return q * 0, q.sum(-1) * 0
     if not torch.is_grad_enabled():
         # no backward can follow: detached inputs tell the forward to keep no carry table
         q, k, v = q.detach(), k.detach(), v.detach()
