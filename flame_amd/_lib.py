@@ -142,16 +142,14 @@ def recompute_carries() -> bool:
 
 
 def matrix_core_head_dim(t: torch.Tensor) -> int:
-    """Head dim that a problem runs with.  The matrix-core kernels exist for bf16 at 64 and 128 and
-    for fp32 at 64; any other head dim below those rides them zero-padded (zero columns add nothing
-    to q.k and give zero output columns), which is far faster than the generic kernels.  fp32 above
-    64 keeps its head dim (generic kernels), and so does everything under SBA_FORCE_GENERIC=1."""
+    """Head dim that a problem runs with.  The matrix-core kernels exist for bf16 and fp32 at 64 and
+    128; any other head dim below those rides them zero-padded (zero columns add nothing to q.k and
+    give zero output columns), which is far faster than the generic kernels.  Everything keeps its
+    head dim under SBA_FORCE_GENERIC=1 (generic kernels)."""
     D = t.shape[-1]
     if D > 128 or os.environ.get("SBA_FORCE_GENERIC") == "1":
         return D
-    if t.dtype == torch.float32:
-        return 64 if D <= 64 else D
-    if t.dtype != torch.bfloat16 or D in (64, 128):
+    if t.dtype not in (torch.bfloat16, torch.float32) or D in (64, 128):
         return D
     return 64 if D < 64 else 128
 

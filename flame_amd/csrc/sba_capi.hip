@@ -23,12 +23,11 @@ bool force_generic() {
     return e && e[0] == '1';
 }
 
-// The matrix-core kernels cover bf16 with head_dim 64 or 128 and fp32 with head_dim 64;
-// everything else takes the generic vector-ALU kernels.
+// The matrix-core kernels cover bf16 and fp32 with head_dim 64 or 128; everything else takes the
+// generic vector-ALU kernels.
 bool use_mfma(const SbaParams* p) {
     if (force_generic()) return false;
-    if (p->dtype == SBA_DTYPE_F32) return p->head_dim == 64;
-    return p->dtype == SBA_DTYPE_BF16 && (p->head_dim == 64 || p->head_dim == 128);
+    return (p->dtype == SBA_DTYPE_F32 || p->dtype == SBA_DTYPE_BF16) && (p->head_dim == 64 || p->head_dim == 128);
 }
 
 // The MFMA backward is a separate switch so that the two directions can be brought up

@@ -97,7 +97,9 @@ def test_workspace_bytes(lib):
     p.workspace = None
     p.dtype = _lib.SBA_DTYPE_F32                    # fp32 at head_dim 64 runs on the matrix cores too: same tables
     assert lib.sba_workspace_bytes(C.byref(p)) == table
-    p.head_dim = 128                                # generic kernels: nothing kept, fp32 dk|dv accumulators
+    p.head_dim = 128                                # and at head_dim 128
+    assert lib.sba_workspace_bytes(C.byref(p)) == table
+    p.head_dim = 96                                 # generic kernels: nothing kept, fp32 dk|dv accumulators
     assert lib.sba_workspace_bytes(C.byref(p)) == 0
     assert lib.sba_bwd_scratch_bytes(C.byref(p)) == 2 * 4096 * 16 * 128 * 4
 

@@ -52,7 +52,7 @@ def test_config1_fp32_forward_and_grads():
 
 
 @pytest.mark.parametrize("T", [1, 2, 31, 64, 65, 130, 257])
-@pytest.mark.parametrize("D", [8, 64, 128])
+@pytest.mark.parametrize("D", [8, 64, 96, 128])
 def test_fp32_ragged_shapes(T, D):
     _check_dense(1, 2, T, D, torch.float32, seed=T + D)
 
@@ -607,15 +607,16 @@ def test_recomputing_the_carries_in_the_backward_gives_the_same_bits(D, monkeypa
             assert torch.equal(x, y)
 
 
-def test_fp32_runs_on_the_matrix_cores_bit_reproducibly_and_agrees_with_the_generic_kernels(monkeypatch):
-    # fp32 at head_dim <= 64 takes the fp32 MFMA kernels (no atomics): two runs give identical bits,
+@pytest.mark.parametrize("D", [64, 128])
+def test_fp32_runs_on_the_matrix_cores_bit_reproducibly_and_agrees_with_the_generic_kernels(D, monkeypatch):
+    # fp32 takes the fp32 MFMA kernels (head_dim 64 and 128, no atomics): two runs give identical bits,
     # dense and packed; the generic vector-ALU kernels (a separate implementation) agree to fp32 accuracy
     sb_attn, sb_attn_varlen = _ops()
-    q, k, v, do = (randn((2, 3, 333, 64), 500 + i, 1.0 if i < 3 else 1.0).cuda() for i in range(4))
+    q, k, v, do = (randn((2, 3, 333, D), 500 + i, 1.0 if i < 3 else 1.0).cuda() for i in range(4))
     drem = randn((2, 3, 333), 505).cuda()
     lens = [70, 1, 200, 129, 266]
     cu = cu_from_lengths(lens).cuda()
-    qp, kp, vp, dop = (x.reshape(6, 333, 64)[:, :, :].reshape(3, 666, 64).contiguous() for x in (q, k, v, do))
+    qp, kp, vp, dop = (x.reshape(6, 333, D)[:, :, :].reshape(3, 666, D).contiguous() for x in (q, k, v, do))
 
     def dense():
         qq, kk, vv = (x.clone().requires_grad_(True) for x in (q, k, v))
