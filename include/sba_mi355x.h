@@ -25,9 +25,10 @@
  *   packed [H, sumT, D]  : n_seq = number of documents, cu_seqlens = device int32[n_seq+1]
  *                          with cu_seqlens[0] == 0, stride_b = 0,
  *                          element (h,t,d) at    base + h*stride_h + t*stride_t + d
- * Strides are in elements; the innermost (D) stride is 1.  bf16 problems at head_dim 64 / 128
+ * Strides are in elements; the innermost (D) stride is 1.  Problems at head_dim 64 / 128
  * (the matrix-core kernels) need 16-byte aligned tensor pointers and outer strides that are
- * multiples of 8 elements (SBA_ERR_SHAPE otherwise); rem / d_rem are contiguous along tokens.
+ * multiples of 16 bytes - 8 bf16 or 4 fp32 elements - (SBA_ERR_SHAPE otherwise); rem / d_rem
+ * are contiguous along tokens.
  */
 #ifndef SBA_MI355X_H
 #define SBA_MI355X_H
