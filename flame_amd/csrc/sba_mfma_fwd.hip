@@ -319,15 +319,11 @@ __global__ __launch_bounds__(G * kThreads) void mfma_fwd_seg_kernel(KParams p) {
 
 }  // namespace sba
 
-// Groups per workgroup of the segmented forward (SBA_FWD_GROUPS overrides it for experiments;
-// read once per process).
+// Groups per workgroup of the segmented forward (SBA_FWD_GROUPS overrides it for experiments and tests).
 static int sba_fwd_groups() {
-    static const int v = [] {
-        const char* e = getenv("SBA_FWD_GROUPS");
-        const int g = e ? atoi(e) : 4;
-        return g == 2 || g == 3 || g == 4 ? g : 4;
-    }();
-    return v;
+    const char* e = getenv("SBA_FWD_GROUPS");
+    const int g = e ? atoi(e) : 4;
+    return g == 2 || g == 3 || g == 4 ? g : 4;
 }
 
 template <bool kCarryOnly>

@@ -364,12 +364,17 @@ def test_torch_compile_fullgraph_matches_eager():
         assert torch.equal(a, b)
 
 
-def test_small_and_large_grids_take_different_forward_kernels_and_agree():
-    # <= 512 workgroups: two-step-per-iteration forward; above: one step per iteration.
-    # Same rows computed both ways (a batch of 1 vs the same sequence repeated 40 times).
+def test_small_and_large_grids_take_different_forward_kernels_and_agree(monkeypatch):
+    # <= 512 workgroups: the segmented forward (2, 3 or 4 key segments per sweep); above: one workgroup per
+    # sweep.  Same rows computed all ways (a batch of 1 vs the same sequence repeated 40 times).
     sb_attn, _ = _ops()
     q, k, v = (randn((1, 4, 1000, 64), 110 + i, 0.5, torch.bfloat16).cuda() for i in range(3))
     o1, r1 = sb_attn(q, k, v)                                   # 8 row-blocks x 4 heads = 32 workgroups
+    for groups in ("2", "3"):
+        monkeypatch.setenv("SBA_FWD_GROUPS", groups)
+        og, rg = sb_attn(q, k, v)
+        assert max_abs(o1.float(), og.float()) <= 2e-2 and max_abs(r1.float(), rg.float()) <= 1e-2
+    monkeypatch.delenv("SBA_FWD_GROUPS")
     qq, kk, vv = (x.expand(40, -1, -1, -1).contiguous() for x in (q, k, v))
     o2, r2 = sb_attn(qq, kk, vv)                                # 1280 workgroups
     assert max_abs(o1.float(), o2[:1].float()) <= 2e-2 and max_abs(r1.float(), r2[:1].float()) <= 1e-2
