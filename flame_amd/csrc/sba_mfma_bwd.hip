@@ -1347,6 +1347,186 @@ __global__ __launch_bounds__(kThreads, D == 64 ? 2 : 1) void mfma_bwd_dkv_own_ke
     }
 }
 
+
+// ---------------------------------------------------------------- pass 2, two waves per 32 keys
+// What a wave of the own-keys kernel holds for its 32 keys at head_dim 128 - K and V fragments and the
+// [32 keys x 128] accumulators of dK and dV - is 190 registers: one wave per SIMD.  Here TWO waves share
+// 32 keys.  Both hold the K and V fragments; wave r of the pair turns query tile r of the step (32 of
+// its 64 queries) into weights and logit gradients and writes them to the pair's tile in LDS; after a
+// barrier each wave reduces ALL 64 queries of the step for ITS half of the head dim (column blocks
+// 2r, 2r + 1 at head_dim 128), so it accumulates [32 keys x D/2] of dK and of dV only.  The vector work
+// of a step is split between the two, the reductions too: eight waves per workgroup (128 keys), two per
+// SIMD.  Two workgroup barriers per step (weights complete; tiles handed over).
+template <int D>
+__global__ __launch_bounds__(2 * kThreads, 2) void mfma_bwd_dkv_pair_kernel(KParams p) {
+    constexpr int kQTile = 64 * D * 2;           // Q or dO tile of one step (64 queries)
+    constexpr int kZTile = 64 * 64 * 2;          // per pair: [64 queries][32 a | 32 dz] bf16
+    constexpr int kStep = 64;
+    constexpr bool kPairPin = true;              // LDS fetch bases pinned in registers: 3 % faster here
+    constexpr int kBlocks = D / 64;              // 32-wide column blocks of dK / dV per wave
+    static_assert(32 * D * 2 <= kZTile, "the pair's tile doubles as the staging of its [32 keys x D] outputs");
+    __shared__ __attribute__((aligned(16))) char lds[4 * kQTile + 4 * kZTile];   // (Q, dO) x 2 buffers | one Z tile per pair
+
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int grp = wave >> 1, r = wave & 1;
+    const int n = lane & 31, h = lane >> 5;
+    LaneOffsets<D> lo;
+    lo.init(lane);
+    LaneOffsets<64> lz;
+    lz.init(lane);
+    const int head = blockIdx.x % p.n_heads;
+    const Job job = decode_key_job(p, blockIdx.x / p.n_heads);
+    const int strict = p.attend_current ? 0 : 1;
+    const int q_begin = job.rb * kRowBlock;            // first key of the block = first query that may see it
+    const int kb0 = q_begin + 32 * grp;                // first key of this pair
+    char* ztile = lds + 4 * kQTile + grp * kZTile;
+
+    const int64_t qbase = (int64_t)job.seq * p.q.sb + (int64_t)head * p.q.sh + (int64_t)job.tok0 * p.q.st;
+    const int64_t kbase = (int64_t)job.seq * p.k.sb + (int64_t)head * p.k.sh + (int64_t)job.tok0 * p.k.st;
+    const int64_t vbase = (int64_t)job.seq * p.v.sb + (int64_t)head * p.v.sh + (int64_t)job.tok0 * p.v.st;
+    const int64_t dobase = (int64_t)job.seq * p.d_o.sb + (int64_t)head * p.d_o.sh + (int64_t)job.tok0 * p.d_o.st;
+
+    // A operands of the score tile: MFMA row m holds key 16*((m>>2)&1) + 4*(m>>3) + (m&3) of the pair,
+    // so that the accumulator registers of a lane are 16 consecutive keys (as in the own-keys kernel)
+    bf16x8 kfr[D / 16], vfr[D / 16];
+    {
+        const int m = lane & 31;
+        const int key = kb0 + 16 * ((m >> 2) & 1) + 4 * (m >> 3) + (m & 3);
+        load_row_frags<D>(kfr, p.k, kbase, key, job.len, lane);
+        load_row_frags<D>(vfr, p.v, vbase, key, job.len, lane);
+        prescale_frags(kfr, p.scale2);
+    }
+    f32x16 dkacc[kBlocks], dvacc[kBlocks];
+#pragma unroll
+    for (int j = 0; j < kBlocks; ++j) { dkacc[j] = f32x16{0}; dvacc[j] = f32x16{0}; }
+
+    const int n_steps = q_begin < job.len ? (job.len - q_begin + kStep - 1) / kStep : 0;
+
+    // waves 0-3 copy the Q tiles, waves 4-7 the dO tiles
+    TileDma<D, true> tc;
+    tc.init(lane, wave & 3, wave < 4 ? p.q : p.d_o, wave < 4 ? qbase : dobase);
+    const int my_tile = wave < 4 ? 0 : kQTile;
+    if (n_steps > 0) tc.issue(q_begin, job.len, lds + my_tile);
+
+    // carries of a (query, this pair's 32 keys) pair, see the own-keys kernel
+    const int kb64 = kb0 / kKeyBlock;
+    const float* rsrc = ((grp & 1) ? p.rtab : p.rmid) + tab_index(p, head, job, 0, kb64);
+    const float* gsrc = ((grp & 1) ? p.gmid : p.gtab) + tab_index(p, head, job, 0, kb64);
+    float Rn = 1.f, Gn = 0.f;
+    auto request_carries = [&](int q0) {
+        const int qi = min(q0 + 32 * r + n, job.len - 1);
+        const int qb = qi >> 7;
+        const int64_t ix = (int64_t)qb * (qb + 1) * kRowBlock + (qi & (kRowBlock - 1));
+        Rn = rsrc[ix];
+        Gn = gsrc[ix];
+    };
+    if (n_steps > 0) request_carries(q_begin);
+    wait_global_memory();
+    __syncthreads();
+
+    for (int step = 0, buf = 0; step < n_steps; ++step, buf ^= 1) {
+        const char* qtile = lds + buf * 2 * kQTile;
+        const char* dotile = qtile + kQTile;
+        const int q0 = q_begin + step * kStep;
+        const float Rin = Rn, Gin = Gn;
+        if (step + 1 < n_steps) {     // next tiles, straight into the other buffer (nobody reads it since the last barrier)
+            tc.issue(q0 + kStep, job.len, lds + (buf ^ 1) * 2 * kQTile + my_tile);
+            request_carries(q0 + kStep);
+        }
+        // whole step left of this pair's first key: nothing visible (the same for both waves of the pair)
+        const bool skip = kb0 + strict > q0 + kStep - 1 || kb0 >= job.len;
+        if (!skip) {
+            const int qt0 = q0 + 32 * r;
+            const int qi = qt0 + n;
+            float x[16], dp[16];
+            if (kb0 + strict > qt0 + 31) {             // this wave's query tile sees none of the keys (the other one does)
+#pragma unroll
+                for (int idx = 0; idx < 16; ++idx) { x[idx] = 0.f; dp[idx] = 0.f; }
+            } else {
+                const int nvis = qi < job.len ? qi - strict - (kb0 + 16 * h) + 1 : 0;
+                const bool sees = qi < job.len && qi - strict - kb0 + 1 > 0;
+                const float Rt = sees ? Rin : 1.0f;      // table entries of invisible pairs are not written
+                const float Gt = sees ? Gin : 0.0f;
+                float beta[16];
+                {
+                    bf16x8 bq[D / 16];
+#pragma unroll
+                    for (int ks = 0; ks < D / 16; ++ks) bq[ks] = fetch_rows_p<D>(qtile, lo, r, ks);
+                    f32x16 acc = {0};
+#pragma unroll
+                    for (int ks = 0; ks < D / 16; ++ks) acc = mfma(kfr[ks], bq[ks], acc);
+#pragma unroll
+                    for (int i = 0; i < 16; ++i) x[i] = acc[i];
+                }
+                if (kb0 + 31 + strict > qt0 || qt0 + 31 >= job.len) {     // diagonal or ragged tile
+#pragma unroll
+                    for (int idx = 0; idx < 16; ++idx)
+                        if (idx >= nvis) x[idx] = -INFINITY;
+                }
+                // dP = dO V^T between the segments of the chain
+                bf16x8 bd[D / 16];
+#pragma unroll
+                for (int ks = 0; ks < D / 16; ++ks) bd[ks] = fetch_rows_p<D>(dotile, lo, r, ks);
+                f32x16 dacc;
+                own_tile_weights(x, beta, Rt, lane, [&](int seg) {
+#pragma unroll
+                    for (int i = 0; i < D / 64; ++i) {
+                        const int ks = (D / 64) * seg + i;
+                        dacc = mfma(vfr[ks], bd[ks], ks == 0 ? f32x16{0} : dacc);
+                    }
+                });
+#pragma unroll
+                for (int i = 0; i < 16; ++i) dp[i] = dacc[i];
+                // a -> columns 16h.. of row (32r + n) now, dz -> columns 32 + 16h.. below
+                *(bf16x8*)(ztile + tile_offset<64>(32 * r + n, 2 * h)) = pack8(&x[0]);
+                *(bf16x8*)(ztile + tile_offset<64>(32 * r + n, 2 * h + 1)) = pack8(&x[8]);
+                own_tile_grads(x, beta, dp, Gt, lane);
+            }
+            if (kb0 + strict > qt0 + 31) {
+                *(bf16x8*)(ztile + tile_offset<64>(32 * r + n, 2 * h)) = pack8(&x[0]);
+                *(bf16x8*)(ztile + tile_offset<64>(32 * r + n, 2 * h + 1)) = pack8(&x[8]);
+            }
+            *(bf16x8*)(ztile + tile_offset<64>(32 * r + n, 4 + 2 * h)) = pack8(&dp[0]);
+            *(bf16x8*)(ztile + tile_offset<64>(32 * r + n, 4 + 2 * h + 1)) = pack8(&dp[8]);
+        }
+        __syncthreads();                       // the pair's weights are complete
+        if (!skip) {
+            // dV += A^T dO, dK += dZ^T Q over the step's 64 queries, this wave's column blocks
+#pragma unroll
+            for (int kk = 0; kk < 4; ++kk) {
+                const bf16x8 af = fetch_nat_o<64, kPairPin>(ztile, lz, 16 * kk, 0);
+                const bf16x8 zf = fetch_nat_o<64, kPairPin>(ztile, lz, 16 * kk, 1);
+#pragma unroll
+                for (int j = 0; j < kBlocks; ++j) {
+                    dvacc[j] = mfma(af, fetch_nat_o<D, kPairPin>(dotile, lo, 16 * kk, kBlocks * r + j), dvacc[j]);
+                    dkacc[j] = mfma(zf, fetch_nat_o<D, kPairPin>(qtile, lo, 16 * kk, kBlocks * r + j), dkacc[j]);
+                }
+            }
+        }
+        wait_global_memory();                  // the next tiles and carries have landed
+        __syncthreads();                       // ... and everybody is through with this step's tiles
+    }
+
+    // ---- rows kb0.. of dK (scaled) and dV: each wave stages its column blocks in the pair's tile, the pair
+    // stores whole rows as coalesced 16-byte chunks
+#pragma unroll
+    for (int which = 0; which < 2; ++which) {
+        const TensorArg& out = which == 0 ? p.dk : p.dv;
+        const int64_t ob = (int64_t)job.seq * out.sb + (int64_t)head * out.sh + (int64_t)job.tok0 * out.st;
+#pragma unroll
+        for (int j = 0; j < kBlocks; ++j)
+            stage_acc_tile<D>(ztile, 0, 32 * (kBlocks * r + j), which == 0 ? dkacc[j] : dvacc[j], which == 0 ? p.scale : 1.0f, lane);
+        __syncthreads();
+        for (int c = lane + 64 * r; c < 32 * D / 8; c += 128) {
+            const int row = c / (D / 8), cc = c % (D / 8);
+            if (kb0 + row < job.len)
+                *(u32x4*)(out.ptr + 2 * (ob + (int64_t)(kb0 + row) * out.st + cc * 8)) = *(const u32x4*)(ztile + row * (D * 2) + cc * 16);
+        }
+        __syncthreads();
+    }
+}
+
 }  // namespace sba
 
 bool sba_mfma_bwd_available() { return true; }
@@ -1368,7 +1548,7 @@ static int sba_cu_count() {
 // both on the same inputs).
 static bool own_keys_kernel(bool by_size) {
     const char* e = getenv("SBA_DKV_KERNEL");
-    if (e && !strcmp(e, "own")) return true;
+    if (e && (!strcmp(e, "own") || !strcmp(e, "pair"))) return true;
     if (e && !strcmp(e, "other")) return false;
     return by_size;
 }
@@ -1412,7 +1592,11 @@ int sba_launch_mfma_bwd(const sba::KParams& kp_in, int phases, hipStream_t s) {
         }
     } else {
         if (p1) hipLaunchKernelGGL((mfma_bwd_dq_kernel<128>), grid, dim3(kThreads), 0, s, kp);
-        if (p2 && own) hipLaunchKernelGGL((mfma_bwd_dkv_own_kernel<128>), grid, dim3(kThreads), 0, s, kp);
+        // key owners at head_dim 128: two waves per 32 keys (6-9 % faster than one wave per 32 keys,
+        // which SBA_DKV_KERNEL=own still selects)
+        const bool pair = !(which && !strcmp(which, "own"));
+        if (p2 && own && pair) hipLaunchKernelGGL((mfma_bwd_dkv_pair_kernel<128>), grid, dim3(2 * kThreads), 0, s, kp);
+        else if (p2 && own) hipLaunchKernelGGL((mfma_bwd_dkv_own_kernel<128>), grid, dim3(kThreads), 0, s, kp);
         else if (p2) hipLaunchKernelGGL((mfma_bwd_dkv_kernel<128>), dim3(2 * grid.x), dim3(kThreads), 0, s, kp);
     }
     return hipGetLastError() == hipSuccess ? SBA_OK : SBA_ERR_LAUNCH;

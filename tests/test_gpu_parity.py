@@ -504,7 +504,7 @@ def test_config4_size_invariants():
 
 
 @pytest.mark.parametrize("dkv_kernel,D", [("", 64), ("own", 64), ("other", 64), ("stream8", 64), ("plain", 64),
-                                          ("own", 128), ("other", 128)])
+                                          ("own", 128), ("other", 128), ("pair", 128)])
 def test_randomized_packed_batches_mfma_vs_generic_backward(dkv_kernel, D, monkeypatch):
     # Seeded random packed batches (document counts, lengths around the 64/128 block edges,
     # head counts that are and are not multiples of 8, both masks): the MFMA kernels against the
