@@ -1425,9 +1425,43 @@ __global__ __launch_bounds__(2 * kThreads, 2) void mfma_bwd_dkv_pair_kernel(KPar
     wait_global_memory();
     __syncthreads();
 
-    for (int step = 0, buf = 0; step < n_steps; ++step, buf ^= 1) {
-        const char* qtile = lds + buf * 2 * kQTile;
-        const char* dotile = qtile + kQTile;
+    // Every LDS address of the loop is "a register that is fixed for the whole sweep + a constant": the sums of
+    // LDS base, lane offset and this wave's share (query tile r, column blocks 2r.., the pair's weight tile) are
+    // made once, and the loop runs in two copies, one per tile buffer, so that buffer and row offsets are compile-time
+    // numbers that go into the offset fields of the fetches.  (With the tile address in a scalar register each
+    // fetch costs one or two vector adds with a scalar operand, 1.8 ns each: 40 of them per step.)
+    const uint32_t lds0 = (uint32_t)(uintptr_t)lds;
+    uint32_t row_at[D / 16], nat_at[2][kBlocks], z_at[2][2];
+#pragma unroll
+    for (int ks = 0; ks < D / 16; ++ks) row_at[ks] = lds_lane_base(lds + r * 32 * D * 2, lo.rows[ks]);
+    {
+        const int hh = lane >> 5, G1 = (lane >> 4) & 1, sl = lane & 15;
+#pragma unroll
+        for (int a2 = 0; a2 < 2; ++a2) {
+#pragma unroll
+            for (int j = 0; j < kBlocks; ++j) {
+                const int chunk = 4 * (kBlocks * r + j) + 2 * G1 + ((sl & 3) >> 1);
+                nat_at[a2][j] = lds_lane_base(lds, tile_offset<D>(8 * hh + 4 * a2 + (sl >> 2), chunk) + ((sl & 1) << 3));
+            }
+#pragma unroll
+            for (int cb = 0; cb < 2; ++cb) z_at[a2][cb] = lds_lane_base(ztile, lz.nat[a2][cb]);
+        }
+    }
+    (void)lds0;
+    auto rows_at = [&](uint32_t base, int imm) __attribute__((always_inline)) {
+        return *(const __attribute__((address_space(3))) bf16x8*)((__attribute__((address_space(3))) char*)(uintptr_t)base + imm);
+    };
+    auto nat_pair = [&](const uint32_t (&at)[2][2], int col, int imm) __attribute__((always_inline)) {
+        union { s16x4 v[2]; bf16x8 b; } u;
+        u.v[0] = lds_read_tr_at(at[0][col], imm);
+        u.v[1] = lds_read_tr_at(at[1][col], imm);
+        return u.b;
+    };
+
+    auto do_step = [&](int step, auto buf_c) __attribute__((always_inline)) {
+        constexpr int buf = decltype(buf_c)::value;
+        constexpr int kQ = buf * 2 * kQTile;             // byte offsets of this step's Q and dO tiles
+        constexpr int kDO = kQ + kQTile;
         const int q0 = q_begin + step * kStep;
         const float Rin = Rn, Gin = Gn;
         if (step + 1 < n_steps) {     // next tiles, straight into the other buffer (nobody reads it since the last barrier)
@@ -1452,7 +1486,7 @@ __global__ __launch_bounds__(2 * kThreads, 2) void mfma_bwd_dkv_pair_kernel(KPar
                 {
                     bf16x8 bq[D / 16];
 #pragma unroll
-                    for (int ks = 0; ks < D / 16; ++ks) bq[ks] = fetch_rows_p<D>(qtile, lo, r, ks);
+                    for (int ks = 0; ks < D / 16; ++ks) bq[ks] = rows_at(row_at[ks], kQ);
                     f32x16 acc = {0};
 #pragma unroll
                     for (int ks = 0; ks < D / 16; ++ks) acc = mfma(kfr[ks], bq[ks], acc);
@@ -1467,7 +1501,7 @@ __global__ __launch_bounds__(2 * kThreads, 2) void mfma_bwd_dkv_pair_kernel(KPar
                 // dP = dO V^T between the segments of the chain
                 bf16x8 bd[D / 16];
 #pragma unroll
-                for (int ks = 0; ks < D / 16; ++ks) bd[ks] = fetch_rows_p<D>(dotile, lo, r, ks);
+                for (int ks = 0; ks < D / 16; ++ks) bd[ks] = rows_at(row_at[ks], kDO);
                 f32x16 dacc;
                 own_tile_weights(x, beta, Rt, lane, [&](int seg) {
 #pragma unroll
@@ -1495,17 +1529,21 @@ __global__ __launch_bounds__(2 * kThreads, 2) void mfma_bwd_dkv_pair_kernel(KPar
             // dV += A^T dO, dK += dZ^T Q over the step's 64 queries, this wave's column blocks
 #pragma unroll
             for (int kk = 0; kk < 4; ++kk) {
-                const bf16x8 af = fetch_nat_o<64, kPairPin>(ztile, lz, 16 * kk, 0);
-                const bf16x8 zf = fetch_nat_o<64, kPairPin>(ztile, lz, 16 * kk, 1);
+                const bf16x8 af = nat_pair(z_at, 0, 16 * kk * 64 * 2);
+                const bf16x8 zf = nat_pair(z_at, 1, 16 * kk * 64 * 2);
 #pragma unroll
                 for (int j = 0; j < kBlocks; ++j) {
-                    dvacc[j] = mfma(af, fetch_nat_o<D, kPairPin>(dotile, lo, 16 * kk, kBlocks * r + j), dvacc[j]);
-                    dkacc[j] = mfma(zf, fetch_nat_o<D, kPairPin>(qtile, lo, 16 * kk, kBlocks * r + j), dkacc[j]);
+                    dvacc[j] = mfma(af, nat_pair(nat_at, j, kDO + 16 * kk * D * 2), dvacc[j]);
+                    dkacc[j] = mfma(zf, nat_pair(nat_at, j, kQ + 16 * kk * D * 2), dkacc[j]);
                 }
             }
         }
         wait_global_memory();                  // the next tiles and carries have landed
         __syncthreads();                       // ... and everybody is through with this step's tiles
+    };
+    for (int step = 0; step < n_steps; step += 2) {
+        do_step(step, std::integral_constant<int, 0>{});
+        if (step + 1 < n_steps) do_step(step + 1, std::integral_constant<int, 1>{});
     }
 
     // ---- rows kb0.. of dK (scaled) and dV: each wave stages its column blocks in the pair's tile, the pair
