@@ -91,7 +91,28 @@ template <int D> struct LaneOffsets {
                 nat[a][b] = tile_offset<D>(8 * h + 4 * a + (s >> 2), chunk) + ((s & 1) << 3);
             }
     }
+    // Turns the offsets into absolute LDS addresses (each pinned in its register), for kernels that name their
+    // tiles by TileAt: every fetch is then "one of these registers + an immediate", with no address arithmetic
+    // in the loop.
+    __device__ inline void rebase(const char* lds) {
+        auto fix = [&](int& v) {
+            uint32_t b = (uint32_t)(uintptr_t)lds + (uint32_t)v;
+            asm("" : "+v"(b));
+            v = (int)b;
+        };
+#pragma unroll
+        for (int ks = 0; ks < D / 16; ++ks) fix(rows[ks]);
+#pragma unroll
+        for (int a = 0; a < 2; ++a)
+#pragma unroll
+            for (int b = 0; b < D / 32; ++b) { fix(cols[a][b]); fix(nat[a][b]); }
+    }
 };
+
+// A tile at a COMPILE-TIME byte offset from the start of the kernel's LDS array (loops that run in one copy per
+// tile buffer), used with rebased LaneOffsets.  With the tile's address in a scalar register instead, each fetch -
+// or, with pinned sums, each offset register per step - costs a vector add with a scalar operand (1.8 ns).
+struct TileAt { int off; };
 
 // Wait for every outstanding global load and store of this wave.  The compiler's wait-count
 // bookkeeping merges control-flow paths pessimistically: a register loaded before a loop, or
@@ -133,6 +154,9 @@ __device__ inline s16x4 lds_read_tr_at(uint32_t base, int imm) {
 template <int D> __device__ inline bf16x8 fetch_rows_o(const char* tile, const LaneOffsets<D>& o, int t, int ks) {
     return *(const bf16x8*)(tile + o.rows[ks] + t * 32 * D * 2);
 }
+template <int D> __device__ inline bf16x8 fetch_rows_o(TileAt tile, const LaneOffsets<D>& o, int t, int ks) {
+    return *(const __attribute__((address_space(3))) bf16x8*)((__attribute__((address_space(3))) char*)(uintptr_t)(uint32_t)o.rows[ks] + (tile.off + t * 32 * D * 2));
+}
 // kPinBase: the sum `tile + lane offset` is pinned in a register (lds_lane_base) and the fetch's constant goes into
 // the offset field; one vector add per offset register and step instead of one per fetch, at the price of registers
 // for the pinned sums of both tile buffers (measured: forward -7 % on small grids and -3 % at head_dim 128, dQ -2 %
@@ -150,6 +174,21 @@ __device__ inline bf16x8 fetch_cols_o(const char* tile, const LaneOffsets<D>& o,
     }
     return u.b;
 }
+template <int D, bool kPinBase = true>
+__device__ inline bf16x8 fetch_cols_o(TileAt tile, const LaneOffsets<D>& o, int db, int c) {
+    union { s16x4 v[2]; bf16x8 b; } u;
+    const int add = tile.off + (32 * (c >> 1) + 16 * (c & 1)) * D * 2;
+    u.v[0] = lds_read_tr_at((uint32_t)o.cols[0][db], add);
+    u.v[1] = lds_read_tr_at((uint32_t)o.cols[1][db], add);
+    return u.b;
+}
+template <int D, bool kPinBase = false>
+__device__ inline bf16x8 fetch_nat_o(TileAt tile, const LaneOffsets<D>& o, int row0, int cb) {
+    union { s16x4 v[2]; bf16x8 b; } u;
+    u.v[0] = lds_read_tr_at((uint32_t)o.nat[0][cb], tile.off + row0 * D * 2);
+    u.v[1] = lds_read_tr_at((uint32_t)o.nat[1][cb], tile.off + row0 * D * 2);
+    return u.b;
+}
 template <int D, bool kPinBase = false>
 __device__ inline bf16x8 fetch_nat_o(const char* tile, const LaneOffsets<D>& o, int row0, int cb) {
     union { s16x4 v[2]; bf16x8 b; } u;
@@ -163,6 +202,9 @@ __device__ inline bf16x8 fetch_nat_o(const char* tile, const LaneOffsets<D>& o, 
     return u.b;
 }
 // fetch_rows_o with the pinned base (see fetch_cols_o): row 32*t + lane%32 of a tile in natural or MFMA order
+template <int D> __device__ inline bf16x8 fetch_rows_p(TileAt tile, const LaneOffsets<D>& o, int t, int ks) {
+    return fetch_rows_o<D>(tile, o, t, ks);
+}
 template <int D> __device__ inline bf16x8 fetch_rows_p(const char* tile, const LaneOffsets<D>& o, int t, int ks) {
     return *(const __attribute__((address_space(3))) bf16x8*)((__attribute__((address_space(3))) char*)(uintptr_t)lds_lane_base(tile, o.rows[ks]) + t * 32 * D * 2);
 }
@@ -359,8 +401,8 @@ __device__ inline f32x16 mfma(bf16x8 a, bf16x8 b, f32x16 c) {
 // S^T tile pair for one wave, raw MFMA accumulators (no vector-ALU instruction touches
 // them here, so the matrix cores run ahead of whatever vector work follows):
 // raw[t][r] = (K Q^T)[key_local = 32h + 16t + r][query n].
-template <int D, bool kBatch = (D == 128)>
-__device__ inline void score_raw_o(f32x16 (&raw)[2], const char* ktile, const LaneOffsets<D>& o,
+template <int D, bool kBatch = (D == 128), class Tile>
+__device__ inline void score_raw_o(f32x16 (&raw)[2], Tile ktile, const LaneOffsets<D>& o,
                                    const bf16x8 (&qf)[D / 16]) {
     // tile 1 first: the product chain starts at its keys (the right half of the lane's 32), and
     // can begin while the MFMAs of tile 0 are still in flight
@@ -387,8 +429,8 @@ __device__ inline void scale_scores(float (&x)[32], const f32x16 (&raw)[2], floa
         for (int r = 0; r < 16; ++r) x[16 * t + r] = raw[t][r] * scale2;
 }
 
-template <int D, bool kBatch = (D == 128)>
-__device__ inline void score_tiles_o(float (&x)[32], const char* ktile, const LaneOffsets<D>& o,
+template <int D, bool kBatch = (D == 128), class Tile>
+__device__ inline void score_tiles_o(float (&x)[32], Tile ktile, const LaneOffsets<D>& o,
                                      const bf16x8 (&qf)[D / 16], float scale2) {
     f32x16 raw[2];
     score_raw_o<D, kBatch>(raw, ktile, o, qf);
@@ -396,8 +438,8 @@ __device__ inline void score_tiles_o(float (&x)[32], const char* ktile, const La
 }
 
 // Score tiles from pre-scaled fragments: x[16*t + r] = raw accumulator, no vector work.
-template <int D, bool kBatch = (D == 128)>
-__device__ inline void score_tiles_ps(float (&x)[32], const char* ktile, const LaneOffsets<D>& o,
+template <int D, bool kBatch = (D == 128), class Tile>
+__device__ inline void score_tiles_ps(float (&x)[32], Tile ktile, const LaneOffsets<D>& o,
                                       const bf16x8 (&qf)[D / 16]) {
     f32x16 raw[2];
     score_raw_o<D, kBatch>(raw, ktile, o, qf);
@@ -558,9 +600,9 @@ __device__ inline void stick_weights_hooked(float (&x)[32], float (&beta)[32], f
 
 // stick_weights<true> with the dP MFMAs of the step (dp[16t + r] = (V dO^T)[key][query], see
 // dp_tiles_o) issued between the segments of the chain, their operands fetched one segment ahead.
-template <int D>
+template <int D, class Tile>
 __device__ inline void stick_weights_and_dp(float (&x)[32], float (&beta)[32], float (&dp)[32], float& R, int lane,
-                                            float* lane_carry, const char* vtile, const LaneOffsets<D>& o,
+                                            float* lane_carry, Tile vtile, const LaneOffsets<D>& o,
                                             const bf16x8 (&dof)[D / 16]) {
     constexpr int kPer = D / 64;               // MFMAs per segment: 2 tiles x D/16 slices over 8 segments
     f32x16 dacc[2];
@@ -626,8 +668,8 @@ template <int ROWD> __device__ inline bf16x8 fetch_row_nat(const char* tile, int
 // gradient is  -beta_ik * d_rem_i * rem_i  (the weights of a row and its remainder sum to one),
 // i.e. a constant d_rem_i * rem_i added to the running prefix of g -- which is how the prefix
 // tables carry it (see the dQ kernels).  `init` is what the accumulators start from (zero).
-template <int D>
-__device__ inline void dp_tiles_o(float (&dp)[32], const char* vtile, const LaneOffsets<D>& o,
+template <int D, class Tile>
+__device__ inline void dp_tiles_o(float (&dp)[32], Tile vtile, const LaneOffsets<D>& o,
                                   const bf16x8 (&dof)[D / 16], float init = 0.f) {
 #pragma unroll
     for (int t = 0; t < 2; ++t) {

@@ -36,6 +36,7 @@ __global__ __launch_bounds__(kThreads, 2) void mfma_bwd_dq_kernel(KParams p) {
     const int n = lane & 31, h = lane >> 5;
     LaneOffsets<D> lo;
     lo.init(lane);
+    lo.rebase(lds);                        // absolute addresses: the loop below runs in one copy per tile buffer
     const int head = blockIdx.x % p.n_heads;
     const Job job = decode_job(p, order_job(blockIdx.x / p.n_heads, p.n_jobs, false));
     const int strict = p.attend_current ? 0 : 1;
@@ -85,9 +86,10 @@ __global__ __launch_bounds__(kThreads, 2) void mfma_bwd_dq_kernel(KParams p) {
     bool mid_pending = false, g_pending = false;
     wait_global_memory();
     __syncthreads();
-    for (int step = 0, buf = 0; step < n_steps; ++step, buf ^= 1) {
-        const char* ktile = lds + buf * 2 * kTile;
-        const char* vtile = ktile + kTile;
+    auto do_step = [&](int step, auto buf_c) __attribute__((always_inline)) {
+        constexpr int buf = decltype(buf_c)::value;
+        constexpr TileAt ktile = {buf * 2 * kTile};
+        constexpr TileAt vtile = {buf * 2 * kTile + kTile};
         const bool more = step + 1 < n_steps;
         const int key0 = step * kKeyBlock;
         const bool skip = key0 + strict > q0w + 31;
@@ -167,6 +169,10 @@ __global__ __launch_bounds__(kThreads, 2) void mfma_bwd_dq_kernel(KParams p) {
         }
         wait_global_memory();                  // the next tiles have landed
         __syncthreads();
+    };
+    for (int step = 0; step < n_steps; step += 2) {
+        do_step(step, std::integral_constant<int, 0>{});
+        if (step + 1 < n_steps) do_step(step + 1, std::integral_constant<int, 1>{});
     }
     if (g_pending && row_ok && h == 0) p.gtab[tix0 + (n_steps - 1) * tstride] = Genter;
     if (mid_pending && row_ok && p.rmid) mid_table[tix0 + (n_steps - 1) * tstride] = mid;
