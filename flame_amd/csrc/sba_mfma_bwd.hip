@@ -1420,12 +1420,15 @@ __global__ __launch_bounds__(2 * kThreads, 2) void mfma_bwd_dkv_pair_kernel(KPar
     const float* rsrc = ((grp & 1) ? p.rtab : p.rmid) + tab_index(p, head, job, 0, kb64);
     const float* gsrc = ((grp & 1) ? p.gmid : p.gtab) + tab_index(p, head, job, 0, kb64);
     float Rn = 1.f, Gn = 0.f;
-    auto request_carries = [&](int q0) {
-        const int qi = min(q0 + 32 * r + n, job.len - 1);
-        const int qb = qi >> 7;
-        const int64_t ix = (int64_t)qb * (qb + 1) * kRowBlock + (qi & (kRowBlock - 1));
-        Rn = rsrc[ix];
-        Gn = gsrc[ix];
+    // A step's 64 queries lie inside one 128-row block: the table index is a uniform base plus the lane's
+    // row.  Rows past the end of the sequence are read too (the tables are allocated in whole row blocks)
+    // and not used.
+    const int my_row = 32 * r + n;
+    auto request_carries = [&](int q0) __attribute__((always_inline)) {
+        const int qb = q0 >> 7;
+        const int64_t ix = (int64_t)qb * (qb + 1) * kRowBlock + (q0 & (kRowBlock - 1));      // uniform
+        Rn = rsrc[ix + my_row];
+        Gn = gsrc[ix + my_row];
     };
     if (n_steps > 0) request_carries(q_begin);
     wait_global_memory();
@@ -1479,11 +1482,12 @@ __global__ __launch_bounds__(2 * kThreads, 2) void mfma_bwd_dkv_pair_kernel(KPar
         if (!skip) {
             const int qt0 = q0 + 32 * r;
             const int qi = qt0 + n;
-            float x[16], dp[16];
             if (kb0 + strict > qt0 + 31) {             // this wave's query tile sees none of the keys (the other one does)
+                const bf16x8 none = {0, 0, 0, 0, 0, 0, 0, 0};
 #pragma unroll
-                for (int idx = 0; idx < 16; ++idx) { x[idx] = 0.f; dp[idx] = 0.f; }
+                for (int c = 0; c < 4; ++c) *(bf16x8*)(ztile + tile_offset<64>(32 * r + n, 2 * c + h)) = none;
             } else {
+                float x[16], dp[16];
                 const int nvis = qi < job.len ? qi - strict - (kb0 + 16 * h) + 1 : 0;
                 const bool sees = qi < job.len && qi - strict - kb0 + 1 > 0;
                 const float Rt = sees ? Rin : 1.0f;      // table entries of invisible pairs are not written
@@ -1493,6 +1497,7 @@ __global__ __launch_bounds__(2 * kThreads, 2) void mfma_bwd_dkv_pair_kernel(KPar
                     bf16x8 bq[D / 16];
 #pragma unroll
                     for (int ks = 0; ks < D / 16; ++ks) bq[ks] = rows_at(row_at[ks], kQ);
+                    __builtin_amdgcn_sched_barrier(0);     // all operands requested before the first MFMA: two waves per SIMD hide no LDS round trip per MFMA
                     f32x16 acc = {0};
 #pragma unroll
                     for (int ks = 0; ks < D / 16; ++ks) acc = mfma(kfr[ks], bq[ks], acc);
@@ -1504,16 +1509,24 @@ __global__ __launch_bounds__(2 * kThreads, 2) void mfma_bwd_dkv_pair_kernel(KPar
                     for (int idx = 0; idx < 16; ++idx)
                         if (idx >= nvis) x[idx] = -INFINITY;
                 }
-                // dP = dO V^T between the segments of the chain
-                bf16x8 bd[D / 16];
+                // dP = dO V^T between the segments of the chain, its operands fetched one segment ahead
+                constexpr int kPer = D / 64;
+                bf16x8 nx[kPer];
 #pragma unroll
-                for (int ks = 0; ks < D / 16; ++ks) bd[ks] = rows_at(row_at[ks], kDO);
+                for (int i = 0; i < kPer; ++i) nx[i] = rows_at(row_at[i], kDO);
                 f32x16 dacc;
                 own_tile_weights(x, beta, Rt, lane, [&](int seg) {
+                    bf16x8 cur[kPer];
 #pragma unroll
-                    for (int i = 0; i < D / 64; ++i) {
-                        const int ks = (D / 64) * seg + i;
-                        dacc = mfma(vfr[ks], bd[ks], ks == 0 ? f32x16{0} : dacc);
+                    for (int i = 0; i < kPer; ++i) cur[i] = nx[i];
+                    if (seg < 3) {
+#pragma unroll
+                        for (int i = 0; i < kPer; ++i) nx[i] = rows_at(row_at[kPer * (seg + 1) + i], kDO);
+                    }
+#pragma unroll
+                    for (int i = 0; i < kPer; ++i) {
+                        const int ks = kPer * seg + i;
+                        dacc = mfma(vfr[ks], cur[i], ks == 0 ? f32x16{0} : dacc);
                     }
                 });
 #pragma unroll
@@ -1522,26 +1535,36 @@ __global__ __launch_bounds__(2 * kThreads, 2) void mfma_bwd_dkv_pair_kernel(KPar
                 *(bf16x8*)(ztile + tile_offset<64>(32 * r + n, 2 * h)) = pack8(&x[0]);
                 *(bf16x8*)(ztile + tile_offset<64>(32 * r + n, 2 * h + 1)) = pack8(&x[8]);
                 own_tile_grads(x, beta, dp, Gt, lane);
+                *(bf16x8*)(ztile + tile_offset<64>(32 * r + n, 4 + 2 * h)) = pack8(&dp[0]);
+                *(bf16x8*)(ztile + tile_offset<64>(32 * r + n, 4 + 2 * h + 1)) = pack8(&dp[8]);
             }
-            if (kb0 + strict > qt0 + 31) {
-                *(bf16x8*)(ztile + tile_offset<64>(32 * r + n, 2 * h)) = pack8(&x[0]);
-                *(bf16x8*)(ztile + tile_offset<64>(32 * r + n, 2 * h + 1)) = pack8(&x[8]);
-            }
-            *(bf16x8*)(ztile + tile_offset<64>(32 * r + n, 4 + 2 * h)) = pack8(&dp[0]);
-            *(bf16x8*)(ztile + tile_offset<64>(32 * r + n, 4 + 2 * h + 1)) = pack8(&dp[8]);
         }
         __syncthreads();                       // the pair's weights are complete
         if (!skip) {
-            // dV += A^T dO, dK += dZ^T Q over the step's 64 queries, this wave's column blocks
-#pragma unroll
-            for (int kk = 0; kk < 4; ++kk) {
-                const bf16x8 af = nat_pair(z_at, 0, 16 * kk * 64 * 2);
-                const bf16x8 zf = nat_pair(z_at, 1, 16 * kk * 64 * 2);
+            // dV += A^T dO, dK += dZ^T Q over the step's 64 queries, this wave's column blocks.  The operands of
+            // 16 queries are requested while the MFMAs of the 16 before them run (left to itself the compiler
+            // requests them right before their MFMA, which then waits for the LDS round trip: 16 per step).
+            bf16x8 w[2][2], o[2][2 * kBlocks];
+            auto fetch_kk = [&](int kk, bf16x8 (&ww)[2], bf16x8 (&oo)[2 * kBlocks]) __attribute__((always_inline)) {
+                ww[0] = nat_pair(z_at, 0, 16 * kk * 64 * 2);
+                ww[1] = nat_pair(z_at, 1, 16 * kk * 64 * 2);
 #pragma unroll
                 for (int j = 0; j < kBlocks; ++j) {
-                    dvacc[j] = mfma(af, nat_pair(nat_at, j, kDO + 16 * kk * D * 2), dvacc[j]);
-                    dkacc[j] = mfma(zf, nat_pair(nat_at, j, kQ + 16 * kk * D * 2), dkacc[j]);
+                    oo[2 * j] = nat_pair(nat_at, j, kDO + 16 * kk * D * 2);
+                    oo[2 * j + 1] = nat_pair(nat_at, j, kQ + 16 * kk * D * 2);
                 }
+            };
+            fetch_kk(0, w[0], o[0]);
+#pragma unroll
+            for (int kk = 0; kk < 4; ++kk) {
+                if (kk < 3) fetch_kk(kk + 1, w[(kk + 1) & 1], o[(kk + 1) & 1]);
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int j = 0; j < kBlocks; ++j) {
+                    dvacc[j] = mfma(w[kk & 1][0], o[kk & 1][2 * j], dvacc[j]);
+                    dkacc[j] = mfma(w[kk & 1][1], o[kk & 1][2 * j + 1], dkacc[j]);
+                }
+                __builtin_amdgcn_sched_barrier(0);
             }
         }
         wait_global_memory();                  // the next tiles and carries have landed
