@@ -24,13 +24,13 @@ KERNEL_TIMING_SAMPLES = 5      # steps of the timed region whose kernels are tim
 # runs summarised under profiles/ (sba_cfg{2,3,4}_hbm_traffic.txt, sba_cfg{2,3,4}_shader_counters.txt) and
 # are reported with that source next to what this run measures itself.
 # HBM bytes per launch (FETCH_SIZE + WRITE_SIZE, scaled by a copy kernel of known size):
-PROFILED_HBM_BYTES = {("cfg2", "fwd"): 51742194, ("cfg2", "bwd_dq"): 83649482, ("cfg2", "bwd_dkv"): 86102698,
-                      ("cfg3", "fwd"): 889818753, ("cfg3", "bwd_dq"): 980241054, ("cfg3", "bwd_dkv"): 1122045651,
-                      ("cfg4", "fwd"): 642239628, ("cfg4", "bwd_dq"): 1398968770, ("cfg4", "bwd_dkv"): 1401995278}
+PROFILED_HBM_BYTES = {("cfg2", "fwd"): 51742121, ("cfg2", "bwd_dq"): 83655099, ("cfg2", "bwd_dkv"): 86107599,
+                      ("cfg3", "fwd"): 888849577, ("cfg3", "bwd_dq"): 978901607, ("cfg3", "bwd_dkv"): 1121756781,
+                      ("cfg4", "fwd"): 643851047, ("cfg4", "bwd_dq"): 1733337426, ("cfg4", "bwd_dkv"): 1399483715}
 # wave instructions per launch: (vector incl. transcendental, transcendental, MFMA)
-PROFILED_INSTRUCTIONS = {("cfg2", "fwd"): (15299136, 2212864, 1064960), ("cfg2", "bwd_dq"): (29313025, 4268032, 1597440), ("cfg2", "bwd_dkv"): (34685467, 4268032, 2146304),
-                   ("cfg3", "fwd"): (124070464, 18619488, 9010688), ("cfg3", "bwd_dq"): (242937969, 36077696, 13516032), ("cfg3", "bwd_dkv"): (286992416, 35163264, 17564160),
-                   ("cfg4", "fwd"): (226918400, 34754560, 33685504), ("cfg4", "bwd_dq"): (466137089, 67387392, 50528256), ("cfg4", "bwd_dkv"): (623136768, 67387392, 67371008)}
+PROFILED_INSTRUCTIONS = {("cfg2", "fwd"): (15299136, 2212864, 1064960), ("cfg2", "bwd_dq"): (29317121, 4268032, 1597440), ("cfg2", "bwd_dkv"): (34685385, 4268032, 2146304),
+                   ("cfg3", "fwd"): (124070464, 18619488, 9010688), ("cfg3", "bwd_dq"): (235383089, 36077696, 13516032), ("cfg3", "bwd_dkv"): (286919360, 35163264, 17564160),
+                   ("cfg4", "fwd"): (226918400, 34754560, 33685504), ("cfg4", "bwd_dq"): (445767681, 67387392, 50528256), ("cfg4", "bwd_dkv"): (514064384, 67272704, 67305472)}
 # issue time of one SIMD per instruction, ns, four waves per SIMD (profiles/gfx950_issue_rates.txt): plain vector,
 # transcendental issued while MFMAs are in flight, MFMA 32x32x16 bf16.  MFMAs and plain vector instructions do not
 # overlap on gfx950, so their times add up.

@@ -250,7 +250,7 @@ __global__ __launch_bounds__(2 * kThreads, 2) void mfma_bwd_dq2_kernel(KParams p
     char* my_tiles = lds + grp * 2 * kTile;          // + buf * 4 * kTile
 
     // each group copies its own tiles (256 threads per tile pair)
-    TileDma<D> kc, vc;
+    TileDma<D, false, false> kc, vc;
     kc.init(lane, qs, p.k, kbase);
     vc.init(lane, qs, p.v, vbase);
     if (grp < n_steps) {
