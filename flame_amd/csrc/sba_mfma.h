@@ -294,6 +294,15 @@ template <int D, bool kNatural = false, bool kScalarBase = true> struct TileDma 
         lane = lane_; w4 = w4_;
         origin = t.ptr + 2 * base;
         st = (int)t.st;
+        // Scalar registers of their own: left as parts of the 16-register tuple that the kernel arguments were
+        // loaded into, they keep the whole tuple alive, and a spilled tuple comes back sixteen lane reads at a
+        // time in every iteration.
+        int st_own;
+        const char* origin_own;
+        asm volatile("s_mov_b32 %0, %1" : "=s"(st_own) : "s"(st));
+        asm volatile("s_mov_b64 %0, %1" : "=s"(origin_own) : "s"(origin));
+        st = st_own;
+        origin = origin_own;
 #pragma unroll
         for (int i = 0; i < kPerWave; ++i) {
             int kl, c;
