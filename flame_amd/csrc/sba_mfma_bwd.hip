@@ -12,10 +12,11 @@
 //           contributes to dz (sum_j a_ij + rem_i = 1), so pass 2 never reads d_rem.
 //   pass 2  (key owner): the owner of a block of keys sweeps the query blocks at or below the
 //           diagonal, recomputes weights and dz of its tiles from the tables, transposes them
-//           through LDS and accumulates dK = dZ^T Q and dV = P^T dO in registers.  Three
+//           through LDS and accumulates dK = dZ^T Q and dV = P^T dO in registers.  Four
 //           kernels, chosen by grid size and head_dim: every wave owning 32 keys outright
-//           (large grids), a resident producer/consumer stream over 64-key items (d = 64,
-//           small grids), one workgroup per 64-key block (d = 128, small grids).
+//           (d = 64, large grids), two waves sharing 32 keys (d = 128, large grids), a resident
+//           producer/consumer stream over 64-key items (d = 64, small grids), one workgroup
+//           per 64-key block (d = 128, small grids).
 //
 // Every element of the score matrix is therefore evaluated twice in the backward (once per
 // pass); in exchange nothing is reduced through memory.
