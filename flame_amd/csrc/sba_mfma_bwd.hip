@@ -728,16 +728,22 @@ __global__ __launch_bounds__((NP + 4) * 64, NP == 4 ? 2 : 3) void mfma_bwd_dkv_s
                     for (int r = 0; r < 16; ++r) dp[r] = dacc[r];
                 }
                 if (x_now) __syncthreads();    // X
+                // (the two cases store separately: one store sequence fed from either case costs the common one a
+                // register copy per value)
                 if (!skip) {
                     own_tile_grads(x, beta, dp, Gt, lane);
+#pragma unroll
+                    for (int c = 0; c < 2; ++c) {
+                        *(bf16x8*)(zp + tile_offset<64>(32 * w4 + n, 4 * kh + 2 * h + c)) = pack8(&x[8 * c]);
+                        *(bf16x8*)(zd + tile_offset<64>(32 * w4 + n, 4 * kh + 2 * h + c)) = pack8(&dp[8 * c]);
+                    }
                 } else {
+                    const bf16x8 none = {0, 0, 0, 0, 0, 0, 0, 0};
 #pragma unroll
-                    for (int idx = 0; idx < 16; ++idx) { x[idx] = 0.f; dp[idx] = 0.f; }
-                }
-#pragma unroll
-                for (int c = 0; c < 2; ++c) {
-                    *(bf16x8*)(zp + tile_offset<64>(32 * w4 + n, 4 * kh + 2 * h + c)) = pack8(&x[8 * c]);
-                    *(bf16x8*)(zd + tile_offset<64>(32 * w4 + n, 4 * kh + 2 * h + c)) = pack8(&dp[8 * c]);
+                    for (int c = 0; c < 2; ++c) {
+                        *(bf16x8*)(zp + tile_offset<64>(32 * w4 + n, 4 * kh + 2 * h + c)) = none;
+                        *(bf16x8*)(zd + tile_offset<64>(32 * w4 + n, 4 * kh + 2 * h + c)) = none;
+                    }
                 }
                 __syncthreads();               // A
             }
@@ -824,16 +830,22 @@ __global__ __launch_bounds__((NP + 4) * 64, NP == 4 ? 2 : 3) void mfma_bwd_dkv_s
                         for (int r = 0; r < 16; ++r) dp[16 * t + r] = dacc[t][r];
                 }
                 if (x_now) __syncthreads();    // X
+                // (the two cases store separately: one store sequence fed from either case costs the common one a
+                // register copy per value)
                 if (!skip) {
                     logit_grads_from<32>(x, beta, dp, Gc);
+#pragma unroll
+                    for (int c = 0; c < 4; ++c) {
+                        *(bf16x8*)(zp + tile_offset<64>(32 * w4 + n, 4 * h + c)) = pack8(&x[8 * c]);
+                        *(bf16x8*)(zd + tile_offset<64>(32 * w4 + n, 4 * h + c)) = pack8(&dp[8 * c]);
+                    }
                 } else {
+                    const bf16x8 none = {0, 0, 0, 0, 0, 0, 0, 0};
 #pragma unroll
-                    for (int idx = 0; idx < 32; ++idx) { x[idx] = 0.f; dp[idx] = 0.f; }
-                }
-#pragma unroll
-                for (int c = 0; c < 4; ++c) {
-                    *(bf16x8*)(zp + tile_offset<64>(32 * w4 + n, 4 * h + c)) = pack8(&x[8 * c]);
-                    *(bf16x8*)(zd + tile_offset<64>(32 * w4 + n, 4 * h + c)) = pack8(&dp[8 * c]);
+                    for (int c = 0; c < 4; ++c) {
+                        *(bf16x8*)(zp + tile_offset<64>(32 * w4 + n, 4 * h + c)) = none;
+                        *(bf16x8*)(zd + tile_offset<64>(32 * w4 + n, 4 * h + c)) = none;
+                    }
                 }
                 __syncthreads();               // A
             }
