@@ -201,13 +201,18 @@ def packed_columns_bound(total_tokens: int, n_docs: int, max_len: int) -> int:
     return (n_max + 1) * (total_tokens // 128 + n_docs)
 
 
-def workspace_upper_bound(n_heads: int, columns: int) -> int:
-    """One carry table (sba_workspace_bytes)."""
+def table_bytes(n_heads: int, columns: int) -> int:
+    """One carry table."""
     return (n_heads * columns * 128 * 4 + 255) & ~255
+
+
+def workspace_upper_bound(n_heads: int, columns: int) -> int:
+    """What the forward hands to the backward (sba_workspace_bytes): two carry tables in bf16, one in fp32."""
+    return 2 * table_bytes(n_heads, columns)
 
 
 def bwd_scratch_upper_bound(n_heads: int, columns: int, tab_tokens: int, head_dim: int) -> int:
     """Four tables (the recompute mode's count) or the generic path's fp32 dk|dv accumulators."""
     dp = 32 if head_dim <= 32 else (64 if head_dim <= 64 else 128)
     acc = (2 * tab_tokens * n_heads * dp * 4 + 255) & ~255
-    return max(4 * workspace_upper_bound(n_heads, columns) + 256, acc)      # + the backward's error word
+    return max(4 * table_bytes(n_heads, columns) + 256, acc)      # + the backward's error word

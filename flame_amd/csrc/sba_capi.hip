@@ -64,6 +64,12 @@ size_t generic_acc_bytes(const SbaParams* p) {
 
 constexpr size_t kErrorWordBytes = 256;     // tail of the MFMA backward's scratch: the error word
 
+// Carry tables of the matrix-core path, four in all.  bf16: the forward writes two - the product of (1 - beta)
+// entering the right 32 keys of every 64-key step (`rtab`) and the one entering its left 32 keys (`rmid`), so
+// that every lane of the backward starts its chain from its own carry - and the dQ pass the two prefix tables
+// (`gtab`, `gmid`).  fp32: the forward writes `rtab`, the dQ pass the other three.
+int forward_tables(const SbaParams* p) { return p->dtype == SBA_DTYPE_BF16 ? 2 : 1; }
+
 sba::TensorArg cvt(const SbaTensor& t) { return sba::TensorArg{(char*)t.ptr, t.stride_b, t.stride_h, t.stride_t}; }
 sba::VectorArg cvt(const SbaVector& t) { return sba::VectorArg{(char*)t.ptr, t.stride_b, t.stride_h}; }
 
@@ -109,14 +115,25 @@ KParams make_kparams(const SbaParams* p) {
     kp.rem = cvt(p->rem); kp.d_rem = cvt(p->d_rem);
     kp.tab_head_stride = table_columns(p) * sba::kRowBlock;
     kp.tab_tokens = tab_tokens(p);
-    if (p->workspace && use_mfma(p)) kp.rtab = (float*)p->workspace;
+    const size_t tb = table_bytes(p);
+    const bool two = forward_tables(p) == 2;
+    // Layout rule that the dQ kernels rely on: gmid - rtab == gtab - rmid (one table size both times), so that a
+    // lane finds its prefix entry at one uniform distance from its carry entry whichever half-wave it is in.
+    if (p->workspace && use_mfma(p)) {
+        if (two) { kp.rmid = (float*)p->workspace; kp.rtab = (float*)((char*)p->workspace + tb); }
+        else kp.rtab = (float*)p->workspace;
+    }
     char* bs = (char*)p->bwd_scratch;
     if (bs && use_mfma_bwd(p)) {
-        kp.gtab = (float*)bs;
-        kp.rmid = (float*)(bs + table_bytes(p));
-        kp.gmid = (float*)(bs + 2 * table_bytes(p));
-        if (!p->workspace) kp.rtab = (float*)(bs + 3 * table_bytes(p));   // recomputed by sba_bwd
-        kp.gave_up = (int*)(bs + (p->workspace ? 3 : 4) * table_bytes(p));
+        int slot = 0;
+        kp.gtab = (float*)(bs + tb * slot++);
+        if (!two) kp.rmid = (float*)(bs + tb * slot++);
+        kp.gmid = (float*)(bs + tb * slot++);
+        if (!p->workspace) {                       // the forward's tables, recomputed by sba_bwd
+            if (two) kp.rmid = (float*)(bs + tb * slot++);
+            kp.rtab = (float*)(bs + tb * slot++);
+        }
+        kp.gave_up = (int*)(bs + tb * slot);
     } else if (bs) {
         kp.dkv32 = (float*)bs;
     }
@@ -165,14 +182,14 @@ const char* sba_error_string(int code) {
 size_t sba_workspace_bytes(const SbaParams* p) {
     if (!p || p->n_heads <= 0 || p->seq_len <= 0 || p->head_dim <= 0 || p->head_dim > 128) return 0;
     if (p->cu_seqlens && p->table_cols <= 0) return 0;
-    return use_mfma(p) ? table_bytes(p) : 0;
+    return use_mfma(p) ? forward_tables(p) * table_bytes(p) : 0;
 }
 
 size_t sba_bwd_scratch_bytes(const SbaParams* p) {
     if (!p || p->n_heads <= 0 || p->seq_len <= 0 || p->head_dim <= 0 || p->head_dim > 128) return 0;
     if (p->cu_seqlens && p->table_cols <= 0 && use_mfma_bwd(p)) return 0;
-    // without a workspace the backward recomputes the forward's table first, into a fourth slot
-    return use_mfma_bwd(p) ? (p->workspace ? 3 : 4) * table_bytes(p) + kErrorWordBytes : generic_acc_bytes(p);
+    // without a workspace the backward recomputes the forward's tables first, into slots of its own
+    return use_mfma_bwd(p) ? (p->workspace ? 4 - forward_tables(p) : 4) * table_bytes(p) + kErrorWordBytes : generic_acc_bytes(p);
 }
 
 int sba_row_block(void) { return sba::kRowBlock; }

@@ -538,6 +538,32 @@ __device__ inline float product_chain_with(float (&x)[N], float (&beta)[kNeedBet
     }
     return clamp01(L);
 }
+// The chain from a given carry.  F = product of (1 - beta) over all keys right of THIS LANE's N keys (both
+// half-waves read their own from the forward's two carry tables).  Run on  W = (1/F) prod (1 + e),  the
+// reciprocals are the finished running products and their differences the finished weights: no scaling
+// pass over the weights afterwards.  F = 0 (a product that has left the fp32 range, or the zero carry
+// given to rows past the end of a sequence) makes W infinite, every reciprocal 0 or NaN and - through the
+// clamps - every weight and beta exactly 0, which is what such a row's values are to fp32 precision.
+// Returns the carry leaving the lane's keys on their left.
+template <bool kNeedBeta, int N, class Between>
+__device__ inline float carried_chain_with(float (&x)[N], float (&beta)[kNeedBeta ? N : 1], float F, Between&& between) {
+    float W = __builtin_amdgcn_rcpf(F), L = F;
+#pragma unroll
+    for (int idx = N - 1; idx >= 0; --idx) {
+        const float e = __builtin_amdgcn_exp2f(x[idx]);
+        const float Wn = __builtin_fmaf(W, e, W);
+        const float Ln = __builtin_amdgcn_rcpf(Wn);
+        x[idx] = clamp01(L - Ln);
+        if (kNeedBeta) beta[idx] = clamp01(__builtin_fmaf(-W, Ln, 1.0f));
+        W = Wn;
+        L = Ln;
+        if ((idx & 3) == 0) {
+            between((N - 1 - idx) >> 2);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    }
+    return clamp01(L);
+}
 template <int N> __device__ inline void scale_clamped(float (&x)[N], float f) {
 #pragma unroll
     for (int idx = 0; idx < N; ++idx) x[idx] = clamp01(x[idx] * f);
@@ -560,7 +586,7 @@ template <int N> __device__ inline void scale_clamped(float (&x)[N], float f) {
 constexpr float kFastChainLimit = 0x1p96f;
 
 template <bool kWeights>
-__device__ inline bool forward_weights_fast(float (&x)[32], bf16x8 (&pf)[4], float& R, int lane) {
+__device__ inline bool forward_weights_fast(float (&x)[32], bf16x8 (&pf)[4], float& R, int lane, float& lane_carry) {
     float W = 1.0f;
 #pragma unroll
     for (int idx = 31; idx >= 0; --idx) {
@@ -571,8 +597,9 @@ __device__ inline bool forward_weights_fast(float (&x)[32], bf16x8 (&pf)[4], flo
     const float Linv = __builtin_amdgcn_rcpf(W);
     float Llo, Lup;
     half_values(Linv, Llo, Lup);
+    lane_carry = (lane >= 32) ? R : R * Lup;                  // the carry entering this lane's 32 keys
     if (kWeights) {
-        float Lt = ((lane >= 32) ? R : R * Lup) * Linv;       // (carry entering this lane's keys) / W_0
+        float Lt = lane_carry * Linv;                         // ... over W_0
 #pragma unroll
         for (int c = 0; c < 4; ++c) {
             float a[8];
@@ -648,6 +675,40 @@ __device__ inline void stick_weights_and_dp(float (&x)[32], float (&beta)[32], f
     for (int t = 0; t < 2; ++t)
 #pragma unroll
         for (int r = 0; r < 16; ++r) dp[16 * t + r] = dacc[t][r];
+}
+
+// The same from this lane's own carry F (carried_chain_with): finished weights, beta and dP; returns the carry
+// leaving the lane's keys.
+template <int D, class Tile>
+__device__ inline float carried_weights_and_dp(float (&x)[32], float (&beta)[32], float (&dp)[32], float F,
+                                               Tile vtile, const LaneOffsets<D>& o, const bf16x8 (&dof)[D / 16]) {
+    constexpr int kPer = D / 64;
+    f32x16 dacc[2];
+    bf16x8 nx[kPer];
+#pragma unroll
+    for (int i = 0; i < kPer; ++i) nx[i] = fetch_rows_o<D>(vtile, o, i & 1, i >> 1);
+    const float Lend = carried_chain_with<true, 32>(x, beta, F, [&](int seg) {
+        bf16x8 cur[kPer];
+#pragma unroll
+        for (int i = 0; i < kPer; ++i) cur[i] = nx[i];
+        if (seg < 7) {
+#pragma unroll
+            for (int i = 0; i < kPer; ++i) {
+                const int m = kPer * (seg + 1) + i;
+                nx[i] = fetch_rows_o<D>(vtile, o, m & 1, m >> 1);
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < kPer; ++i) {
+            const int m = kPer * seg + i, t = m & 1, ks = m >> 1;
+            dacc[t] = mfma(cur[i], dof[ks], ks == 0 ? f32x16{0} : dacc[t]);
+        }
+    });
+#pragma unroll
+    for (int t = 0; t < 2; ++t)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) dp[16 * t + r] = dacc[t][r];
+    return Lend;
 }
 
 // The same in two parts, for kernels in which another wave-group handles the neighbouring
@@ -764,6 +825,41 @@ __device__ inline void logit_grads_from(const float (&a)[N], const float (&beta)
 // only the exchange after the chain supplies).  Returns the lane's product of (1 - beta) (clamped,
 // see product_chain) and in `gsum` the lane's sum of g'.  Part 2 walks left-to-right from the
 // prefix `G` entering the lane's keys:  t = F g',  G += t,  dz = t - beta G,  packed as it goes.
+// chain_beta_gprime from this lane's own carry F (see carried_chain_with): dp[idx] <- g = a * dP with the finished
+// weight, gsum their sum; returns the carry leaving the lane's keys.
+__device__ inline float carried_beta_g(float (&x)[32], float (&dp)[32], float F, float& gsum) {
+    float W = __builtin_amdgcn_rcpf(F), L = F, c = 0.f;
+#pragma unroll
+    for (int idx = 31; idx >= 0; --idx) {
+        const float e = __builtin_amdgcn_exp2f(x[idx]);
+        const float Wn = __builtin_fmaf(W, e, W);
+        const float Ln = __builtin_amdgcn_rcpf(Wn);
+        x[idx] = clamp01(__builtin_fmaf(-W, Ln, 1.0f));       // beta
+        dp[idx] = clamp01(L - Ln) * dp[idx];                  // g (the clamps map the NaN of an overflowed chain to 0)
+        c += dp[idx];
+        W = Wn;
+        L = Ln;
+    }
+    gsum = c;
+    return clamp01(L);
+}
+// dz from beta, g and the prefix G entering the lane's keys
+// (The running sum must stay a plain add: fused with the product that made g - which the compiler does across
+// function boundaries when allowed to - it would need the two factors of every g alive instead of g itself,
+// 32 registers more than this kernel has.)
+__device__ inline void walk_logit_grads_g(const float (&beta)[32], const float (&g)[32], float G, bf16x8 (&zf)[4]) {
+#pragma clang fp contract(off)
+#pragma unroll
+    for (int c = 0; c < 4; ++c) {
+        float dz[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            G += g[8 * c + i];
+            dz[i] = __builtin_fmaf(-beta[8 * c + i], G, g[8 * c + i]);
+        }
+        zf[c] = pack8(dz);
+    }
+}
 __device__ inline float chain_beta_gprime(float (&x)[32], float (&dp)[32], float& gsum) {
     float W = 1.0f, L = 1.0f, c = 0.f;
 #pragma unroll

@@ -79,12 +79,16 @@ __global__ __launch_bounds__(kThreads, 2) void mfma_bwd_dq_kernel(KParams p) {
     // carry-table traffic is kept off the critical path: the value of the NEXT step is loaded
     // while this one is computed, and this step's prefix is stored before the tile loads are
     // issued (vector memory operations retire in order)
+    // Per lane ONE cursor into the tables: the entry of (this query, the step at hand) in the table of the forward
+    // that holds the carry entering this LANE's 32 keys (right half-wave: rtab, left: rmid).  The prefix entering
+    // the same 32 keys goes to the same entry of gmid / gtab, which lies the same distance from the cursor for
+    // both half-waves (gmid - rtab == gtab - rmid: the library lays the tables out that way).
     constexpr int64_t tstride = kRowBlock;
-    const int64_t tix0 = tab_index(p, head, job, job.rb, 0) + 32 * wave + n;
-    float Rnext = (row_ok && n_steps > 0) ? p.rtab[tix0] : 1.0f;
-    float* mid_table = h == 0 ? p.rmid : p.gmid;
-    float mid = 0.f, Genter = 0.f;
-    bool mid_pending = false, g_pending = false;
+    const float* rcur = (h ? p.rtab : p.rmid) + tab_index(p, head, job, job.rb, 0) + 32 * wave + n;
+    const int64_t g_from_r = (const char*)p.gtab - (const char*)p.rmid;
+    float Rnext = (row_ok && n_steps > 0) ? *rcur : 1.0f;
+    float Gstore = 0.f;
+    bool g_pending = false;
     wait_global_memory();
     __syncthreads();
     auto do_step = [&](int step, auto buf_c) __attribute__((always_inline)) {
@@ -94,16 +98,13 @@ __global__ __launch_bounds__(kThreads, 2) void mfma_bwd_dq_kernel(KParams p) {
         const bool more = step + 1 < n_steps;
         const int key0 = step * kKeyBlock;
         const bool skip = key0 + strict > q0w + 31;
-        const int64_t tix = tix0 + step * tstride;
-        // the prefix that entered the previous step (the first block's is only known once that
-        // block's weights are: it starts at d_rem * rem, see below)
-        if (g_pending && row_ok && h == 0) p.gtab[tix - tstride] = Genter;
-        if (mid_pending && row_ok && p.rmid) mid_table[tix - tstride] = mid;
-        mid_pending = false;
+        // the prefixes that entered the previous step (the first block's are only known once that
+        // block's weights are: they start at d_rem * rem, see below)
+        if (g_pending && row_ok) *(float*)((char*)(rcur - tstride) + g_from_r) = Gstore;
         g_pending = false;
-        float R = Rnext;
+        const float F = Rnext;
         if (more) {
-            if (row_ok) Rnext = p.rtab[tix + tstride];
+            if (row_ok) Rnext = rcur[tstride];
             // next tiles, straight into the other buffer (free since the last barrier)
             kc.issue((step + 1) * kKeyBlock, job.len, lds + (buf ^ 1) * 2 * kTile);
             vc.issue((step + 1) * kKeyBlock, job.len, lds + (buf ^ 1) * 2 * kTile + kTile);
@@ -118,43 +119,44 @@ __global__ __launch_bounds__(kThreads, 2) void mfma_bwd_dq_kernel(KParams p) {
                 dp_tiles_o<D>(dp, vtile, lo, dof);
                 if (key0 + 63 + strict > q0w) mask_step(x, key0 + 32 * h, qi, strict);
                 float gsum;
-                const float L = chain_beta_gprime(x, dp, gsum);
-                float Llo, Lup;
-                half_values(L, Llo, Lup);
-                const float F = h ? R : R * Lup;         // the carry entering this lane's 32 keys
-                R = R * Llo * Lup;
-                if (step == 0) Gc = dr * R;              // the gradient of rem rides in the prefix, see below
-                Genter = Gc;
-                g_pending = true;
+                const float Lend = carried_beta_g(x, dp, F, gsum);
+                if (step == 0) {                         // the gradient of rem rides in the prefix, see below
+                    float Llo, Lup;
+                    half_values(Lend, Llo, Lup);
+                    Gc = dr * Llo;                       // what leaves the left half of the leftmost block is rem
+                }
                 float clo, cup;
-                half_values(F * gsum, clo, cup);
-                const float Glane = h ? Gc + clo : Gc;   // the prefix entering this lane's 32 keys
+                half_values(gsum, clo, cup);
+                const float Glane = h ? Gc + clo : Gc;   // the prefix entering this lane's 32 keys: block edge (left half-wave) or middle
                 Gc = Gc + clo + cup;
-                mid = h == 0 ? F : Glane;                // carries in the middle of the block, see below
-                mid_pending = true;
-                walk_logit_grads(x, dp, F, Glane, zf);
+                Gstore = Glane;
+                g_pending = true;
+                walk_logit_grads_g(x, dp, Glane, zf);
             } else {
                 float x[32], beta[32], dp[32];
-                float Rlane, Glane;
+                float Glane;
                 score_tiles_ps<D>(x, ktile, lo, qf);
                 if (key0 + 63 + strict > q0w) {
     mask_step(x, key0 + 32 * h, qi, strict);
                 }
                 // dP does not depend on the weights: its MFMAs go between the segments of the chain,
                 // where the chain's exp/rcp overlap them
-                stick_weights_and_dp<D>(x, beta, dp, R, lane, &Rlane, vtile, lo, dof);
+                const float Lend = carried_weights_and_dp<D>(x, beta, dp, F, vtile, lo, dof);
                 // The gradient of rem rides in the prefix: g is formed from the plain dP, and the term
                 // -beta_ik * d_rem_i * rem_i that d_rem adds to dz_ik is a constant d_rem_i * rem_i in
-                // the running prefix.  After the leftmost block R is the product over all keys, rem_i.
-                if (step == 0) Gc = dr * R;
-                Genter = Gc;
-                g_pending = true;
+                // the running prefix.  What leaves the left half of the leftmost block is the product over
+                // all keys, rem_i.
+                if (step == 0) {
+                    float Llo, Lup;
+                    half_values(Lend, Llo, Lup);
+                    Gc = dr * Llo;
+                }
                 logit_grads<false>(x, beta, dp, Gc, lane, &Glane);
-                // carries in the middle of the block, for the key-owner pass whose waves own 32 keys:
-                // the left half-wave holds the product entering the left 32 keys, the right half-wave
-                // the prefix entering the right 32 (stored at the top of the next iteration)
-                mid = h == 0 ? Rlane : Glane;
-                mid_pending = true;
+                // the prefix entering this lane's 32 keys - the block's edge for the left half-wave, its middle
+                // (for the key-owner pass whose waves own 32 keys) for the right one -, stored at the top of the
+                // next iteration
+                Gstore = Glane;
+                g_pending = true;
 #pragma unroll
                 for (int c = 0; c < 4; ++c) zf[c] = pack8(&dp[8 * c]);
             }
@@ -168,6 +170,7 @@ __global__ __launch_bounds__(kThreads, 2) void mfma_bwd_dq_kernel(KParams p) {
                 for (int db = 0; db < D / 32; ++db) dqacc[db] = mfma(kt[db], zf[c], dqacc[db]);
             }
         }
+        rcur += tstride;
         wait_global_memory();                  // the next tiles have landed
         __syncthreads();
     };
@@ -175,8 +178,7 @@ __global__ __launch_bounds__(kThreads, 2) void mfma_bwd_dq_kernel(KParams p) {
         do_step(step, std::integral_constant<int, 0>{});
         if (step + 1 < n_steps) do_step(step + 1, std::integral_constant<int, 1>{});
     }
-    if (g_pending && row_ok && h == 0) p.gtab[tix0 + (n_steps - 1) * tstride] = Genter;
-    if (mid_pending && row_ok && p.rmid) mid_table[tix0 + (n_steps - 1) * tstride] = mid;
+    if (g_pending && row_ok) *(float*)((char*)(rcur - tstride) + g_from_r) = Gstore;
 
     if (row_ok) {
         const int64_t ob = (int64_t)job.seq * p.dq.sb + (int64_t)head * p.dq.sh + (int64_t)(job.tok0 + qi) * p.dq.st;
@@ -261,11 +263,12 @@ __global__ __launch_bounds__(2 * kThreads, 2) void mfma_bwd_dq2_kernel(KParams p
 
     // the forward's carry for this group's NEXT step is loaded while this one is computed
     constexpr int64_t tstride = kRowBlock;
-    const int64_t tix0 = tab_index(p, head, job, job.rb, 0) + 32 * qs + n;
-    float Rnext = (row_ok && grp < n_steps) ? p.rtab[tix0 + grp * tstride] : 1.0f;
-    float* mid_table = h == 0 ? p.rmid : p.gmid;
-    float mid = 0.f;
-    bool mid_pending = false;
+    // this lane's cursor into the carry tables and the distance to its prefix entry, see the one-step kernel
+    const float* rcur = (h ? p.rtab : p.rmid) + tab_index(p, head, job, job.rb, 0) + 32 * qs + n + grp * tstride;
+    const int64_t g_from_r = (const char*)p.gtab - (const char*)p.rmid;
+    float Rnext = (row_ok && grp < n_steps) ? *rcur : 1.0f;
+    float Gstore = 0.f;
+    bool g_pending = false;
     wait_global_memory();
     __syncthreads();
     for (int it = 0, buf = 0; it < n_it; ++it, buf ^= 1) {
@@ -275,29 +278,29 @@ __global__ __launch_bounds__(2 * kThreads, 2) void mfma_bwd_dq2_kernel(KParams p
         const bool more = step + 2 < n_steps;
         const int key0 = step * kKeyBlock;
         const bool active = step < n_steps && !(key0 + strict > q0w + 31);
-        const int64_t tix = tix0 + step * tstride;
-        if (mid_pending && row_ok && p.rmid) mid_table[tix - 2 * tstride] = mid;
-        mid_pending = false;
-        const float R = Rnext;
+        if (g_pending && row_ok) *(float*)((char*)(rcur - 2 * tstride) + g_from_r) = Gstore;
+        g_pending = false;
+        const float F = Rnext;
         if (more) {
-            if (row_ok) Rnext = p.rtab[tix + 2 * tstride];
+            if (row_ok) Rnext = rcur[2 * tstride];
             // next tiles, straight into the other buffer (free since the last barrier)
             kc.issue((step + 2) * kKeyBlock, job.len, my_tiles + (buf ^ 1) * 4 * kTile);
             vc.issue((step + 2) * kKeyBlock, job.len, my_tiles + (buf ^ 1) * 4 * kTile + kTile);
         }
         float x[32], beta[32], dp[32];
-        float total = 0.f, start = 0.f, Rlane = 1.f;
+        float total = 0.f, start = 0.f;
         if (active) {
             score_tiles_ps<D, true>(x, ktile, lo, qf);
             if (key0 + 63 + strict > q0w) mask_step(x, key0 + 32 * h, qi, strict);
-            float Rc = R;
-            stick_weights_and_dp<D>(x, beta, dp, Rc, lane, &Rlane, vtile, lo, dof);
+            const float Lend = carried_weights_and_dp<D>(x, beta, dp, F, vtile, lo, dof);
             start = logit_grads_local(x, dp, total, lane);
             // the gradient of rem rides in the prefix as the constant d_rem * rem (see the one-step
             // kernel).  The leftmost block is group 0's first step: the constant joins its total
             // (which carries it to the other group and into Gc) and its own prefix
             if (step == 0) {
-                const float c0 = dr * Rc;
+                float Llo, Lup;
+                half_values(Lend, Llo, Lup);
+                const float c0 = dr * Llo;
                 total += c0;
                 start += c0;
             }
@@ -309,11 +312,9 @@ __global__ __launch_bounds__(2 * kThreads, 2) void mfma_bwd_dq2_kernel(KParams p
         const float Gmy = grp == 0 ? Gc : Gc + other;
         Gc = Gc + total + other;
         if (active) {
-            const float Glane = Gmy + start;       // the prefix entering this lane's 32 keys
-            if (row_ok && h == 0) p.gtab[tix] = Glane;
-            // carries in the middle of the block (see the one-step kernel)
-            mid = h == 0 ? Rlane : Glane;
-            mid_pending = true;
+            const float Glane = Gmy + start;       // the prefix entering this lane's 32 keys: block edge or middle (see the one-step kernel)
+            Gstore = Glane;
+            g_pending = true;
             logit_grads_apply(beta, dp, Glane);
             bf16x8 zf[4];
 #pragma unroll
@@ -324,11 +325,12 @@ __global__ __launch_bounds__(2 * kThreads, 2) void mfma_bwd_dq2_kernel(KParams p
                 for (int c = 0; c < 4; ++c)
                     dqacc[db] = mfma(fetch_cols_o<D>(ktile, lo, db, c), zf[c], dqacc[db]);
         }
+        rcur += 2 * tstride;
         wait_global_memory();                  // the next tiles have landed
         __syncthreads();
     }
 
-    if (mid_pending && row_ok && p.rmid) mid_table[tix0 + (2 * (n_it - 1) + grp) * tstride] = mid;
+    if (g_pending && row_ok) *(float*)((char*)(rcur - 2 * tstride) + g_from_r) = Gstore;
 
     // ---- dQ = dQ(group 0) + dQ(group 1): group 1 parks its accumulators in LDS
     float* park = (float*)lds;                              // [qs][db][r][lane]
@@ -819,11 +821,10 @@ __global__ __launch_bounds__((NP + 4) * 64, NP == 4 ? 2 : 3) void mfma_bwd_dkv_s
                     // segments of the chain, where the chain's exp/rcp overlap them
                     static_assert(D == 64, "one dP MFMA per chain segment");
                     f32x16 dacc[2];
-                    product_chain_with<true, 32>(x, beta, [&](int seg) {
+                    carried_chain_with<true, 32>(x, beta, R, [&](int seg) {      // finished weights: no scaling pass
                         const int t = seg & 1, ks = seg >> 1;
                         dacc[t] = mfma(vfr[t][ks], dof[ks], ks == 0 ? f32x16{0} : dacc[t]);
                     });
-                    scale_clamped<32>(x, R);
 #pragma unroll
                     for (int t = 0; t < 2; ++t)
 #pragma unroll
@@ -1650,9 +1651,6 @@ int sba_launch_mfma_bwd(const sba::KParams& kp_in, int phases, hipStream_t s) {
     // the stream with eight half-block producers (12 waves): measured within 1 % of the one with four
     // full-block producers (109.1 against 110.3 us at B=1 H=16 T=4096), which stays the default
     const bool stream8 = which && !strcmp(which, "stream8");
-    // the mid-block carries are read by the own-keys kernel and by the stream: otherwise the dQ pass
-    // skips them
-    if (!own && (kp.head_dim != 64 || plain)) kp.rmid = kp.gmid = nullptr;
     if (kp.head_dim == 64) {
         // small grids last as long as their longest sweep: take the variant that halves it
         if (p1 && grid.x <= sba_two_step_max_grid()) hipLaunchKernelGGL((mfma_bwd_dq2_kernel<64>), grid, dim3(2 * kThreads), 0, s, kp);

@@ -9,21 +9,23 @@ namespace sba {
 
 // One sweep step of one wave: 32 queries x 64 keys.  Scores (from the pre-scaled Q fragments),
 // mask on the diagonal, weights, O^T += V^T P^T.  kFast: the one-reciprocal chain; it may refuse
-// the step (returns false, nothing changed), see forward_weights_fast().
+// the step (returns false, nothing changed), see forward_weights_fast().  lane_carry: the product of
+// (1 - beta) over all keys right of this LANE's 32 keys (the right half-wave's is the carry that entered
+// the step), which is what the carry tables keep.
 template <int D, bool kCarryOnly, bool kFast, bool kPinBase>
 __device__ inline bool fwd_step(const char* ktile, const char* vtile, const LaneOffsets<D>& lo,
                                 const bf16x8 (&qf)[D / 16], f32x16 (&oacc)[D / 32], float& R, int lane,
-                                int key0, int q0w, int qi, int strict) {
+                                int key0, int q0w, int qi, int strict, float& lane_carry) {
     const int h = lane >> 5;
     float x[32];
     score_tiles_ps<D>(x, ktile, lo, qf);
     if (key0 + 63 + strict > q0w) mask_step(x, key0 + 32 * h, qi, strict);     // diagonal region
     bf16x8 pf[4];
     if (kFast) {
-        if (!forward_weights_fast<!kCarryOnly>(x, pf, R, lane)) return false;
+        if (!forward_weights_fast<!kCarryOnly>(x, pf, R, lane, lane_carry)) return false;
     } else {
         float dummy[1];
-        stick_weights<false>(x, dummy, R, lane);
+        stick_weights<false>(x, dummy, R, lane, &lane_carry);
         if (!kCarryOnly) {
 #pragma unroll
             for (int c = 0; c < 4; ++c) pf[c] = pack8(&x[8 * c]);
@@ -114,17 +116,24 @@ __global__ __launch_bounds__(kThreads) void mfma_fwd_kernel(KParams p) {
     wait_global_memory();
     __syncthreads();
 
+    // Carry tables: the right half-wave's carries go to `rtab`, the left one's to `rmid` (one store of the whole
+    // wave).  A step's carries are only known after its chain (the left half's contain the right half's
+    // product) and are stored at the top of the NEXT step, in front of its tile loads: vector-memory
+    // operations retire in order, so the wait for those loads at the end of that step also covers the store,
+    // long after it has completed, and no wait ever falls on a fresh store.
+    float* const my_tab = h ? p.rtab : p.rmid;
+    float carry_out = 1.0f;
+    int carry_step = -1;                       // wave-uniform: the step whose carries wait to be stored
+    auto store_carries = [&]() {
+        if (carry_step >= 0 && p.save) {
+            if (rows_full) my_tab[tabq + carry_step * kRowBlock] = carry_out;      // no lane mask
+            else if (qi < job.len) my_tab[tabq + carry_step * kRowBlock] = carry_out;
+        }
+        carry_step = -1;
+    };
     // what a step does before its arithmetic
     auto open_step = [&](int step, int buf, bool skip) {
-        // The carry-table store goes FIRST: vector-memory operations retire in order, so the
-        // wait for the tile loads at the end of the step then also covers this store, long
-        // after it has completed, instead of stalling the next iteration's loads on it.
-        // (A wave whose 32 rows all exist stores with every lane - both half-waves hold the same carry and
-        // write it to the same entry -, which spares the lane mask per step.)
-        if (!skip && p.save) {
-            if (rows_full) p.rtab[tabq + step * kRowBlock] = R;
-            else if (h == 0 && qi < job.len) p.rtab[tabq + step * kRowBlock] = R;
-        }
+        store_carries();
         if (step > 0) {   // next tiles, straight into the other buffer (free since the last barrier);
                           // every tile left of the sweep's first lies inside the sequence
             kc.issue_full((step - 1) * kKeyBlock, lds + (buf ^ 1) * 2 * kTile);
@@ -141,9 +150,12 @@ __global__ __launch_bounds__(kThreads) void mfma_fwd_kernel(KParams p) {
         const int key0 = step * kKeyBlock;
         const bool skip = key0 + strict > q0w + 31;       // whole step right of this wave's last query
         open_step(step, buf, skip);
-        if (!skip && !fwd_step<D, kCarryOnly, true, D == 128>(ktile, ktile + kTile, lo, qf, oacc, R, lane, key0, q0w, qi, strict)) {
-            redo = true;
-            break;
+        if (!skip) {
+            if (!fwd_step<D, kCarryOnly, true, D == 128>(ktile, ktile + kTile, lo, qf, oacc, R, lane, key0, q0w, qi, strict, carry_out)) {
+                redo = true;
+                break;
+            }
+            carry_step = step;
         }
         wait_global_memory();                  // the next tiles have landed
         __syncthreads();
@@ -154,10 +166,14 @@ __global__ __launch_bounds__(kThreads) void mfma_fwd_kernel(KParams p) {
         const bool skip = key0 + strict > q0w + 31;
         if (!redo) open_step(step, buf, skip);
         redo = false;
-        if (!skip) fwd_step<D, kCarryOnly, false, D == 128>(ktile, ktile + kTile, lo, qf, oacc, R, lane, key0, q0w, qi, strict);
+        if (!skip) {
+            fwd_step<D, kCarryOnly, false, D == 128>(ktile, ktile + kTile, lo, qf, oacc, R, lane, key0, q0w, qi, strict, carry_out);
+            carry_step = step;
+        }
         wait_global_memory();
         __syncthreads();
     }
+    store_carries();
 
     if (qi < job.len && !kCarryOnly) {
         store_o_row<D>(p, job, head, qi, lane, oacc);
@@ -228,11 +244,20 @@ __global__ __launch_bounds__(G * kThreads) void mfma_fwd_seg_kernel(KParams p) {
     wait_global_memory();
     __syncthreads();
 
-    auto open_step = [&](int step, int buf, bool skip) {
-        if (!skip && p.save) {                 // relative to the segment's right edge
-            if (rows_full) p.rtab[tabq + step * kRowBlock] = R;          // every lane stores: no lane mask per step
-            else if (h == 0 && qi < job.len) p.rtab[tabq + step * kRowBlock] = R;
+    // carry tables as in mfma_fwd_kernel (right half-wave -> rtab, left -> rmid, stored a step late), here
+    // relative to the segment's right edge
+    float* const my_tab = h ? p.rtab : p.rmid;
+    float carry_out = 1.0f;
+    int carry_step = -1;
+    auto store_carries = [&]() {
+        if (carry_step >= 0 && p.save) {
+            if (rows_full) my_tab[tabq + carry_step * kRowBlock] = carry_out;
+            else if (qi < job.len) my_tab[tabq + carry_step * kRowBlock] = carry_out;
         }
+        carry_step = -1;
+    };
+    auto open_step = [&](int step, int buf, bool skip) {
+        store_carries();
         if (step - 1 >= low) {
             kc.issue_full((step - 1) * kKeyBlock, my_tiles + (buf ^ 1) * 2 * kTile);
             if (!kCarryOnly) vc.issue_full((step - 1) * kKeyBlock, my_tiles + (buf ^ 1) * 2 * kTile + kTile);
@@ -246,9 +271,12 @@ __global__ __launch_bounds__(G * kThreads) void mfma_fwd_seg_kernel(KParams p) {
         const int key0 = step * kKeyBlock;
         const bool skip = step < low || key0 + strict > q0w + 31;
         open_step(step, buf, skip);
-        if (!skip && !fwd_step<D, kCarryOnly, true, true>(ktile, ktile + kTile, lo, qf, oacc, R, lane, key0, q0w, qi, strict)) {
-            redo = true;
-            break;
+        if (!skip) {
+            if (!fwd_step<D, kCarryOnly, true, true>(ktile, ktile + kTile, lo, qf, oacc, R, lane, key0, q0w, qi, strict, carry_out)) {
+                redo = true;
+                break;
+            }
+            carry_step = step;
         }
         wait_global_memory();
         __syncthreads();
@@ -260,10 +288,15 @@ __global__ __launch_bounds__(G * kThreads) void mfma_fwd_seg_kernel(KParams p) {
         const bool skip = step < low || key0 + strict > q0w + 31;
         if (!redo) open_step(step, buf, skip);
         redo = false;
-        if (!skip) fwd_step<D, kCarryOnly, false, true>(ktile, ktile + kTile, lo, qf, oacc, R, lane, key0, q0w, qi, strict);
+        if (!skip) {
+            fwd_step<D, kCarryOnly, false, true>(ktile, ktile + kTile, lo, qf, oacc, R, lane, key0, q0w, qi, strict, carry_out);
+            carry_step = step;
+        }
         wait_global_memory();
         __syncthreads();
     }
+    store_carries();
+    wait_global_memory();                      // the group's last entries are in memory before they are rescaled below
 
     // ---- segment totals -> F (what this group's results are relative to) and rem
     if (h == 0) totals[grp][32 * qs + n] = R;
@@ -275,19 +308,18 @@ __global__ __launch_bounds__(G * kThreads) void mfma_fwd_seg_kernel(KParams p) {
         if (g < grp) F *= t;
         all *= t;
     }
-    // carry-table entries of this group, written relative to its own right edge: times F.  Both
-    // half-waves take part (alternate steps); the loads go out in batches so that their
-    // latencies overlap.  The entries were written by this wave; its stores have completed
-    // (every iteration ends with a wait for all of the wave's memory traffic).
+    // carry-table entries of this group, written relative to its own right edge: times F.  Every lane
+    // rescales the entries it wrote (the half-waves have a table each); the loads go out in batches so that
+    // their latencies overlap.  Its stores have completed (wait above).
     if (p.save && grp > 0 && qi < job.len) {
-        for (int s0 = low + h; s0 < hi; s0 += 8) {
-            float v[4];
+        for (int s0 = low; s0 < hi; s0 += 8) {
+            float v[8];
 #pragma unroll
-            for (int j = 0; j < 4; ++j)
-                if (s0 + 2 * j < hi) v[j] = p.rtab[tabq + (s0 + 2 * j) * kRowBlock];
+            for (int j = 0; j < 8; ++j)
+                if (s0 + j < hi) v[j] = my_tab[tabq + (s0 + j) * kRowBlock];
 #pragma unroll
-            for (int j = 0; j < 4; ++j)
-                if (s0 + 2 * j < hi) p.rtab[tabq + (s0 + 2 * j) * kRowBlock] = v[j] * F;
+            for (int j = 0; j < 8; ++j)
+                if (s0 + j < hi) my_tab[tabq + (s0 + j) * kRowBlock] = v[j] * F;
         }
     }
     if (kCarryOnly) return;

@@ -90,13 +90,18 @@ def test_workspace_bytes(lib):
     # one carry table: per head, row block qb keeps 128 queries x its 2*qb + 2 visible 64-key blocks:
     # 32 * 33 columns of 128 floats at T = 4096 (half of a full [T/64][T] rectangle, plus the diagonal)
     table = 16 * 32 * 33 * 128 * 4
-    assert lib.sba_workspace_bytes(C.byref(p)) == table          # what the forward hands to the backward
-    assert lib.sba_bwd_scratch_bytes(C.byref(p)) == 4 * table + 256    # no workspace: the backward recomputes that table (+ error word)
+    # bf16: the forward hands two tables to the backward (the carries entering the right and the left half of every 64-key step)
+    assert lib.sba_workspace_bytes(C.byref(p)) == 2 * table
+    assert lib.sba_bwd_scratch_bytes(C.byref(p)) == 4 * table + 256    # no workspace: the backward recomputes those tables (+ error word)
     p.workspace = 1
-    assert lib.sba_bwd_scratch_bytes(C.byref(p)) == 3 * table + 256    # what the backward needs for itself
+    assert lib.sba_bwd_scratch_bytes(C.byref(p)) == 2 * table + 256    # what the backward needs for itself
     p.workspace = None
-    p.dtype = _lib.SBA_DTYPE_F32                    # fp32 at head_dim 64 runs on the matrix cores too: same tables
+    p.dtype = _lib.SBA_DTYPE_F32                    # fp32 at head_dim 64 runs on the matrix cores too: one table from the forward
     assert lib.sba_workspace_bytes(C.byref(p)) == table
+    assert lib.sba_bwd_scratch_bytes(C.byref(p)) == 4 * table + 256
+    p.workspace = 1
+    assert lib.sba_bwd_scratch_bytes(C.byref(p)) == 3 * table + 256
+    p.workspace = None
     p.head_dim = 128                                # and at head_dim 128
     assert lib.sba_workspace_bytes(C.byref(p)) == table
     p.head_dim = 96                                 # generic kernels: nothing kept, fp32 dk|dv accumulators
