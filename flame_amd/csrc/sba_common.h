@@ -30,10 +30,12 @@ struct KParams {
     const int32_t* schedule;
     TensorArg q, k, v, o, d_o, dq, dk, dv;
     VectorArg rem, d_rem;
-    float* rtab;                   // forward carry table (layout: tab_index() below)
-    float* gtab;                   // backward prefix table, same shape
-    float* rmid;                   // the same two carries in the MIDDLE of each 64-key block (entering
-    float* gmid;                   //   its left / right 32 keys), written by the dQ pass
+    float* rtab;                   // forward carry table (layout: tab_index() below): the product of (1 - beta) over all keys
+                                   //   right of a 64-key block, i.e. the carry entering its RIGHT 32 keys
+    float* gtab;                   // backward prefix table, same shape: sum of g over all keys left of the block
+    float* rmid;                   // the carry entering the block's LEFT 32 keys (bf16: written by the forward)
+    float* gmid;                   // the prefix entering the block's RIGHT 32 keys (written by the dQ pass, like gtab);
+                                   //   the bf16 dQ kernels rely on gmid - rtab == gtab - rmid
     float* dkv32;                  // generic path: fp32 dk|dv accumulators
     int* gave_up;                  // backward error word (set if a kernel abandoned a bounded internal wait)
     int64_t tab_head_stride;       // floats per head in each carry table

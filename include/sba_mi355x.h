@@ -115,16 +115,18 @@ const char* sba_error_string(int code);
 
 /*
  * Bytes of device workspace the pair (sba_fwd with save_for_backward, sba_bwd) shares for
- * this problem.  The forward writes its per-key-block carry table there and the backward
- * reads it back, so the SAME buffer, untouched in between, must be given to both calls
+ * this problem.  The forward writes its per-key-block carry tables there (bf16: two, the carry
+ * entering the right and the left half of every 64-key block; fp32: one) and the backward
+ * reads them back, so the SAME buffer, untouched in between, must be given to both calls
  * (the Python layer keeps it in the autograd context the way the reference keeps
  * neg_log_acc, sb_attn/__init__.py:30).  Only the size fields of `p` are read.
  */
 size_t sba_workspace_bytes(const SbaParams* p);
 
 /*
- * Bytes of device memory sba_bwd needs for the duration of the call only (three more
- * tables between its two kernels, or the generic path's fp32 accumulators): allocate before
+ * Bytes of device memory sba_bwd needs for the duration of the call only (the tables that its
+ * first kernel hands to its second - two in bf16, three in fp32 -, or the generic path's fp32
+ * accumulators): allocate before
  * the call, free after it has run.  With bwd_phases 1 and 2 issued as two calls, the same
  * buffer goes to both.  For bf16 at head_dim 64 / 128 the last 256 bytes hold an error word
  * (int32): the backward clears it and sets it to 1 if a kernel abandoned one of its bounded
@@ -132,8 +134,8 @@ size_t sba_workspace_bytes(const SbaParams* p);
  *
  * Memory-lean mode: a forward run WITHOUT save_for_backward keeps nothing, and sba_bwd called
  * with workspace = NULL first repeats the forward's sweep for the carries alone (about 0.7 of
- * a forward) into a fourth table of the scratch; this function then asks for four tables
- * (it looks at whether p->workspace is NULL).
+ * a forward) into further tables of the scratch; this function then asks for four tables in
+ * all (it looks at whether p->workspace is NULL).
  */
 size_t sba_bwd_scratch_bytes(const SbaParams* p);
 
