@@ -1191,17 +1191,18 @@ __global__ __launch_bounds__(kThreads, D == 64 ? 2 : 1) void mfma_bwd_dkv_own_ke
     // carries of a (query, this wave's 32 keys) pair: the right half of a 64-key block takes the
     // forward's block-edge carry and the mid-block prefix, the left half the other two
     const int kb64 = (q_begin + 32 * wave) / kKeyBlock;      // 2*rb or 2*rb + 1: a column of every row block's slab from rb on
-    const float* rsrc = ((wave & 1) ? p.rtab : p.rmid) + tab_index(p, head, job, 0, kb64);
-    const float* gsrc = ((wave & 1) ? p.gmid : p.gtab) + tab_index(p, head, job, 0, kb64);
+    const float* rsrc = ((wave & 1) ? p.rtab : p.rmid) + tab_index(p, head, job, 0, kb64) + n;
+    const float* gsrc = ((wave & 1) ? p.gmid : p.gtab) + tab_index(p, head, job, 0, kb64) + n;
     float Rn[2] = {1.f, 1.f}, Gn[2] = {0.f, 0.f};
+    // A step's 64 queries lie inside one 128-row block: the table index is a uniform base plus the lane's row.
+    // Rows past the end of the sequence are read too (the tables are allocated in whole row blocks) and not used.
     auto request_carries = [&](int q0) {
+        const int qb = q0 >> 7;
+        const int64_t ix = (int64_t)qb * (qb + 1) * kRowBlock + (q0 & (kRowBlock - 1));      // uniform
 #pragma unroll
         for (int t = 0; t < 2; ++t) {
-            const int qi = min(q0 + 32 * t + n, job.len - 1);
-            const int qb = qi >> 7;
-            const int64_t ix = (int64_t)qb * (qb + 1) * kRowBlock + (qi & (kRowBlock - 1));
-            Rn[t] = rsrc[ix];
-            Gn[t] = gsrc[ix];
+            Rn[t] = rsrc[ix + 32 * t];
+            Gn[t] = gsrc[ix + 32 * t];
         }
     };
     if (n_steps > 0) request_carries(q_begin);
