@@ -1488,10 +1488,16 @@ __global__ __launch_bounds__(2 * kThreads, 2) void mfma_bwd_dkv_pair_kernel(KPar
         constexpr int kDO = kQ + kQTile;
         const int q0 = q_begin + step * kStep;
         const float Rin = Rn, Gin = Gn;
+        // the score operands are requested first: their LDS round trip passes under the scalar work of the tile requests
+        bf16x8 bq[D / 16];
+#pragma unroll
+        for (int ks = 0; ks < D / 16; ++ks) bq[ks] = rows_at(row_at[ks], kQ);
+        __builtin_amdgcn_sched_barrier(0);
         if (step + 1 < n_steps) {     // next tiles, straight into the other buffer (nobody reads it since the last barrier)
             tc.issue(q0 + kStep, job.len, lds + (buf ^ 1) * 2 * kQTile + my_tile);
             request_carries(q0 + kStep);
         }
+        __builtin_amdgcn_sched_barrier(0);
         // whole step left of this pair's first key: nothing visible (the same for both waves of the pair)
         const bool skip = kb0 + strict > q0 + kStep - 1 || kb0 >= job.len;
         if (!skip) {
@@ -1509,10 +1515,6 @@ __global__ __launch_bounds__(2 * kThreads, 2) void mfma_bwd_dkv_pair_kernel(KPar
                 const float Gt = sees ? Gin : 0.0f;
                 float beta[16];
                 {
-                    bf16x8 bq[D / 16];
-#pragma unroll
-                    for (int ks = 0; ks < D / 16; ++ks) bq[ks] = rows_at(row_at[ks], kQ);
-                    __builtin_amdgcn_sched_barrier(0);     // all operands requested before the first MFMA: two waves per SIMD hide no LDS round trip per MFMA
                     f32x16 acc = {0};
 #pragma unroll
                     for (int ks = 0; ks < D / 16; ++ks) acc = mfma(kfr[ks], bq[ks], acc);
