@@ -923,12 +923,16 @@ __global__ __launch_bounds__((NP + 4) * 64, NP == 4 ? 2 : 3) void mfma_bwd_dkv_s
             const int qi = min(row0 + (ct & (kRowBlock - 1)), t.len - 1);
             const int qb = qi >> 7;            // row block of the query: its slab starts qb*(qb+1) columns in
             const int64_t ix = (int64_t)qb * (qb + 1) * kRowBlock + (qi & (kRowBlock - 1));
-            cR = t.rt[ix]; cG = t.gt[ix];
-            cRm = t.rm[ix]; cGm = t.gm[ix];
+            // (The pointers went through registers that the compiler cannot see into, see item_ptrs: it no longer knows
+            // that they point to global memory, and plain loads would become FLAT instructions, which also count as LDS
+            // traffic - every wait for an LDS read in the reduction would wait for these loads too.)
+            auto gl = [](const float* q) { return *(const __attribute__((address_space(1))) float*)q; };
+            cR = gl(t.rt + ix); cG = gl(t.gt + ix);
+            cRm = gl(t.rm + ix); cGm = gl(t.gm + ix);
 #pragma unroll
             for (int i = 0; i < 8; ++i) {
                 const uint32_t row = (uint32_t)min(row0 + crow + 16 * i, t.len - 1);
-                tx[i] = *(const u32x4*)(t.x + (size_t)row * x_st2);
+                tx[i] = *(const __attribute__((address_space(1))) u32x4*)(t.x + (size_t)row * x_st2);
             }
         };
         constexpr int kLoadsPerStep = 8 + 4;        // per lane: what request_step issues
@@ -1642,6 +1646,9 @@ int sba_launch_mfma_bwd(const sba::KParams& kp_in, int phases, hipStream_t s) {
     KParams kp = kp_in;
     dim3 grid((unsigned)kp.n_jobs * kp.n_heads);
     const bool p1 = phases != 2, p2 = phases != 1;
+    // the dQ kernels reach a lane's prefix entry from its carry entry by one uniform distance (see there)
+    if (!kp.rtab || !kp.rmid || !kp.gtab || !kp.gmid ||
+        (const char*)kp.gmid - (const char*)kp.rtab != (const char*)kp.gtab - (const char*)kp.rmid) return SBA_ERR_WORKSPACE;
     // Key-owner pass.  head_dim 64: from about three workgroups per CU on, the kernel whose waves
     // own their keys outright is ahead; below, the resident producer/consumer stream, which splits
     // the work into twice as many items and balances them itself.  head_dim 128: the own-keys
