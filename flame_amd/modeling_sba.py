@@ -19,7 +19,7 @@ import torch
 import torch.nn as nn
 import torch.nn.functional as F
 
-from .sba_layer import SBA
+from .sba_layer import SBA, fused_weight
 
 
 @dataclass
@@ -43,6 +43,15 @@ class SBAConfig:
         return 256 * ((w + 255) // 256)
 
 
+def _autocast_once(t: torch.Tensor) -> torch.Tensor:
+    """Under autocast every nn.Linear casts its fp32 input by itself: the norm output that feeds
+    q/k/v (or gate/up) would be cast three (two) times forward and its gradient as often backward.
+    Casting it once here gives the linears the same bits."""
+    if t.is_cuda and torch.is_autocast_enabled("cuda"):
+        return t.to(torch.get_autocast_dtype("cuda"))
+    return t
+
+
 class SBAMLP(nn.Module):
     def __init__(self, cfg: SBAConfig):
         super().__init__()
@@ -52,7 +61,9 @@ class SBAMLP(nn.Module):
         self.down_proj = nn.Linear(w, cfg.hidden_size, bias=False)
 
     def forward(self, x):
-        return self.down_proj(F.silu(self.gate_proj(x)) * self.up_proj(x))
+        # gate and up in one [hidden, 2*width] product (see SBA.forward); the parameters stay gate_proj / up_proj
+        g, u = F.linear(x, fused_weight(x, self.gate_proj.weight, self.up_proj.weight)).chunk(2, dim=-1)
+        return self.down_proj(F.silu(g) * u)
 
 
 class SBABlock(nn.Module):
@@ -65,9 +76,9 @@ class SBABlock(nn.Module):
         self.mlp = SBAMLP(cfg)
 
     def forward(self, x, **kwargs):
-        h, _, _ = self.attn(self.attn_norm(x), **kwargs)
+        h, _, _ = self.attn(_autocast_once(self.attn_norm(x)), **kwargs)
         x = x + h
-        return x + self.mlp(self.mlp_norm(x))
+        return x + self.mlp(_autocast_once(self.mlp_norm(x)))
 
 
 class SBAModel(nn.Module):

@@ -16,8 +16,33 @@ from typing import Callable, Optional
 
 import torch
 import torch.nn as nn
+import torch.nn.functional as F
 
 from .stickbreaking_attention import sb_attn, sb_attn_varlen
+
+
+class _CatCast(torch.autograd.Function):
+    """Row-wise concatenation of weight matrices, cast to `dtype` on the way (one multi-tensor copy instead of
+    a concatenation in fp32 plus autocast's cast of the result); the gradient goes back in slices, in each
+    weight's own dtype."""
+
+    @staticmethod
+    def forward(ctx, dtype, *ws):
+        ctx.rows = [w.shape[0] for w in ws]
+        ctx.dtypes = [w.dtype for w in ws]
+        out = torch.empty((sum(ctx.rows),) + tuple(ws[0].shape[1:]), dtype=dtype, device=ws[0].device)
+        torch._foreach_copy_(list(out.split(ctx.rows)), [w.detach() for w in ws])
+        return out
+
+    @staticmethod
+    def backward(ctx, g):
+        return (None,) + tuple(gi.to(dt) for gi, dt in zip(g.split(ctx.rows), ctx.dtypes))
+
+
+def fused_weight(like: torch.Tensor, *ws: torch.Tensor) -> torch.Tensor:
+    """The weights `ws` stacked for one GEMM, in the dtype the product will run in (autocast's, else the input's)."""
+    dtype = torch.get_autocast_dtype("cuda") if (like.is_cuda and torch.is_autocast_enabled("cuda")) else like.dtype
+    return _CatCast.apply(dtype, *ws)
 
 
 class SBA(nn.Module):
@@ -47,6 +72,7 @@ class SBA(nn.Module):
         self.k_proj = nn.Linear(hidden_size, self.kv_dim, bias=qkv_bias)
         self.v_proj = nn.Linear(hidden_size, self.kv_dim, bias=qkv_bias)
         self.o_proj = nn.Linear(hidden_size, hidden_size, bias=False)
+        self.fuse_qkv = True       # one GEMM for the three projections (same parameters, same results)
         # tests swap these for the CPU oracle to check the model wiring
         self.attn_fn: Callable = sb_attn
         self.attn_varlen_fn: Callable = sb_attn_varlen
@@ -57,20 +83,28 @@ class SBA(nn.Module):
         cu_seqlens = kwargs.get('cu_seqlens', None)
         B, T, _ = hidden_states.shape
         H, D = self.num_heads, self.head_dim
-        q = self.q_proj(hidden_states)
-        k = self.k_proj(hidden_states)
-        v = self.v_proj(hidden_states)
+        if self.fuse_qkv:
+            # one [hidden, 3*hidden] product instead of three [hidden, hidden] ones (the library's choice of
+            # GEMM kernel for the narrow ones runs at a fraction of the wide one's rate); q, k, v are column
+            # slices of its output - the kernels take strides - and the parameters stay q_proj / k_proj / v_proj
+            w = fused_weight(hidden_states, self.q_proj.weight, self.k_proj.weight, self.v_proj.weight)
+            b = fused_weight(hidden_states, self.q_proj.bias, self.k_proj.bias, self.v_proj.bias) if self.qkv_bias else None
+            q, k, v = F.linear(hidden_states, w, b).split((H * D, self.kv_dim, self.kv_dim), dim=-1)
+        else:
+            q = self.q_proj(hidden_states)
+            k = self.k_proj(hidden_states)
+            v = self.v_proj(hidden_states)
         if cu_seqlens is not None:
             if B != 1:
                 raise ValueError("cu_seqlens needs a packed batch of size 1")
             max_len = kwargs.get('max_seqlen', None)
             if max_len is None:
                 max_len = T            # an upper bound is enough (the carry tables are sized from the documents)
-            q, k, v = (x.view(T, H, D).transpose(0, 1) for x in (q, k, v))     # [H, T, D] views
+            q, k, v = (x.unflatten(-1, (H, D)).squeeze(0).transpose(0, 1) for x in (q, k, v))     # [H, T, D] views
             o, _ = self.attn_varlen_fn(q, k, v, cu_seqlens, max_len)
             o = o.transpose(0, 1).reshape(1, T, H * D)
         else:
-            q, k, v = (x.view(B, T, H, D).transpose(1, 2) for x in (q, k, v))  # [B, H, T, D] views
+            q, k, v = (x.unflatten(-1, (H, D)).transpose(1, 2) for x in (q, k, v))  # [B, H, T, D] views
             o, _ = self.attn_fn(q, k, v, None)
             o = o.transpose(1, 2).reshape(B, T, H * D)
         o = self.o_proj(o)
