@@ -47,6 +47,39 @@ def test_packed_documents_do_not_see_each_other():
     assert torch.allclose(lab[:, :17], la, atol=1e-5) and torch.allclose(lab[:, 17:], lb, atol=1e-5)
 
 
+def test_stacked_projections_equal_the_separate_ones():
+    # q/k/v (and gate/up) run as one product on stacked weights: same logits, same loss, and the same gradient
+    # for every one of the separate parameters, with and without biases
+    from flame_amd import modeling_sba as M
+    for bias in (False, True):
+        cfg = SBAConfig(hidden_size=64, num_hidden_layers=2, num_heads=2, vocab_size=97, qkv_bias=bias)
+        m = _oracle_model(cfg, seed=3)
+        if bias:
+            for layer in m.model.layers:
+                for proj in (layer.attn.q_proj, layer.attn.k_proj, layer.attn.v_proj):
+                    torch.nn.init.normal_(proj.bias, std=0.1)
+        ids = torch.randint(0, 97, (2, 21))
+        results = []
+        for fused in (True, False):
+            for layer in m.model.layers:
+                layer.attn.fuse_qkv = fused
+            mlp_forward = M.SBAMLP.forward
+            if not fused:
+                M.SBAMLP.forward = lambda self, x: self.down_proj(torch.nn.functional.silu(self.gate_proj(x)) * self.up_proj(x))
+            try:
+                m.zero_grad(set_to_none=True)
+                loss, logits = m(ids, labels=ids)
+                loss.backward()
+            finally:
+                M.SBAMLP.forward = mlp_forward
+            results.append((loss.detach(), logits.detach(), {n: p.grad.clone() for n, p in m.named_parameters()}))
+        (l1, g1, p1), (l2, g2, p2) = results
+        assert torch.allclose(l1, l2, atol=1e-6) and torch.allclose(g1, g2, atol=1e-5)
+        assert p1.keys() == p2.keys()
+        for n in p1:
+            assert torch.allclose(p1[n], p2[n], atol=1e-5, rtol=1e-4), n
+
+
 def test_label_shift_ignores_last_position():
     cfg = SBAConfig(hidden_size=32, num_hidden_layers=1, num_heads=2, vocab_size=11)
     m = _oracle_model(cfg)
