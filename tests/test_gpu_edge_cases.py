@@ -90,3 +90,34 @@ def test_longest_dense_row_65536_tokens_invariants():
     qs, ks, vs = (x[:, :1, T - W:].float().cpu() for x in (q, k, v))
     o_tail, rem_tail = O.sb_attn_oracle(qs, ks, vs)
     assert max_abs(o.detach()[:, :1, T - 256:].float().cpu(), o_tail[:, :, W - 256:]) <= 2e-2
+
+
+@pytest.mark.parametrize("D", [64, 128])
+def test_carries_that_underflow_to_zero(D):
+    # Logits around +6 in natural units (beta ~ 0.998): the product of (1 - beta) entering a key block is
+    # below the fp32 range after a few tens of keys, so the carry tables hold exact zeros for almost every
+    # (query, key block) pair, and the backward's chains start from a zero carry (an infinite W, NaNs mapped
+    # to 0 by the clamps).  Everything must stay finite and agree with the oracle: only the nearest keys
+    # have weight, all gradients of far keys are exactly zero.
+    from flame_amd import sb_attn
+    B, H, T = 1, 2, 1024
+    g = torch.Generator().manual_seed(900 + D)
+    base = torch.randn(D, generator=g)
+    base = base / base.norm()
+    amp = (6.0 * D ** 0.5) ** 0.5                      # q . k / sqrt(D) ~ 6
+    q = (amp * base + 0.05 * torch.randn(B, H, T, D, generator=g)).to(torch.bfloat16)
+    k = (amp * base + 0.05 * torch.randn(B, H, T, D, generator=g)).to(torch.bfloat16)
+    v = randn((B, H, T, D), 903, 0.25, torch.bfloat16)     # |o| <= 1: the tolerance on o is an absolute one
+    do = randn((B, H, T, D), 904, 1.0, torch.bfloat16)
+    drem = randn((B, H, T), 905, 1.0, torch.bfloat16)
+    print(f"underflowing carries, D={D}", flush=True)
+    qg, kg, vg = (x.cuda().requires_grad_(True) for x in (q, k, v))
+    o, rem = sb_attn(qg, kg, vg)
+    torch.autograd.backward([o, rem], [do.cuda(), drem.cuda()])
+    o_ref, rem_ref, dq, dk, dv = O.sb_attn_grads_oracle(q, k, v, do, drem, compute_dtype=torch.float64)
+    for t in (o, rem, qg.grad, kg.grad, vg.grad):
+        assert torch.isfinite(t).all()
+    assert max_abs(o.detach().float().cpu(), o_ref.float()) <= 2e-2
+    assert max_abs(rem.detach().float().cpu(), rem_ref.float()) <= 2e-2
+    for got, ref in ((qg.grad, dq), (kg.grad, dk), (vg.grad, dv)):
+        assert rel_l2(got.float().cpu(), ref.float()) <= 5e-2
