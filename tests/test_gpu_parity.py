@@ -545,6 +545,36 @@ def test_randomized_packed_batches_mfma_vs_generic_backward(dkv_kernel, D, monke
             assert rel_l2(x.float(), y.float()) <= 5e-2
 
 
+def test_seeded_random_sweep_of_shapes_layouts_and_dtypes_against_the_oracle():
+    # 120 seeded draws over what the fixed cases above leave between them: batch and head counts,
+    # lengths from 1 to 2 000 at and off the 64 / 128 block edges, head dims on the matrix-core
+    # kernels (64, 128) and on the zero-padded route (16, 32, 80, 96), both dtypes, both masks,
+    # dense and packed (with empty documents), with and without a gradient for rem, inputs scaled
+    # 0.5 and 0.75 (|o| stays below 4, where half a bf16 ulp of the output is 0.008).
+    import random
+    rng = random.Random(20240607)
+    for case in range(120):
+        D = rng.choice([64, 64, 128, 128, 16, 32, 80, 96])
+        dtype = rng.choice([torch.bfloat16, torch.bfloat16, torch.bfloat16, torch.float32])
+        ac = rng.random() < 0.3
+        seed = rng.randrange(10 ** 6)
+        scale = rng.choice([0.5, 0.75])
+        if rng.random() < 0.5:
+            B, H = rng.choice([1, 1, 2, 3]), rng.choice([1, 2, 3, 5])
+            T = max(1, rng.choice([rng.randrange(1, 70), rng.randrange(1, 400), rng.randrange(1, 2000),
+                                   128 * rng.randrange(1, 13), 64 * rng.randrange(1, 25) + rng.choice([-1, 0, 1])]))
+            _check_dense(B, H, T, D, dtype, ac, seed=seed, in_scale=scale, with_drem=rng.random() < 0.8)
+        else:
+            H = rng.choice([1, 2, 4, 16])
+            lens = [max(0 if rng.random() < 0.1 else 1,
+                        rng.choice([rng.randrange(0, 40), rng.randrange(1, 300), rng.randrange(1, 1200),
+                                    128 * rng.randrange(1, 6), 64 * rng.randrange(1, 10) + rng.choice([-1, 1])]))
+                    for _ in range(rng.randrange(1, 14))]
+            if sum(lens) == 0:
+                lens.append(5)
+            _check_varlen(H, D, lens, dtype, ac, seed=seed, in_scale=scale)
+
+
 def test_forward_backward_captured_in_a_graph_replays_like_eager():
     # The C ABI allocates nothing and never synchronises, so a forward + backward can be captured
     # in a HIP graph.  Replayed three times with new input contents, with eager work in between,
