@@ -21,6 +21,7 @@
 // Every element of the score matrix is therefore evaluated twice in the backward (once per
 // pass); in exchange nothing is reduced through memory.
 #include <string.h>
+#include <atomic>
 #include <type_traits>
 #include "sba_mfma.h"
 
@@ -1621,15 +1622,15 @@ bool sba_mfma_bwd_available() { return true; }
 
 // compute units of the current device (asked once per device)
 static int sba_cu_count() {
-    static int cached[64] = {0};
+    static std::atomic<int> cached[64];       // zero-initialised; threads that race here store the same value
     int dev = 0;
     if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) dev = 0;
-    if (cached[dev] == 0) {
-        int n = 0;
+    int n = cached[dev].load(std::memory_order_relaxed);
+    if (n == 0) {
         if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
-        cached[dev] = n;
+        cached[dev].store(n, std::memory_order_relaxed);
     }
-    return cached[dev];
+    return n;
 }
 
 // SBA_DKV_KERNEL=own / =other overrides the choice between the key-owner kernels (tests run
