@@ -134,6 +134,24 @@ def usable(t: torch.Tensor) -> torch.Tensor:
     return t if ok else t.contiguous()
 
 
+def empty_grads_like(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor):
+    """Uninitialised dq, dk, dv.  When q, k and v are the three column slices of one [.., 3*H*D] tensor (the
+    output of a stacked q/k/v projection), the gradients are laid out the same way in ONE allocation, so that
+    the caller's backward can hand the whole of it to the projection without concatenating."""
+    if not torch.compiler.is_compiling() and q.shape == k.shape == v.shape and q.stride() == k.stride() == v.stride():
+        n = q.numel()
+        span = sum((sz - 1) * st for sz, st in zip(q.shape, q.stride())) + 1      # elements from q's first to its last
+        base = q.untyped_storage().data_ptr()
+        if (k.untyped_storage().data_ptr() == base and v.untyped_storage().data_ptr() == base and n > 0
+                and q.stride(-1) == 1):
+            step = k.storage_offset() - q.storage_offset()
+            # interleaved thirds of one dense buffer: q's span plus the two slices to its right is exactly 3n
+            if step > 0 and v.storage_offset() - k.storage_offset() == step and span + 2 * step == 3 * n:
+                buf = torch.empty(3 * n, dtype=q.dtype, device=q.device)
+                return tuple(buf.as_strided(q.shape, q.stride(), i * step) for i in range(3))
+    return torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+
+
 def recompute_carries() -> bool:
     """SBA_RECOMPUTE_CARRIES=1: keep nothing between forward and backward (the reference keeps one
     float per query, the default here one carry table of H x T/64 x tokens floats); the backward

@@ -52,6 +52,36 @@ def _autocast_once(t: torch.Tensor) -> torch.Tensor:
     return t
 
 
+class _SwiGLU(torch.autograd.Function):
+    """silu(g) * u on y = [g | u] (the output of the stacked gate/up product).  What autograd would do, except
+    that the two halves of the gradient are written straight into one [.., 2*width] tensor - the shape the
+    stacked product's backward wants - instead of being concatenated afterwards."""
+
+    @staticmethod
+    def forward(ctx, y):
+        g, u = y.chunk(2, dim=-1)
+        s = F.silu(g)
+        ctx.save_for_backward(y, s)
+        return s * u
+
+    @staticmethod
+    def backward(ctx, do):
+        y, s = ctx.saved_tensors
+        g, u = y.chunk(2, dim=-1)
+        dy = torch.empty_like(y)
+        dg, du = dy.chunk(2, dim=-1)
+        torch.mul(do, s, out=du)
+        torch.ops.aten.silu_backward.grad_input(do * u, g, grad_input=dg)
+        return dy
+
+
+def swiglu(y: torch.Tensor) -> torch.Tensor:
+    if torch.compiler.is_compiling():       # the compiler fuses the plain form by itself
+        g, u = y.chunk(2, dim=-1)
+        return F.silu(g) * u
+    return _SwiGLU.apply(y)
+
+
 class SBAMLP(nn.Module):
     def __init__(self, cfg: SBAConfig):
         super().__init__()
@@ -62,8 +92,7 @@ class SBAMLP(nn.Module):
 
     def forward(self, x):
         # gate and up in one [hidden, 2*width] product (see SBA.forward); the parameters stay gate_proj / up_proj
-        g, u = F.linear(x, fused_weight(x, self.gate_proj.weight, self.up_proj.weight)).chunk(2, dim=-1)
-        return self.down_proj(F.silu(g) * u)
+        return self.down_proj(swiglu(F.linear(x, fused_weight(x, self.gate_proj.weight, self.up_proj.weight))))
 
 
 class SBABlock(nn.Module):

@@ -39,6 +39,51 @@ class _CatCast(torch.autograd.Function):
         return (None,) + tuple(gi.to(dt) for gi, dt in zip(g.split(ctx.rows), ctx.dtypes))
 
 
+class _SplitColumns(torch.autograd.Function):
+    """y.split(sizes, -1).  Its backward looks whether the incoming gradients already lie side by side as the
+    column slices of one dense tensor (the attention operator allocates dq, dk, dv that way when q, k, v are
+    such slices) and then returns that tensor as it is; otherwise it concatenates, as autograd would."""
+
+    @staticmethod
+    def forward(ctx, y, *sizes):
+        ctx.sizes = sizes
+        ctx.like = (y.shape, y.dtype, y.device)
+        return y.split(sizes, dim=-1)
+
+    @staticmethod
+    def backward(ctx, *gs):
+        shape, dtype, device = ctx.like
+        whole = None if torch.compiler.is_compiling() else _adjacent_columns(gs, shape)
+        if whole is None:
+            lead = shape[:-1]
+            whole = torch.cat([g if g is not None else torch.zeros(lead + (n,), dtype=dtype, device=device)
+                               for g, n in zip(gs, ctx.sizes)], dim=-1)
+        return (whole,) + (None,) * len(ctx.sizes)
+
+
+def _adjacent_columns(gs, shape):
+    """The tensor of shape `shape` whose column slices the `gs` are, if there is one."""
+    if any(g is None for g in gs):
+        return None
+    dense, acc = [], 1
+    for n in reversed(shape):
+        dense.append(acc)
+        acc *= max(n, 1)
+    dense = tuple(reversed(dense))
+    g0 = gs[0]
+    off = g0.storage_offset()
+    base = g0.untyped_storage().data_ptr()
+    for g in gs:
+        same_rows = all(a == b or n == 1 for a, b, n in zip(g.stride()[:-1], dense[:-1], shape[:-1]))
+        if (g.shape[:-1] != shape[:-1] or not same_rows or (g.stride(-1) != 1 and g.shape[-1] > 1) or g.dtype != g0.dtype
+                or g.storage_offset() != off or g.untyped_storage().data_ptr() != base):
+            return None
+        off += g.shape[-1]
+    if off - g0.storage_offset() != shape[-1]:
+        return None
+    return g0.as_strided(shape, dense, g0.storage_offset())
+
+
 def fused_weight(like: torch.Tensor, *ws: torch.Tensor) -> torch.Tensor:
     """The weights `ws` stacked for one GEMM, in the dtype the product will run in (autocast's, else the input's)."""
     dtype = torch.get_autocast_dtype("cuda") if (like.is_cuda and torch.is_autocast_enabled("cuda")) else like.dtype
@@ -89,7 +134,7 @@ class SBA(nn.Module):
             # slices of its output - the kernels take strides - and the parameters stay q_proj / k_proj / v_proj
             w = fused_weight(hidden_states, self.q_proj.weight, self.k_proj.weight, self.v_proj.weight)
             b = fused_weight(hidden_states, self.q_proj.bias, self.k_proj.bias, self.v_proj.bias) if self.qkv_bias else None
-            q, k, v = F.linear(hidden_states, w, b).split((H * D, self.kv_dim, self.kv_dim), dim=-1)
+            q, k, v = _SplitColumns.apply(F.linear(hidden_states, w, b), H * D, self.kv_dim, self.kv_dim)
         else:
             q = self.q_proj(hidden_states)
             k = self.k_proj(hidden_states)

@@ -95,7 +95,7 @@ def _fwd(q, k, v, logit_scale, attend_current=False, no_grad=False):
 
 
 def _bwd(do, dr, q, k, v, ws, logit_scale, attend_current=False):
-    dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+    dq, dk, dv = _lib.empty_grads_like(q, k, v)     # one allocation when q, k, v are slices of one tensor
     # freed when this call returns: only the forward's table is kept between the two directions
     scratch = torch.empty(max(bwd_scratch_bytes(q, ws.numel() > 16), 16), dtype=torch.uint8, device=q.device)
     _compileable_backward(do, dr, q, k, v, ws, scratch, float(logit_scale), bool(attend_current), dq, dk, dv)

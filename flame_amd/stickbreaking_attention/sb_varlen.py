@@ -155,7 +155,7 @@ def varlen_fwd(q, k, v, cu_seqlens, max_seqlens, logit_scale, attend_current=Fal
 
 
 def varlen_bwd(do, dr, q, k, v, cu_seqlens, max_seqlens, ws, logit_scale, attend_current=False):
-    dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+    dq, dk, dv = _lib.empty_grads_like(q, k, v)     # one allocation when q, k, v are slices of one tensor
     # freed when this call returns: only the forward's table is kept between the two directions
     scratch = torch.empty(max(bwd_scratch_bytes(q, cu_seqlens, max_seqlens, ws.numel() > 16), 16), dtype=torch.uint8,
                           device=q.device)

@@ -89,6 +89,33 @@ def test_no_grad_forward_keeps_no_carry_table():
     assert torch.equal(o_train, o_eval)
 
 
+def test_layer_backward_of_the_stacked_projection_needs_no_concatenation(monkeypatch):
+    # q, k, v are column slices of the stacked projection's output; the operator lays dq, dk, dv out the same
+    # way in one allocation and the layer's split hands that allocation to the projection's backward.  Both
+    # routes (dense, packed), against the layer with three separate projections.
+    from flame_amd import sba_layer
+    from flame_amd.sba_layer import SBA
+    handed = []
+    found = sba_layer._adjacent_columns
+    monkeypatch.setattr(sba_layer, "_adjacent_columns", lambda gs, shape: handed.append(found(gs, shape)) or handed[-1])
+    torch.manual_seed(5)
+    layer = SBA(hidden_size=256, num_heads=4).cuda().to(torch.bfloat16)
+    x = (torch.randn(2, 200, 256, device="cuda") * 0.5).to(torch.bfloat16)
+    cu = cu_from_lengths([130, 7, 200, 63]).cuda()
+    for kwargs, xin in (({}, x), ({"cu_seqlens": cu}, x.reshape(1, 400, 256))):
+        grads = []
+        for fused in (True, False):
+            layer.fuse_qkv = fused
+            layer.zero_grad(set_to_none=True)
+            xi = xin.clone().requires_grad_(True)
+            o, _, _ = layer(xi, **kwargs)
+            o.float().square().sum().backward()
+            grads.append([xi.grad.float()] + [p.grad.float() for p in layer.parameters()])
+        for a, b in zip(*grads):
+            assert rel_l2(a, b) <= 2e-2
+    assert len(handed) == 2 and all(h is not None for h in handed)
+
+
 def test_torch_compile_fullgraph_on_the_layer_dense_and_packed():
     # flame compiles every block (flame/models/parallelize_fla.py:369-403); the layer has to
     # trace as one graph on both routes, and match eager and the oracle

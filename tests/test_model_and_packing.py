@@ -80,6 +80,42 @@ def test_stacked_projections_equal_the_separate_ones():
             assert torch.allclose(p1[n], p2[n], atol=1e-5, rtol=1e-4), n
 
 
+def test_column_split_hands_adjacent_gradients_through_without_a_copy():
+    # the q/k/v split of the stacked projection: gradients that already lie side by side in one buffer (how the
+    # operator allocates dq, dk, dv for such inputs) go back as that buffer; anything else is concatenated
+    from flame_amd import _lib
+    from flame_amd.sba_layer import _SplitColumns
+    H, D, T = 4, 8, 10
+    y = torch.randn(1, T, 3 * H * D, requires_grad=True)
+    q, k, v = (x.unflatten(-1, (H, D)).squeeze(0).transpose(0, 1) for x in _SplitColumns.apply(y, H * D, H * D, H * D))
+    dq, dk, dv = _lib.empty_grads_like(q.detach(), k.detach(), v.detach())
+    assert dq.stride() == q.stride() and dq.untyped_storage().data_ptr() == dv.untyped_storage().data_ptr()
+    for t in (dq, dk, dv):
+        t.copy_(torch.randn_like(t))
+    expect = torch.cat([t.transpose(0, 1).reshape(1, T, H * D) for t in (dq, dk, dv)], -1)
+    (g,) = torch.autograd.grad((q, k, v), y, (dq, dk, dv), retain_graph=True)
+    assert torch.equal(g, expect) and g.untyped_storage().data_ptr() == dq.untyped_storage().data_ptr()
+    # separate allocations, a missing gradient, a different order: the concatenating route, same values
+    sep = tuple(t.clone() for t in (dq, dk, dv))
+    (g,) = torch.autograd.grad((q, k, v), y, sep, retain_graph=True)
+    assert torch.equal(g, expect)
+    (g,) = torch.autograd.grad((q, v), y, (dq, dv), retain_graph=True)
+    assert torch.equal(g[..., :H * D], expect[..., :H * D]) and not g[..., H * D:2 * H * D].any()
+    (g,) = torch.autograd.grad((q, k, v), y, (dk, dq, dv), retain_graph=True)
+    assert torch.equal(g[..., :H * D], expect[..., H * D:2 * H * D])
+    # tensors that are not slices of one buffer get plain allocations
+    a, b, c = _lib.empty_grads_like(torch.zeros(2, 3, 4), torch.zeros(2, 3, 4), torch.zeros(2, 3, 4))
+    assert a.is_contiguous() and a.untyped_storage().data_ptr() != b.untyped_storage().data_ptr()
+
+
+def test_swiglu_function_matches_autograd():
+    from flame_amd.modeling_sba import _SwiGLU
+    y = torch.randn(3, 5, 12, dtype=torch.float64, requires_grad=True)
+    assert torch.autograd.gradcheck(_SwiGLU.apply, (y,))
+    g, u = y.chunk(2, dim=-1)
+    assert torch.equal(_SwiGLU.apply(y), torch.nn.functional.silu(g) * u)
+
+
 def test_label_shift_ignores_last_position():
     cfg = SBAConfig(hidden_size=32, num_hidden_layers=1, num_heads=2, vocab_size=11)
     m = _oracle_model(cfg)
