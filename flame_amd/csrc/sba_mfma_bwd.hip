@@ -1214,26 +1214,40 @@ __global__ __launch_bounds__(kThreads, D == 64 ? 2 : 1) void mfma_bwd_dkv_own_ke
     wait_global_memory();
     __syncthreads();
 
-    auto second_tile_reduction = [&](const char* qt, const char* dot) {
+    // Every LDS address of the loop is "a register that is fixed for the whole sweep + a constant": the lane offsets are
+    // made absolute once (Q / dO tiles from the start of the array, the weight tile from this wave's tile), and the loop
+    // runs in one copy per tile buffer, so that buffer and row offsets are compile-time numbers in the offset fields of
+    // the fetches (with the tile address in a scalar register each fetch or pinned sum costs a vector add with a scalar
+    // operand: 25 of them per step here).
+    lo.rebase(lds);
+    lz.rebase(ztile);
+    constexpr TileAt zt{0};
+    uint32_t zst[4];              // this lane's row of the weight tile: chunks 2h, 2h + 1 (a) and 4 + 2h, 4 + 2h + 1 (dz)
+#pragma unroll
+    for (int c = 0; c < 4; ++c) zst[c] = lds_lane_base(ztile, tile_offset<64>(n, (c >> 1) * 4 + 2 * h + (c & 1)));
+    auto put_z = [&](int c, int t, bf16x8 v) __attribute__((always_inline)) {
+        *(__attribute__((address_space(3))) bf16x8*)((__attribute__((address_space(3))) char*)(uintptr_t)zst[c] + t * 32 * 64 * 2) = v;
+    };
+
+    auto second_tile_reduction = [&](auto qt, auto dot) __attribute__((always_inline)) {
 #pragma unroll
         for (int kk = 2; kk < 4; ++kk) {
-            const bf16x8 af = fetch_nat_o<64, kOwnPin>(ztile, lz, 16 * kk, 0);
-            const bf16x8 zf = fetch_nat_o<64, kOwnPin>(ztile, lz, 16 * kk, 1);
+            const bf16x8 af = fetch_nat_o<64>(zt, lz, 16 * kk, 0);
+            const bf16x8 zf = fetch_nat_o<64>(zt, lz, 16 * kk, 1);
 #pragma unroll
             for (int db = 0; db < D / 32; ++db) {
-                dvacc[db] = mfma(af, fetch_nat_o<D, kOwnPin>(dot, lo, 16 * kk, db), dvacc[db]);
-                dkacc[db] = mfma(zf, fetch_nat_o<D, kOwnPin>(qt, lo, 16 * kk, db), dkacc[db]);
+                dvacc[db] = mfma(af, fetch_nat_o<D>(dot, lo, 16 * kk, db), dvacc[db]);
+                dkacc[db] = mfma(zf, fetch_nat_o<D>(qt, lo, 16 * kk, db), dkacc[db]);
             }
         }
     };
     bool pending = false;                      // the previous step left its second tile's reduction to this one
-    int buf = 0, pbuf = 0;
-    for (int step = 0; step < n_steps; ++step) {
-        const char* qtile = lds + buf * 2 * kQTile;
-        const char* dotile = qtile + kQTile;
-        const char* pqtile = lds + pbuf * 2 * kQTile;        // the previous step's tiles (kDefer)
-        const char* pdotile = pqtile + kQTile;
-        const int nbuf = buf + 1 == kNBuf ? 0 : buf + 1;
+    auto do_step = [&](int step, auto buf_c) __attribute__((always_inline)) {
+        constexpr int buf = decltype(buf_c)::value;
+        constexpr int nbuf = buf + 1 == kNBuf ? 0 : buf + 1;
+        constexpr int pbuf = buf == 0 ? kNBuf - 1 : buf - 1;
+        constexpr TileAt qtile{buf * 2 * kQTile}, dotile{buf * 2 * kQTile + kQTile};
+        constexpr TileAt pqtile{pbuf * 2 * kQTile}, pdotile{pbuf * 2 * kQTile + kQTile};      // the previous step's tiles (kDefer)
         const int q0 = q_begin + step * kStep;
         const bool more = step + 1 < n_steps;
         float Rin[2], Gin[2];
@@ -1262,7 +1276,7 @@ __global__ __launch_bounds__(kThreads, D == 64 ? 2 : 1) void mfma_bwd_dkv_own_ke
                     // each MFMA: all operands of the tile are requested first
                     bf16x8 bq[D / 16];
 #pragma unroll
-                    for (int ks = 0; ks < D / 16; ++ks) bq[ks] = kOwnPin ? fetch_rows_p<D>(qtile, lo, t, ks) : fetch_row_nat<D>(qtile, 32 * t + n, ks, lane);
+                    for (int ks = 0; ks < D / 16; ++ks) bq[ks] = fetch_rows_o<D>(qtile, lo, t, ks);
                     if (D == 128) __builtin_amdgcn_sched_barrier(0);
                     f32x16 acc = {0};
 #pragma unroll
@@ -1278,8 +1292,10 @@ __global__ __launch_bounds__(kThreads, D == 64 ? 2 : 1) void mfma_bwd_dkv_own_ke
                 if (t == 0 && kDefer && pending) {
                     // the previous step's second tile: rows 32.. of the wave's weight tile (not yet
                     // overwritten: this step's second tile comes later) and of the previous Q / dO tiles
-                    auto red_a = [&](int seg) { return fetch_nat_o<64, kOwnPin>(ztile, lz, 32 + 16 * (seg >> 1), seg & 1); };
-                    auto red_b = [&](int seg, int db) { return fetch_nat_o<D, kOwnPin>((seg & 1) ? pqtile : pdotile, lo, 32 + 16 * (seg >> 1), db); };
+                    auto red_a = [&](int seg) { return fetch_nat_o<64>(zt, lz, 32 + 16 * (seg >> 1), seg & 1); };
+                    auto red_b = [&](int seg, int db) {
+                        return (seg & 1) ? fetch_nat_o<D>(pqtile, lo, 32 + 16 * (seg >> 1), db) : fetch_nat_o<D>(pdotile, lo, 32 + 16 * (seg >> 1), db);
+                    };
                     bf16x8 na = red_a(0), nb[D / 32];
 #pragma unroll
                     for (int db = 0; db < D / 32; ++db) nb[db] = red_b(0, db);
@@ -1305,8 +1321,10 @@ __global__ __launch_bounds__(kThreads, D == 64 ? 2 : 1) void mfma_bwd_dkv_own_ke
                     // The reduction over the first tile's 32 queries only needs that tile's weights, which
                     // this wave wrote above: its MFMAs go between the segments of the second tile's chain,
                     // whose exp/rcp overlap them.  Segment 2kk: dV += A^T dO, segment 2kk + 1: dK += dZ^T Q.
-                    auto red_a = [&](int seg) { return fetch_nat_o<64, kOwnPin>(ztile, lz, 16 * (seg >> 1), seg & 1); };
-                    auto red_b = [&](int seg, int db) { return fetch_nat_o<D, kOwnPin>((seg & 1) ? qtile : dotile, lo, 16 * (seg >> 1), db); };
+                    auto red_a = [&](int seg) { return fetch_nat_o<64>(zt, lz, 16 * (seg >> 1), seg & 1); };
+                    auto red_b = [&](int seg, int db) {
+                        return (seg & 1) ? fetch_nat_o<D>(qtile, lo, 16 * (seg >> 1), db) : fetch_nat_o<D>(dotile, lo, 16 * (seg >> 1), db);
+                    };
                     bf16x8 na = red_a(0), nb[D / 32];
 #pragma unroll
                     for (int db = 0; db < D / 32; ++db) nb[db] = red_b(0, db);
@@ -1330,7 +1348,7 @@ __global__ __launch_bounds__(kThreads, D == 64 ? 2 : 1) void mfma_bwd_dkv_own_ke
                 {
                     bf16x8 bd[D / 16];
 #pragma unroll
-                    for (int ks = 0; ks < D / 16; ++ks) bd[ks] = kOwnPin ? fetch_rows_p<D>(dotile, lo, t, ks) : fetch_row_nat<D>(dotile, 32 * t + n, ks, lane);
+                    for (int ks = 0; ks < D / 16; ++ks) bd[ks] = fetch_rows_o<D>(dotile, lo, t, ks);
                     if (D == 128) __builtin_amdgcn_sched_barrier(0);
                     f32x16 acc = {0};
 #pragma unroll
@@ -1339,11 +1357,11 @@ __global__ __launch_bounds__(kThreads, D == 64 ? 2 : 1) void mfma_bwd_dkv_own_ke
                     for (int r = 0; r < 16; ++r) dp[r] = acc[r];
                 }
                 // a -> columns 16h.. of row (32t + n), dz -> columns 32 + 16h..
-                *(bf16x8*)(ztile + tile_offset<64>(32 * t + n, 2 * h)) = pack8(&x[0]);
-                *(bf16x8*)(ztile + tile_offset<64>(32 * t + n, 2 * h + 1)) = pack8(&x[8]);
+                put_z(0, t, pack8(&x[0]));
+                put_z(1, t, pack8(&x[8]));
                 own_tile_grads(x, beta, dp, Gt, lane);
-                *(bf16x8*)(ztile + tile_offset<64>(32 * t + n, 4 + 2 * h)) = pack8(&dp[0]);
-                *(bf16x8*)(ztile + tile_offset<64>(32 * t + n, 4 + 2 * h + 1)) = pack8(&dp[8]);
+                put_z(2, t, pack8(&dp[0]));
+                put_z(3, t, pack8(&dp[8]));
             }
             // dV += A^T dO, dK += dZ^T Q over the second tile's queries (the first tile's went with the
             // second chain): now, or with the next step's first chain
@@ -1352,10 +1370,20 @@ __global__ __launch_bounds__(kThreads, D == 64 ? 2 : 1) void mfma_bwd_dkv_own_ke
         }
         wait_global_memory();                  // the next tiles and carries have landed
         __syncthreads();
-        pbuf = buf;
-        buf = nbuf;
+    };
+    // one copy of the step per tile buffer
+    int last_buf = 0;
+    for (int step = 0; step < n_steps; step += kNBuf) {
+        do_step(step, std::integral_constant<int, 0>{});
+        last_buf = 0;
+        if (step + 1 < n_steps) { do_step(step + 1, std::integral_constant<int, 1>{}); last_buf = 1; }
+        if (kNBuf == 3 && step + 2 < n_steps) { do_step(step + 2, std::integral_constant<int, kNBuf - 1>{}); last_buf = 2; }
     }
-    if (kDefer && pending) second_tile_reduction(lds + pbuf * 2 * kQTile, lds + pbuf * 2 * kQTile + kQTile);
+    if (kDefer && pending) {
+        if (last_buf == 0) second_tile_reduction(TileAt{0}, TileAt{kQTile});
+        else if (last_buf == 1) second_tile_reduction(TileAt{2 * kQTile}, TileAt{3 * kQTile});
+        else second_tile_reduction(TileAt{(kNBuf - 1) * 2 * kQTile}, TileAt{(kNBuf - 1) * 2 * kQTile + kQTile});
+    }
 
     // ---- rows kb0.. of dK (scaled) and dV, through the wave's own tile as coalesced 16-byte stores
 #pragma unroll
