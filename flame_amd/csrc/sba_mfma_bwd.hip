@@ -272,10 +272,14 @@ __global__ __launch_bounds__(2 * kThreads, 2) void mfma_bwd_dq2_kernel(KParams p
     bool g_pending = false;
     wait_global_memory();
     __syncthreads();
-    for (int it = 0, buf = 0; it < n_it; ++it, buf ^= 1) {
+    // Every LDS address of the loop is a sweep-constant register plus an immediate: the lane offsets are made absolute
+    // for this group's tiles once, and the loop runs in one copy per tile buffer (see the one-step kernel).
+    lo.rebase(my_tiles);
+    auto do_iteration = [&](int it, auto buf_c) __attribute__((always_inline)) {
+        constexpr int buf = decltype(buf_c)::value;
+        constexpr TileAt ktile = {buf * 4 * kTile};
+        constexpr TileAt vtile = {buf * 4 * kTile + kTile};
         const int step = 2 * it + grp;                   // == n_steps: this group idles in the last iteration
-        const char* ktile = my_tiles + buf * 4 * kTile;
-        const char* vtile = ktile + kTile;
         const bool more = step + 2 < n_steps;
         const int key0 = step * kKeyBlock;
         const bool active = step < n_steps && !(key0 + strict > q0w + 31);
@@ -329,6 +333,10 @@ __global__ __launch_bounds__(2 * kThreads, 2) void mfma_bwd_dq2_kernel(KParams p
         rcur += 2 * tstride;
         wait_global_memory();                  // the next tiles have landed
         __syncthreads();
+    };
+    for (int it = 0; it < n_it; it += 2) {
+        do_iteration(it, std::integral_constant<int, 0>{});
+        if (it + 1 < n_it) do_iteration(it + 1, std::integral_constant<int, 1>{});
     }
 
     if (g_pending && row_ok) *(float*)((char*)(rcur - 2 * tstride) + g_from_r) = Gstore;
