@@ -98,7 +98,7 @@ __global__ __launch_bounds__(kThreads, 2) void mfma_bwd_dq_kernel(KParams p) {
         constexpr TileAt vtile = {buf * 2 * kTile + kTile};
         const bool more = step + 1 < n_steps;
         const int key0 = step * kKeyBlock;
-        const bool skip = key0 + strict > q0w + 31;
+        const bool skip = key0 + strict > q0w + 31 || q0w >= job.len;     // nothing visible, or no query of this wave inside the sequence
         // the prefixes that entered the previous step (the first block's are only known once that
         // block's weights are: they start at d_rem * rem, see below)
         if (g_pending && row_ok) *(float*)((char*)(rcur - tstride) + g_from_r) = Gstore;
@@ -282,7 +282,7 @@ __global__ __launch_bounds__(2 * kThreads, 2) void mfma_bwd_dq2_kernel(KParams p
         const int step = 2 * it + grp;                   // == n_steps: this group idles in the last iteration
         const bool more = step + 2 < n_steps;
         const int key0 = step * kKeyBlock;
-        const bool active = step < n_steps && !(key0 + strict > q0w + 31);
+        const bool active = step < n_steps && !(key0 + strict > q0w + 31) && q0w < job.len;
         if (g_pending && row_ok) *(float*)((char*)(rcur - 2 * tstride) + g_from_r) = Gstore;
         g_pending = false;
         const float F = Rnext;

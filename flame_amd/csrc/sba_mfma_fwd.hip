@@ -148,7 +148,8 @@ __global__ __launch_bounds__(kThreads) void mfma_fwd_kernel(KParams p) {
     for (; step >= 0; --step, buf ^= 1) {
         const char* ktile = lds + buf * 2 * kTile;
         const int key0 = step * kKeyBlock;
-        const bool skip = key0 + strict > q0w + 31;       // whole step right of this wave's last query
+        // whole step right of this wave's last query, or all of this wave's queries past the end of the sequence
+        const bool skip = key0 + strict > q0w + 31 || q0w >= job.len;
         open_step(step, buf, skip);
         if (!skip) {
             if (!fwd_step<D, kCarryOnly, true, D == 128>(ktile, ktile + kTile, lo, qf, oacc, R, lane, key0, q0w, qi, strict, carry_out)) {
@@ -163,7 +164,7 @@ __global__ __launch_bounds__(kThreads) void mfma_fwd_kernel(KParams p) {
     for (; step >= 0; --step, buf ^= 1) {
         const char* ktile = lds + buf * 2 * kTile;
         const int key0 = step * kKeyBlock;
-        const bool skip = key0 + strict > q0w + 31;
+        const bool skip = key0 + strict > q0w + 31 || q0w >= job.len;
         if (!redo) open_step(step, buf, skip);
         redo = false;
         if (!skip) {
