@@ -24,13 +24,13 @@ KERNEL_TIMING_SAMPLES = 5      # steps of the timed region whose kernels are tim
 # runs summarised under profiles/ (sba_cfg{2,3,4}_hbm_traffic.txt, sba_cfg{2,3,4}_shader_counters.txt) and
 # are reported with that source next to what this run measures itself.
 # HBM bytes per launch (FETCH_SIZE + WRITE_SIZE, scaled by a copy kernel of known size):
-PROFILED_HBM_BYTES = {("cfg2", "fwd"): 68866728, ("cfg2", "bwd_dq"): 83544130, ("cfg2", "bwd_dkv"): 86576018,
-                      ("cfg3", "fwd"): 996747649, ("cfg3", "bwd_dq"): 980689662, ("cfg3", "bwd_dkv"): 1124612953,
-                      ("cfg4", "fwd"): 819919850, ("cfg4", "bwd_dq"): 1669251269, ("cfg4", "bwd_dkv"): 1398555781}
+PROFILED_HBM_BYTES = {("cfg2", "fwd"): 68880405, ("cfg2", "bwd_dq"): 83539243, ("cfg2", "bwd_dkv"): 86576464,
+                      ("cfg3", "fwd"): 993377418, ("cfg3", "bwd_dq"): 1091328401, ("cfg3", "bwd_dkv"): 1125204967,
+                      ("cfg4", "fwd"): 817857184, ("cfg4", "bwd_dq"): 1671649641, ("cfg4", "bwd_dkv"): 1398538195}
 # wave instructions per launch: (vector incl. transcendental, transcendental, MFMA)
-PROFILED_INSTRUCTIONS = {("cfg2", "fwd"): (15223616, 2212864, 1064960), ("cfg2", "bwd_dq"): (27205633, 4334592, 1597440), ("cfg2", "bwd_dkv"): (31456637, 4334592, 2146304),
-                   ("cfg3", "fwd"): (123588912, 18619488, 9010688), ("cfg3", "bwd_dq"): (210976193, 36640864, 13516032), ("cfg3", "bwd_dkv"): (259319808, 35163264, 17564160),
-                   ("cfg4", "fwd"): (226951168, 34754560, 33685504), ("cfg4", "bwd_dq"): (404537345, 68440064, 50528256), ("cfg4", "bwd_dkv"): (516210688, 67272704, 67305472)}
+PROFILED_INSTRUCTIONS = {("cfg2", "fwd"): (15223616, 2212864, 1064960), ("cfg2", "bwd_dq"): (27205633, 4334592, 1597440), ("cfg2", "bwd_dkv"): (31456645, 4334592, 2146304),
+                   ("cfg3", "fwd"): (119268016, 17871840, 8648192), ("cfg3", "bwd_dq"): (204901281, 35168224, 12972288), ("cfg3", "bwd_dkv"): (259319808, 35163264, 17564160),
+                   ("cfg4", "fwd"): (226951168, 34754560, 33685504), ("cfg4", "bwd_dq"): (405098497, 68440064, 50528256), ("cfg4", "bwd_dkv"): (516210688, 67272704, 67305472)}
 # issue time of one SIMD per instruction, ns, four waves per SIMD (profiles/gfx950_issue_rates.txt): plain vector,
 # transcendental issued while MFMAs are in flight, MFMA 32x32x16 bf16.  MFMAs and plain vector instructions do not
 # overlap on gfx950, so their times add up.
