@@ -1681,6 +1681,15 @@ static bool own_keys_kernel(bool by_size) {
     return by_size;
 }
 
+// SBA_DQ_KERNEL=lean / =plain overrides the choice between the two arrangements of the one-step dQ kernel at
+// head_dim 64 (tests run both on the same inputs).
+static bool lean_dq_kernel(bool by_size) {
+    const char* e = getenv("SBA_DQ_KERNEL");
+    if (e && !strcmp(e, "lean")) return true;
+    if (e && !strcmp(e, "plain")) return false;
+    return by_size;
+}
+
 int sba_launch_mfma_bwd(const sba::KParams& kp_in, int phases, hipStream_t s) {
     using namespace sba;
     KParams kp = kp_in;
@@ -1704,7 +1713,7 @@ int sba_launch_mfma_bwd(const sba::KParams& kp_in, int phases, hipStream_t s) {
     if (kp.head_dim == 64) {
         // small grids last as long as their longest sweep: take the variant that halves it
         if (p1 && grid.x <= sba_two_step_max_grid()) hipLaunchKernelGGL((mfma_bwd_dq2_kernel<64>), grid, dim3(2 * kThreads), 0, s, kp);
-        else if (p1 && grid.x >= 8u * cus) hipLaunchKernelGGL((mfma_bwd_dq_kernel<64, true>), grid, dim3(kThreads), 0, s, kp);
+        else if (p1 && lean_dq_kernel(grid.x >= 8u * cus)) hipLaunchKernelGGL((mfma_bwd_dq_kernel<64, true>), grid, dim3(kThreads), 0, s, kp);
         else if (p1) hipLaunchKernelGGL((mfma_bwd_dq_kernel<64>), grid, dim3(kThreads), 0, s, kp);
         if (p2 && plain) {
             hipLaunchKernelGGL((mfma_bwd_dkv_kernel<64>), dim3(2 * grid.x), dim3(kThreads), 0, s, kp);

@@ -545,6 +545,17 @@ def test_randomized_packed_batches_mfma_vs_generic_backward(dkv_kernel, D, monke
             assert rel_l2(x.float(), y.float()) <= 5e-2
 
 
+@pytest.mark.parametrize("which", ["lean", "plain"])
+def test_both_arrangements_of_the_one_step_dq_kernel_against_the_oracle(which, monkeypatch):
+    # head_dim 64, grids above the two-step kernels' range: the library picks between the two arrangements of the
+    # dQ kernel by launch size; each is forced here on a packed and a dense problem (ragged ends, both masks)
+    # (every problem has more than 512 workgroups: 36, 36 and 17 row blocks times 16, 16 and 32 heads)
+    monkeypatch.setenv("SBA_DQ_KERNEL", which)
+    _check_varlen(16, 64, [300, 1, 129, 64, 517, 31, 1000, 128, 77, 640, 900], torch.bfloat16, False, seed=41)
+    _check_varlen(16, 64, [2100, 65, 2300], torch.bfloat16, True, seed=42)
+    _check_dense(4, 8, 2100, 64, torch.bfloat16, False, seed=43, in_scale=0.5)
+
+
 def test_seeded_random_sweep_of_shapes_layouts_and_dtypes_against_the_oracle():
     # 120 seeded draws over what the fixed cases above leave between them: batch and head counts,
     # lengths from 1 to 2 000 at and off the 64 / 128 block edges, head dims on the matrix-core
