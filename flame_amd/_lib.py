@@ -15,7 +15,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "csrc", "libsba_mi355x.so")
 
 SBA_DTYPE_F32, SBA_DTYPE_BF16 = 0, 1
-SBA_ABI_VERSION = 5
+SBA_ABI_VERSION = 6
 
 
 class SbaTensor(C.Structure):
@@ -78,6 +78,8 @@ def load() -> C.CDLL:
         lib.sba_bwd.argtypes = [C.POINTER(SbaParams)]
         lib.sba_bwd_static.restype = C.c_int
         lib.sba_bwd_static.argtypes = [C.POINTER(SbaParams)]
+        lib.sba_bwd_gave_up.restype = C.c_int
+        lib.sba_bwd_gave_up.argtypes = [C.POINTER(SbaParams), C.c_int, C.POINTER(C.c_int)]
         if lib.sba_abi_version() != SBA_ABI_VERSION:
             raise RuntimeError("libsba_mi355x.so ABI version mismatch; rebuild it")
         _lib = lib
@@ -86,7 +88,7 @@ def load() -> C.CDLL:
 
 EXPORTED_SYMBOLS = ("sba_abi_version", "sba_error_string", "sba_workspace_bytes", "sba_bwd_scratch_bytes",
                     "sba_build_schedule", "sba_row_block", "sba_table_columns", "sba_fwd", "sba_bwd",
-                    "sba_bwd_static")
+                    "sba_bwd_static", "sba_bwd_gave_up")
 
 STATIC_SCRATCH_BYTES = 64 << 20     # SBA_STATIC_SCRATCH_BYTES: what sba_bwd_static() holds per GPU
 
@@ -152,11 +154,64 @@ def empty_grads_like(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor):
     return torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
 
 
-def recompute_carries() -> bool:
-    """SBA_RECOMPUTE_CARRIES=1: keep nothing between forward and backward (the reference keeps one
-    float per query, the default here one carry table of H x T/64 x tokens floats); the backward
-    then repeats the forward's sweep for the carries alone, about 15 % more time per fwd + bwd."""
-    return os.environ.get("SBA_RECOMPUTE_CARRIES") == "1"
+# What a layer may keep from its forward to its backward (the forward's carry tables) before the operator
+# switches to the memory-lean mode by itself: the forward then keeps nothing and the backward repeats the
+# forward's sweep for the carries alone (bit-identical gradients, 12-13 % more time per forward + backward).
+# The reference keeps one float per query (sb_fwd.py:146); the tables grow with the square of the sequence
+# length: 17 MB at B=1, H=16, T=4096, 270 MB at T=16384, 4.3 GB for a dense 65 536-token row.
+DEFAULT_WORKSPACE_BUDGET = 128 << 20
+_workspace_budget = None            # set_workspace_budget(); None: SBA_WORKSPACE_BUDGET_MB or the default
+
+
+def set_workspace_budget(nbytes) -> None:
+    """Largest carry-table workspace (bytes) a forward may keep for its backward; larger ones are
+    recomputed in the backward instead.  None restores the default (SBA_WORKSPACE_BUDGET_MB megabytes if
+    that is set, else 128 MiB); 0 never keeps anything; float('inf') always keeps the tables."""
+    global _workspace_budget
+    _workspace_budget = nbytes
+
+
+def workspace_budget():
+    if _workspace_budget is not None:
+        return _workspace_budget
+    e = os.environ.get("SBA_WORKSPACE_BUDGET_MB")
+    return float(e) * (1 << 20) if e else DEFAULT_WORKSPACE_BUDGET
+
+
+def recompute_carries(workspace_nbytes: int = 0) -> bool:
+    """Whether the forward keeps nothing for the backward (which then recomputes the carries):
+    under SBA_RECOMPUTE_CARRIES=1 always, otherwise when the tables would exceed workspace_budget()."""
+    if os.environ.get("SBA_RECOMPUTE_CARRIES") == "1":
+        return True
+    return workspace_nbytes > workspace_budget()
+
+
+# Error word of the bf16 matrix-core backward (set if a kernel abandoned one of its bounded internal waits,
+# see sba_bwd_gave_up in include/sba_mi355x.h).  Reading it waits for the stream, so it is off by default:
+# SBA_CHECK_GAVE_UP=1 or check_gave_up(True) (the test-suite's GPU tests) make every backward read it and raise.
+_check_gave_up = None
+
+
+def check_gave_up(on) -> None:
+    global _check_gave_up
+    _check_gave_up = on
+
+
+def gave_up_checked() -> bool:
+    if _check_gave_up is not None:
+        return bool(_check_gave_up)
+    return os.environ.get("SBA_CHECK_GAVE_UP") == "1"
+
+
+def raise_if_gave_up(p, static_scratch_used: bool = False) -> None:
+    """Reads the error word of the backward just launched with `p` (waits for its stream) and raises if set."""
+    if torch.compiler.is_compiling() or torch.cuda.is_current_stream_capturing():
+        return
+    flag = C.c_int(0)
+    check(load().sba_bwd_gave_up(C.byref(p), int(static_scratch_used), C.byref(flag)), "sba_bwd_gave_up")
+    if flag.value != 0:
+        raise RuntimeError("stick-breaking attention backward: a kernel abandoned a bounded internal wait "
+                           "(error word set); the gradients of this call are invalid")
 
 
 def matrix_core_head_dim(t: torch.Tensor) -> int:

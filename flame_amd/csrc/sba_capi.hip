@@ -62,16 +62,24 @@ size_t generic_acc_bytes(const SbaParams* p) {
     return (b + 255) & ~(size_t)255;
 }
 
-constexpr size_t kErrorWordBytes = 256;     // tail of the MFMA backward's scratch: the error word
+constexpr size_t kErrorWordBytes = 256;     // tail of the bf16 matrix-core backward's scratch: the error word
 
-// Carry tables of the matrix-core path, four in all.  bf16: the forward writes two - the product of (1 - beta)
+// Carry tables of the matrix-core path.  bf16, four in all: the forward writes two - the product of (1 - beta)
 // entering the right 32 keys of every 64-key step (`rtab`) and the one entering its left 32 keys (`rmid`), so
 // that every lane of the backward starts its chain from its own carry - and the dQ pass the two prefix tables
-// (`gtab`, `gmid`).  fp32: the forward writes `rtab`, the dQ pass the other three.
+// (`gtab`, `gmid`).  fp32, two in all: the forward writes `rtab`, the dQ pass `gtab`.
 int forward_tables(const SbaParams* p) { return p->dtype == SBA_DTYPE_BF16 ? 2 : 1; }
+// tables in the backward's scratch: the dQ pass's own, plus the forward's when no workspace brings them
+int scratch_tables(const SbaParams* p) { return forward_tables(p) * (p->workspace ? 1 : 2); }
+// the bounded waits (and with them the error word) exist in the bf16 matrix-core backward only
+bool has_error_word(const SbaParams* p) { return use_mfma_bwd(p) && p->dtype == SBA_DTYPE_BF16; }
 
 sba::TensorArg cvt(const SbaTensor& t) { return sba::TensorArg{(char*)t.ptr, t.stride_b, t.stride_h, t.stride_t}; }
 sba::VectorArg cvt(const SbaVector& t) { return sba::VectorArg{(char*)t.ptr, t.stride_b, t.stride_h}; }
+
+// Largest token stride (elements) the matrix-core kernels take: 64 rows of it, in bytes of the wider
+// element type, stay below 2^31.
+constexpr int64_t kMaxTokenStride = (INT64_C(1) << 31) / (64 * 4) - 1;
 
 int check_common(const SbaParams* p) {
     if (!p) return SBA_ERR_NULL;
@@ -91,6 +99,8 @@ int check_common(const SbaParams* p) {
         for (const SbaTensor* t : {&p->q, &p->k, &p->v, &p->o, &p->d_o, &p->dq, &p->dk, &p->dv}) {
             if (!t->ptr) continue;          // presence is checked per direction
             if (((uintptr_t)t->ptr & 15) || (t->stride_b & per16) || (t->stride_h & per16) || (t->stride_t & per16)) return SBA_ERR_SHAPE;
+            // the tile copies address a 64-row tile with 32-bit byte offsets from its first row
+            if (t->stride_t < 0 || t->stride_t > kMaxTokenStride) return SBA_ERR_SHAPE;
         }
     }
     return SBA_OK;
@@ -127,13 +137,12 @@ KParams make_kparams(const SbaParams* p) {
     if (bs && use_mfma_bwd(p)) {
         int slot = 0;
         kp.gtab = (float*)(bs + tb * slot++);
-        if (!two) kp.rmid = (float*)(bs + tb * slot++);
-        kp.gmid = (float*)(bs + tb * slot++);
+        if (two) kp.gmid = (float*)(bs + tb * slot++);
         if (!p->workspace) {                       // the forward's tables, recomputed by sba_bwd
             if (two) kp.rmid = (float*)(bs + tb * slot++);
             kp.rtab = (float*)(bs + tb * slot++);
         }
-        kp.gave_up = (int*)(bs + tb * slot);
+        if (has_error_word(p)) kp.gave_up = (int*)(bs + tb * slot);
     } else if (bs) {
         kp.dkv32 = (float*)bs;
     }
@@ -168,7 +177,7 @@ const char* sba_error_string(int code) {
     switch (code) {
         case SBA_OK: return "ok";
         case SBA_ERR_NULL: return "a required pointer is NULL";
-        case SBA_ERR_SHAPE: return "bad shape: sizes must be positive, head_dim <= 128, dense total_tokens == seq_len; bf16 at head_dim 64 / 128 and fp32 at head_dim 64 need 16-byte aligned pointers and strides that are multiples of 16 bytes";
+        case SBA_ERR_SHAPE: return "bad shape: sizes must be positive, head_dim <= 128, dense total_tokens == seq_len; at head_dim 64 / 128 (the matrix-core kernels, bf16 and fp32) tensors need 16-byte aligned pointers, outer strides that are multiples of 16 bytes and a token stride below 2^23 elements";
         case SBA_ERR_DTYPE: return "unsupported dtype (float32 and bfloat16 only)";
         case SBA_ERR_WORKSPACE: return "workspace / bwd_scratch missing or smaller than sba_workspace_bytes() / sba_bwd_scratch_bytes()";
         case SBA_ERR_SCHEDULE: return "packed layout needs a row-block schedule from sba_build_schedule()";
@@ -189,7 +198,8 @@ size_t sba_bwd_scratch_bytes(const SbaParams* p) {
     if (!p || p->n_heads <= 0 || p->seq_len <= 0 || p->head_dim <= 0 || p->head_dim > 128) return 0;
     if (p->cu_seqlens && p->table_cols <= 0 && use_mfma_bwd(p)) return 0;
     // without a workspace the backward recomputes the forward's tables first, into slots of its own
-    return use_mfma_bwd(p) ? (p->workspace ? 4 - forward_tables(p) : 4) * table_bytes(p) + kErrorWordBytes : generic_acc_bytes(p);
+    if (!use_mfma_bwd(p)) return generic_acc_bytes(p);
+    return scratch_tables(p) * table_bytes(p) + (has_error_word(p) ? kErrorWordBytes : 0);
 }
 
 int sba_row_block(void) { return sba::kRowBlock; }
@@ -282,6 +292,27 @@ int sba_bwd(const SbaParams* p) {
     if (!use_mfma_bwd(p) && p->bwd_phases == 2) return SBA_OK;
     if (use_mfma_bwd(p) && p->dtype == SBA_DTYPE_F32) return sba_launch_mfma_f32_bwd(kp, p->bwd_phases, s);
     return use_mfma_bwd(p) ? sba_launch_mfma_bwd(kp, p->bwd_phases, s) : sba_launch_generic_bwd(kp, p->dtype, s);
+}
+
+int sba_bwd_gave_up(const SbaParams* p, int static_scratch_used, int* gave_up) {
+    if (!gave_up) return SBA_ERR_NULL;
+    *gave_up = 0;
+    int rc = check_common(p);
+    if (rc) return rc;
+    if (!has_error_word(p)) return SBA_OK;
+    void* bs = p->bwd_scratch;
+    if (static_scratch_used) {
+        rc = static_scratch(&bs);
+        if (rc) return rc;
+    }
+    if (!bs) return SBA_ERR_WORKSPACE;
+    const char* word = (const char*)bs + scratch_tables(p) * table_bytes(p);
+    hipStream_t s = (hipStream_t)p->stream;
+    int host = 0;
+    if (hipMemcpyAsync(&host, word, sizeof(int), hipMemcpyDeviceToHost, s) != hipSuccess) return SBA_ERR_LAUNCH;
+    if (hipStreamSynchronize(s) != hipSuccess) return SBA_ERR_LAUNCH;
+    *gave_up = host;
+    return SBA_OK;
 }
 
 int sba_bwd_static(const SbaParams* p) {

@@ -702,11 +702,7 @@ __global__ __launch_bounds__((NP + 4) * 64, NP == 4 ? 2 : 3) void mfma_bwd_dkv_s
                 const char* dotile = qtile + kQTile;
                 const int q0w = (cur.job.rb + it) * kRowBlock + 32 * w4;
                 const int qi = q0w + n;
-#ifdef SBA_EXP_IDLE_PRODUCERS
-                const bool skip = true;
-#else
                 const bool skip = key0 + strict > q0w + 31 || q0w >= len || key0 >= len;
-#endif
                 float x[16], beta[16], dp[16];
                 float Gt = 0.f;
                 if (!skip) {
@@ -1087,9 +1083,7 @@ __global__ __launch_bounds__((NP + 4) * 64, NP == 4 ? 2 : 3) void mfma_bwd_dkv_s
                 __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
                 request_keys(decode_item(p, nxt_idx), vtiles + ((item + 1) & 1) * kTile);
             }
-#ifndef SBA_EXP_IDLE_REDUCE
             if (s > 0) reduce(s - 1);
-#endif
             // B, only where a finished dK/dV is staged into the Z buffer just reduced: every
             // consumer must be through with it
             if (finish_after_reduce) {
@@ -1098,15 +1092,11 @@ __global__ __launch_bounds__((NP + 4) * 64, NP == 4 ? 2 : 3) void mfma_bwd_dkv_s
                 fin_store = fin_stage;
                 store_pending = true;
             }
-#ifndef SBA_EXP_NO_REQUEST
             deposit(s + 1);                    // requested at the end of the previous iteration
-#endif
             finish_after_reduce = last;
             if (last) fin_stage = cur_idx;
             __builtin_amdgcn_sched_barrier(0);
-#ifndef SBA_EXP_NO_REQUEST
             request_front();                   // step s + 2
-#endif
             wait_all_but_requests();
             __syncthreads();                   // A
             ++s;

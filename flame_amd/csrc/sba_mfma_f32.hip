@@ -380,6 +380,7 @@ int sba_launch_mfma_f32_fwd(const sba::KParams& kp, hipStream_t s) {
 
 int sba_launch_mfma_f32_bwd(const sba::KParams& kp, int phases, hipStream_t s) {
     using namespace sba;
+    if (!kp.rtab || !kp.gtab) return SBA_ERR_WORKSPACE;
     dim3 grid((unsigned)kp.n_jobs * kp.n_heads);
     if (kp.head_dim == 64) {
         if (phases != 2) hipLaunchKernelGGL((f32::bwd_dq_kernel<64>), grid, dim3(kThreads), 0, s, kp);

@@ -63,7 +63,8 @@ class SBAModel(SBAPreTrainedModel):
 
 
 class SBAForCausalLM(SBAPreTrainedModel):
-    _tied_weights_keys = ['lm_head.weight']
+    # target -> source, the form transformers 5 expects (a bare list of names fails in its tie_weights())
+    _tied_weights_keys = {'lm_head.weight': 'model.embeddings.weight'}
 
     def __init__(self, config: SBAConfig):
         super().__init__(config)

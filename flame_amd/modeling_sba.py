@@ -34,6 +34,8 @@ class SBAConfig:
     norm_eps: float = 1e-6
     vocab_size: int = 32000
     qkv_bias: bool = False
+    num_kv_heads: Optional[int] = None
+    window_size: Optional[int] = None
     tie_word_embeddings: bool = False
 
     def mlp_width(self) -> int:
@@ -99,7 +101,13 @@ class SBABlock(nn.Module):
     def __init__(self, cfg: SBAConfig, layer_idx: int):
         super().__init__()
         self.attn_norm = nn.RMSNorm(cfg.hidden_size, eps=cfg.norm_eps)
-        self.attn = SBA(hidden_size=cfg.hidden_size, num_heads=cfg.num_heads, qkv_bias=cfg.qkv_bias,
+        # every attention field the reference block forwards (modeling_sba.py:44-53): a num_kv_heads the layer
+        # cannot do raises there instead of silently building full multi-head attention
+        self.attn = SBA(hidden_size=cfg.hidden_size, num_heads=cfg.num_heads,
+                        num_kv_heads=getattr(cfg, "num_kv_heads", None), qkv_bias=cfg.qkv_bias,
+                        window_size=getattr(cfg, "window_size", None),
+                        rope_theta=getattr(cfg, "rope_theta", None),
+                        max_position_embeddings=getattr(cfg, "max_position_embeddings", None),
                         layer_idx=layer_idx)
         self.mlp_norm = nn.RMSNorm(cfg.hidden_size, eps=cfg.norm_eps)
         self.mlp = SBAMLP(cfg)

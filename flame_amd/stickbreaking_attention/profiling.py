@@ -68,6 +68,8 @@ def mark(name: str):
 def launch_bwd(lib, p):
     if not _on():
         _lib.check(lib.sba_bwd(C.byref(p)), "sba_bwd")
+        if _lib.gave_up_checked():
+            _lib.raise_if_gave_up(p)
         return
     mark("start")
     p.bwd_phases = 1
@@ -77,3 +79,5 @@ def launch_bwd(lib, p):
     _lib.check(lib.sba_bwd(C.byref(p)), "sba_bwd")
     mark("bwd_dkv")
     p.bwd_phases = 0
+    if _lib.gave_up_checked():
+        _lib.raise_if_gave_up(p)

@@ -87,8 +87,11 @@ def _compileable_backward(do: torch.Tensor, dr: Optional[torch.Tensor], q: torch
 def _fwd(q, k, v, logit_scale, attend_current=False, no_grad=False):
     o = torch.empty_like(q)              # same strides as q (sb_fwd.py:144 does the same)
     rem = torch.empty(q.shape[:-1], dtype=q.dtype, device=q.device)
-    keep = not (no_grad or _lib.recompute_carries())
-    nbytes = max(workspace_bytes(q), 16) if keep else 16
+    # above the workspace budget nothing is kept and the backward recomputes the carries (_lib.recompute_carries)
+    nbytes = 16 if no_grad else max(workspace_bytes(q), 16)
+    keep = not (no_grad or _lib.recompute_carries(nbytes))
+    if not keep:
+        nbytes = 16
     ws = torch.empty(nbytes, dtype=torch.uint8, device=q.device)
     _compileable_fwd(q, k, v, float(logit_scale), bool(attend_current), keep, o, rem, ws)
     return o, rem, ws

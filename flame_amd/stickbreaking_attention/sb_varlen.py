@@ -146,8 +146,11 @@ def _compileable_backward(do: torch.Tensor, dr: Optional[torch.Tensor], q: torch
 def varlen_fwd(q, k, v, cu_seqlens, max_seqlens, logit_scale, attend_current=False, no_grad=False):
     o = torch.empty_like(q)
     rem = torch.empty(q.shape[:-1], dtype=q.dtype, device=q.device)
-    keep = not (no_grad or _lib.recompute_carries())
-    nbytes = max(workspace_bytes(q, cu_seqlens, max_seqlens), 16) if keep else 16
+    # above the workspace budget nothing is kept and the backward recomputes the carries (_lib.recompute_carries)
+    nbytes = 16 if no_grad else max(workspace_bytes(q, cu_seqlens, max_seqlens), 16)
+    keep = not (no_grad or _lib.recompute_carries(nbytes))
+    if not keep:
+        nbytes = 16
     ws = torch.empty(nbytes, dtype=torch.uint8, device=q.device)
     _compileable_forward(q, k, v, cu_seqlens, int(max_seqlens), float(logit_scale), bool(attend_current),
                          keep, o, rem, ws)
@@ -203,14 +206,32 @@ class StickBreakingAttention(torch.autograd.Function):
         return (*(_lib.cut_head_dim(g, ctx.head_dim) for g in (dq, dk, dv)), None, None, None, None)
 
 
+# cu_seqlens without its leading 0 (the reference's inner convention) -> the tensor with the 0 in front, one per
+# source tensor and version, so that the 24 layers of a model that pass the same tensor share one schedule entry.
+_WITH_ZERO: dict = {}
+
+
+def _with_leading_zero(cu_seqlens: torch.Tensor) -> torch.Tensor:
+    if torch.compiler.is_compiling():
+        return torch.cat([cu_seqlens.new_zeros(1), cu_seqlens])
+    key = id(cu_seqlens)
+    hit = _WITH_ZERO.get(key)
+    if hit is not None and hit[0]() is cu_seqlens and hit[1] == cu_seqlens._version:
+        return hit[2]
+    full = torch.cat([cu_seqlens.new_zeros(1), cu_seqlens])
+    ref = weakref.ref(cu_seqlens, lambda _r, key=key: _WITH_ZERO.pop(key, None))
+    _WITH_ZERO[key] = (ref, cu_seqlens._version, full)
+    return full
+
+
 def sb_attn_varlen(q, k, v, cu_seqlens, max_seqlens, inv_temp=None, zero_start=True,
                    attend_current=False):
     """cu_seqlens with its leading 0 when zero_start (the default), document ends only
     otherwise, as in the reference (sb_varlen/__init__.py:71-78).  The kernels always work from
-    the form with the leading 0, and the schedule is cached per cu_seqlens tensor: pass the
-    same tensor to every layer."""
+    the form with the leading 0, and the schedule is cached per cu_seqlens tensor (for the form
+    without the 0 too: its zero-prefixed copy is made once per tensor): pass the same tensor to every layer."""
     if not zero_start:
-        cu_seqlens = torch.cat([cu_seqlens.new_zeros(1), cu_seqlens])
+        cu_seqlens = _with_leading_zero(cu_seqlens)
     if inv_temp is None:
         inv_temp = 1 / math.sqrt(q.size(-1))
     return _apply(q, k, v, cu_seqlens, max_seqlens, inv_temp, attend_current)
@@ -229,5 +250,4 @@ def _apply(q, k, v, cu_seqlens, max_seqlens, inv_temp, attend_current):
 def sb_attn_varlen_(q, k, v, inv_temp, cu_seqlens, max_seqlens, attend_current):
     """The reference's inner entry point (sb_varlen/__init__.py:81-82): cu_seqlens arrives with
     the leading 0 already stripped (document ends only)."""
-    cu_seqlens = torch.cat([cu_seqlens.new_zeros(1), cu_seqlens])
-    return _apply(q, k, v, cu_seqlens, max_seqlens, inv_temp, attend_current)
+    return _apply(q, k, v, _with_leading_zero(cu_seqlens), max_seqlens, inv_temp, attend_current)

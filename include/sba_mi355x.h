@@ -26,9 +26,10 @@
  *                          with cu_seqlens[0] == 0, stride_b = 0,
  *                          element (h,t,d) at    base + h*stride_h + t*stride_t + d
  * Strides are in elements; the innermost (D) stride is 1.  Problems at head_dim 64 / 128
- * (the matrix-core kernels) need 16-byte aligned tensor pointers and outer strides that are
- * multiples of 16 bytes - 8 bf16 or 4 fp32 elements - (SBA_ERR_SHAPE otherwise); rem / d_rem
- * are contiguous along tokens.
+ * (the matrix-core kernels) need 16-byte aligned tensor pointers, outer strides that are
+ * multiples of 16 bytes - 8 bf16 or 4 fp32 elements - and a token stride below 2^23 elements
+ * (the tile copies address a 64-row tile with 32-bit byte offsets); SBA_ERR_SHAPE otherwise.
+ * rem / d_rem are contiguous along tokens.
  */
 #ifndef SBA_MI355X_H
 #define SBA_MI355X_H
@@ -40,7 +41,7 @@
 extern "C" {
 #endif
 
-#define SBA_ABI_VERSION 5
+#define SBA_ABI_VERSION 6
 #define SBA_SCHEDULE_INTS 8   /* int32 per scheduled job, see sba_build_schedule() */
 #define SBA_DOC_MAJOR_GRID 8192 /* workgroups from which the schedule is document-major */
 
@@ -124,18 +125,18 @@ const char* sba_error_string(int code);
 size_t sba_workspace_bytes(const SbaParams* p);
 
 /*
- * Bytes of device memory sba_bwd needs for the duration of the call only (the tables that its
- * first kernel hands to its second - two in bf16, three in fp32 -, or the generic path's fp32
- * accumulators): allocate before
- * the call, free after it has run.  With bwd_phases 1 and 2 issued as two calls, the same
- * buffer goes to both.  For bf16 at head_dim 64 / 128 the last 256 bytes hold an error word
- * (int32): the backward clears it and sets it to 1 if a kernel abandoned one of its bounded
- * internal waits (the results are then invalid); a caller may read it after synchronising.
+ * Bytes of device memory sba_bwd needs for the duration of the call only (the prefix tables that
+ * its first kernel hands to its second - two in bf16, one in fp32 -, or the generic path's fp32
+ * accumulators): allocate before the call, free after it has run.  With bwd_phases 1 and 2 issued
+ * as two calls, the same buffer goes to both.  For bf16 at head_dim 64 / 128 the last 256 bytes
+ * hold an error word (int32): the first kernel of a backward (bwd_phases 0 or 1) clears it, and a
+ * kernel that abandoned one of its bounded internal waits sets it to 1 (the gradients are then
+ * invalid); a bwd_phases = 2 call leaves what phase 1 left.  sba_bwd_gave_up() reads it.
  *
  * Memory-lean mode: a forward run WITHOUT save_for_backward keeps nothing, and sba_bwd called
  * with workspace = NULL first repeats the forward's sweep for the carries alone (about 0.7 of
- * a forward) into further tables of the scratch; this function then asks for four tables in
- * all (it looks at whether p->workspace is NULL).
+ * a forward) into further tables of the scratch; this function then asks for twice as many
+ * tables (it looks at whether p->workspace is NULL).
  */
 size_t sba_bwd_scratch_bytes(const SbaParams* p);
 
@@ -177,6 +178,18 @@ int sba_fwd(const SbaParams* p);
 
 /* Backward: dq, dk, dv from d_o, d_rem, q, k, v and the forward's carry table. */
 int sba_bwd(const SbaParams* p);
+
+/*
+ * Error word of the last backward that ran on this problem's scratch: *gave_up = 1 if one of its
+ * kernels abandoned a bounded internal wait (its gradients are invalid), else 0.  `p` is the
+ * SbaParams of that backward (sizes, workspace, bwd_scratch, stream); pass static_scratch_used = 1
+ * after sba_bwd_static(), whose scratch the caller does not see.  Copies four bytes to the host on
+ * p->stream and WAITS for that stream: a debugging and testing aid, not for a training loop or a
+ * graph capture.  Problems without such waits (fp32, generic kernels) report 0 without a copy.
+ * The reference's counterpart is the spin lock of locked_add (sb_varlen/sb_varlen_bwd.py:13-52),
+ * which waits without bound and reports nothing.
+ */
+int sba_bwd_gave_up(const SbaParams* p, int static_scratch_used, int* gave_up);
 
 /*
  * Backward without any allocation.  No counterpart in the reference: it is for callers that

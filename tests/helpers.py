@@ -44,3 +44,15 @@ def rel_l2(a, b):
 
 def max_abs(a, b):
     return float((a.double() - b.double()).abs().max())
+
+
+# (label, quantity, error, tolerance) of every check made through within(): the test session writes them
+# out, worst first, when SBA_MARGINS_FILE names a file (see conftest.py), so that the distance of each
+# parity check from its tolerance can be tracked from one kernel change to the next.
+MARGINS = []
+
+
+def within(label, quantity, err, tol):
+    """assert err <= tol, and remember how close it came."""
+    MARGINS.append((label, quantity, float(err), float(tol)))
+    assert err <= tol, f"{label}: {quantity} error {err:.3e} exceeds {tol:.1e}"

@@ -30,7 +30,7 @@ def test_exports_every_declared_symbol(lib):
 
 
 def test_abi_version_and_struct_size(lib):
-    assert lib.sba_abi_version() == 5
+    assert lib.sba_abi_version() == 6
     p = _lib.SbaParams()
     p.struct_size = C.sizeof(_lib.SbaParams) - 8
     assert lib.sba_fwd(C.byref(p)) == -7          # SBA_ERR_ABI, before anything touches a GPU
@@ -74,6 +74,9 @@ def test_error_codes_of_the_call_sequence_without_gpu(lib):
     assert lib.sba_fwd(C.byref(p)) == -2
     p.q.ptr, p.k.stride_t = 256, 68                           # stride not a multiple of 8 elements
     assert lib.sba_fwd(C.byref(p)) == -2
+    p.k.stride_t = 1 << 23                                    # beyond the 32-bit tile addressing
+    assert lib.sba_fwd(C.byref(p)) == -2
+    assert b"token stride" in lib.sba_error_string(-2)
     p.k.stride_t = 64
     p.cu_seqlens = 256                                        # packed layout ...
     assert lib.sba_fwd(C.byref(p)) == -5                      # ... without a schedule: SBA_ERR_SCHEDULE
@@ -98,9 +101,9 @@ def test_workspace_bytes(lib):
     p.workspace = None
     p.dtype = _lib.SBA_DTYPE_F32                    # fp32 at head_dim 64 runs on the matrix cores too: one table from the forward
     assert lib.sba_workspace_bytes(C.byref(p)) == table
-    assert lib.sba_bwd_scratch_bytes(C.byref(p)) == 4 * table + 256
+    assert lib.sba_bwd_scratch_bytes(C.byref(p)) == 2 * table      # the forward's table again and the dQ pass's; no bounded waits, no error word
     p.workspace = 1
-    assert lib.sba_bwd_scratch_bytes(C.byref(p)) == 3 * table + 256
+    assert lib.sba_bwd_scratch_bytes(C.byref(p)) == table
     p.workspace = None
     p.head_dim = 128                                # and at head_dim 128
     assert lib.sba_workspace_bytes(C.byref(p)) == table
@@ -121,6 +124,60 @@ def test_static_backward_refuses_oversize_without_gpu(lib):
     assert lib.sba_bwd_scratch_bytes(C.byref(p)) > _lib.STATIC_SCRATCH_BYTES
     assert lib.sba_bwd_static(C.byref(p)) == -8
     assert b"sba_bwd_static" in lib.sba_error_string(-8)
+
+
+def test_gave_up_helper_without_gpu(lib):
+    # argument checks come first; problems without bounded waits (fp32, generic kernels) report 0 without a copy
+    flag = C.c_int(7)
+    assert lib.sba_bwd_gave_up(None, 0, C.byref(flag)) == -1
+    p = _lib.SbaParams()
+    p.struct_size = C.sizeof(_lib.SbaParams)
+    p.dtype = _lib.SBA_DTYPE_F32
+    p.n_seq, p.n_heads, p.seq_len, p.total_tokens, p.head_dim = 1, 2, 256, 256, 64
+    for t in ("q", "k", "v"):
+        getattr(p, t).ptr = 256
+        getattr(p, t).stride_h, getattr(p, t).stride_t = 256 * 64, 64
+    assert lib.sba_bwd_gave_up(C.byref(p), 0, None) == -1
+    assert lib.sba_bwd_gave_up(C.byref(p), 0, C.byref(flag)) == 0 and flag.value == 0
+    p.dtype, p.head_dim = _lib.SBA_DTYPE_BF16, 96          # generic kernels
+    flag.value = 7
+    assert lib.sba_bwd_gave_up(C.byref(p), 0, C.byref(flag)) == 0 and flag.value == 0
+    p.head_dim = 64                                        # bf16 matrix-core path: needs the scratch it is to read
+    assert lib.sba_bwd_gave_up(C.byref(p), 0, C.byref(flag)) == -4
+
+
+def test_python_raises_when_the_error_word_is_set(lib, monkeypatch):
+    # the Python side of the check, with the library call replaced (no test makes a kernel's wait expire)
+    calls = []
+
+    class Fake:
+        def sba_bwd_gave_up(self, p, static_used, flag):
+            calls.append(static_used)
+            flag._obj.value = 1
+            return 0
+    monkeypatch.setattr(_lib, "load", lambda: Fake())
+    monkeypatch.setattr(torch.cuda, "is_current_stream_capturing", lambda: False)
+    with pytest.raises(RuntimeError, match="abandoned a bounded internal wait"):
+        _lib.raise_if_gave_up(_lib.SbaParams(), static_scratch_used=True)
+    assert calls == [1]
+
+
+def test_workspace_budget_switch(monkeypatch):
+    monkeypatch.delenv("SBA_RECOMPUTE_CARRIES", raising=False)
+    monkeypatch.delenv("SBA_WORKSPACE_BUDGET_MB", raising=False)
+    _lib.set_workspace_budget(None)
+    assert _lib.workspace_budget() == 128 << 20
+    assert not _lib.recompute_carries(17 << 20)            # B=1, H=16, T=4096: kept
+    assert _lib.recompute_carries(270 << 20)               # T=16384: recomputed
+    monkeypatch.setenv("SBA_WORKSPACE_BUDGET_MB", "512")
+    assert not _lib.recompute_carries(270 << 20)
+    _lib.set_workspace_budget(0)
+    assert _lib.recompute_carries(16)
+    _lib.set_workspace_budget(float("inf"))
+    assert not _lib.recompute_carries(1 << 40)
+    monkeypatch.setenv("SBA_RECOMPUTE_CARRIES", "1")
+    assert _lib.recompute_carries(0)
+    _lib.set_workspace_budget(None)
 
 
 def test_schedule_builder(lib):

@@ -11,7 +11,7 @@ import torch
 
 from oracle import sb_oracle as O
 from oracle import c_oracle
-from helpers import max_abs, rel_l2
+from helpers import max_abs, rel_l2, within
 
 GOLDEN = sorted(glob.glob(os.path.join(os.path.dirname(__file__), "golden", "sb_*.npz")))
 OUTPUTS = ("o", "rem", "dq", "dk", "dv")
@@ -76,11 +76,11 @@ def test_hip_operator_reproduces_golden_vectors(path, dtype):
         o, rem = sb_attn_varlen(q, k, v, cu.cuda(), max(lens), scale, attend_current=ac)
     loss = (o.float() * t["do"].float().cuda()).sum() + (rem.float() * t["drem"].float().cuda()).sum()
     loss.backward()
-    assert max_abs(o.float().cpu(), t["o"]) <= fwd_tol
-    assert max_abs(rem.float().cpu(), t["rem"]) <= fwd_tol
+    label = f"golden {os.path.basename(path)} {'bf16' if dtype == torch.bfloat16 else 'fp32'}"
+    within(label, "o", max_abs(o.float().cpu(), t["o"]), fwd_tol)
+    within(label, "rem", max_abs(rem.float().cpu(), t["rem"]), fwd_tol)
     for name, g in (("dq", q.grad), ("dk", k.grad), ("dv", v.grad)):
-        err = rel_l2(g.float().cpu(), t[name])
-        assert err <= grad_tol, f"{name} rel-L2 {err}"
+        within(label, name, rel_l2(g.float().cpu(), t[name]), grad_tol)
 
 
 # ---- matrix-core shapes: full forward, gradients along random directions ----
@@ -119,7 +119,7 @@ def test_oracle_reproduces_directional_vectors(path):
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["fp32", "bf16"])
 @pytest.mark.parametrize("path", DIRECTIONAL, ids=os.path.basename)
 def test_hip_operator_reproduces_directional_vectors(path, dtype):
-    # bf16 at D = 64 / 128 runs the matrix-core kernels, fp32 the generic ones
+    # D = 64 / 128: the matrix-core kernels in both dtypes (bf16 and fp32 MFMA)
     from flame_amd import sb_attn, sb_attn_varlen
     t, cu, scale, ac = _load_directional(path)
     print(f"golden {os.path.basename(path)} {dtype}", flush=True)
@@ -132,8 +132,9 @@ def test_hip_operator_reproduces_directional_vectors(path, dtype):
         o, rem = sb_attn_varlen(q, k, v, cu.cuda(), max(lens), scale, attend_current=ac)
     loss = (o.float() * t["do"].float().cuda()).sum() + (rem.float() * t["drem"].float().cuda()).sum()
     loss.backward()
-    assert max_abs(o.detach().float().cpu(), t["o"]) <= fwd_tol
-    assert max_abs(rem.detach().float().cpu(), t["rem"]) <= fwd_tol
+    label = f"golden {os.path.basename(path)} {'bf16' if dtype == torch.bfloat16 else 'fp32'}"
+    within(label, "o", max_abs(o.detach().float().cpu(), t["o"]), fwd_tol)
+    within(label, "rem", max_abs(rem.detach().float().cpu(), t["rem"]), fwd_tol)
     grads = [g.detach().float().cpu() for g in (q.grad, k.grad, v.grad)]
     got = _slopes(grads, t["directions"])
     for i, name in enumerate(("dq", "dk", "dv")):
@@ -144,4 +145,4 @@ def test_hip_operator_reproduces_directional_vectors(path, dtype):
             bound = grad_tol * float(grads[i].double().norm()) * float(u.norm()) / math.sqrt(u.numel())
             err = abs(float(got[i, n] - t["slopes"][i, n]))
             print(f"  {name}[{n}] slope {float(t['slopes'][i, n]):+.5f} error {err:.2e} bound {bound:.2e}", flush=True)
-            assert err <= bound, (name, n)
+            within(label, name, err, bound)

@@ -176,3 +176,38 @@ def test_hf_auto_model_from_config_trains_one_step_on_the_gpu():
     # and the dense route
     with torch.autocast("cuda", dtype=torch.bfloat16):
         assert torch.isfinite(model(input_ids=ids.view(2, 192), labels=ids.view(2, 192)).loss)
+
+
+def test_hf_auto_model_loss_matches_oracle_attention_packed_and_dense():
+    # the HF route held to the oracle like the plain model is: AutoModelForCausalLM.from_config on the GPU
+    # (HIP operator, bf16 autocast) against the same weights with the CPU oracle as attention (fp32)
+    from transformers import AutoModelForCausalLM
+    import flame_amd.hf as hf
+    torch.manual_seed(0)
+    cfg = hf.SBAConfig(hidden_size=256, num_hidden_layers=2, num_heads=4, vocab_size=512)
+    ref = AutoModelForCausalLM.from_config(cfg)
+    for layer in ref.model.layers:
+        layer.attn.attn_fn = lambda q, k, v, t: O.sb_attn_oracle(q, k, v)
+        layer.attn.attn_varlen_fn = lambda q, k, v, cu, ml: O.sb_attn_varlen_oracle(q, k, v, cu)
+    gpu = AutoModelForCausalLM.from_config(cfg)
+    gpu.load_state_dict(ref.state_dict())
+    gpu.cuda()
+    ids = torch.randint(0, 512, (1, 384))
+    cu = torch.tensor([0, 100, 101, 300, 384], dtype=torch.int32)
+    out_ref = ref(input_ids=ids, labels=ids, cu_seqlens=cu)
+    out_ref_dense = ref(input_ids=ids.view(2, 192), labels=ids.view(2, 192))
+    with torch.autocast("cuda", dtype=torch.bfloat16):
+        out = gpu(input_ids=ids.cuda(), labels=ids.cuda(), cu_seqlens=cu.cuda(), max_seqlen=199)
+        out_dense = gpu(input_ids=ids.view(2, 192).cuda(), labels=ids.view(2, 192).cuda())
+    print("hf vs oracle: packed", float(out.loss), float(out_ref.loss), "dense", float(out_dense.loss), float(out_ref_dense.loss), flush=True)
+    assert abs(float(out.loss) - float(out_ref.loss)) <= 2e-2
+    assert abs(float(out_dense.loss) - float(out_ref_dense.loss)) <= 2e-2
+    assert max_abs(out.logits.float().cpu(), out_ref.logits) <= 5e-2
+    assert max_abs(out_dense.logits.float().cpu(), out_ref_dense.logits) <= 5e-2
+    # the gradients of the attention projections against the oracle's (the operator's backward on this route)
+    out.loss.backward()
+    out_ref.loss.backward()
+    for name in ("q_proj", "k_proj", "v_proj", "o_proj"):
+        g = getattr(gpu.model.layers[0].attn, name).weight.grad.float().cpu()
+        r = getattr(ref.model.layers[0].attn, name).weight.grad
+        assert rel_l2(g, r) <= 5e-2, name

@@ -129,6 +129,39 @@ def test_kv_heads_must_equal_heads():
     from flame_amd.sba_layer import SBA
     with pytest.raises(ValueError):
         SBA(hidden_size=64, num_heads=4, num_kv_heads=2)
+    # the blocks forward the field (modeling_sba.py:44-53 of the reference does): a config that asks for
+    # grouped keys raises instead of silently building full multi-head attention
+    with pytest.raises(ValueError):
+        SBAForCausalLM(SBAConfig(hidden_size=64, num_hidden_layers=1, num_heads=4, num_kv_heads=2, vocab_size=11))
+    import flame_amd.hf as hf
+    from transformers import AutoModelForCausalLM
+    with pytest.raises(ValueError):
+        AutoModelForCausalLM.from_config(hf.SBAConfig(hidden_size=64, num_hidden_layers=1, num_heads=4, num_kv_heads=2,
+                                                      vocab_size=11))
+    blk = SBAForCausalLM(SBAConfig(hidden_size=64, num_hidden_layers=1, num_heads=4, num_kv_heads=4, window_size=77,
+                                   vocab_size=11)).model.layers[0]
+    assert blk.attn.num_kv_heads == 4 and blk.attn.window_size == 77      # kept, as the reference layer keeps it
+
+
+def test_hf_tied_word_embeddings(tmp_path):
+    # transformers 5 wants the tie declared as {target: source}; a bare list of names fails in from_config
+    import flame_amd.hf as hf
+    from transformers import AutoModelForCausalLM
+    cfg = hf.SBAConfig(hidden_size=64, num_hidden_layers=2, num_heads=2, vocab_size=97, tie_word_embeddings=True)
+    lm = AutoModelForCausalLM.from_config(cfg)
+    assert lm.lm_head.weight.data_ptr() == lm.model.embeddings.weight.data_ptr()
+    n_tied = sum(p.numel() for p in lm.parameters())
+    cfg_untied = hf.SBAConfig(hidden_size=64, num_hidden_layers=2, num_heads=2, vocab_size=97)
+    untied = AutoModelForCausalLM.from_config(cfg_untied)
+    assert untied.lm_head.weight.data_ptr() != untied.model.embeddings.weight.data_ptr()
+    assert sum(p.numel() for p in untied.parameters()) == n_tied + 97 * 64
+    lm.save_pretrained(tmp_path)
+    back = AutoModelForCausalLM.from_pretrained(tmp_path)
+    assert torch.equal(back.lm_head.weight, lm.lm_head.weight)
+    assert back.lm_head.weight.data_ptr() == back.model.embeddings.weight.data_ptr()
+    # the plain model ties the same way
+    plain = SBAForCausalLM(SBAConfig(hidden_size=64, num_hidden_layers=1, num_heads=2, vocab_size=97, tie_word_embeddings=True))
+    assert plain.lm_head.weight is plain.model.embeddings.weight
 
 
 def test_cu_seqlens_from_bos():
@@ -156,14 +189,15 @@ def test_context_len_rechunking():
 def test_hf_registration_and_340m_config_values():
     # custom_models/sba/__init__.py:7-9: importing the package registers model_type 'sba'
     import json
+    import os
     from transformers import AutoConfig, AutoModel, AutoModelForCausalLM
     import flame_amd.hf as hf
-    # the values of the reference's configs/sba_340m.json (the file itself is not part of this tree)
-    sba_340m = {"attention_bias": False, "bos_token_id": 1, "eos_token_id": 2, "fuse_cross_entropy": True,
-                "fuse_norm": True, "hidden_act": "swish", "hidden_size": 1024, "initializer_range": 0.006,
-                "max_position_embeddings": 8192, "model_type": "sba", "num_heads": 16, "num_hidden_layers": 24,
-                "norm_eps": 1e-06, "tie_word_embeddings": False, "use_cache": True, "vocab_size": 32000}
-    cfg = AutoConfig.for_model(**json.loads(json.dumps(sba_340m)))
+    # the values of the reference's configs/sba_340m.json, read from that file by tests/golden/make_config_fixture.py
+    fixture = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "sba_340m_config.json")
+    sba_340m = json.load(open(fixture))
+    cfg = AutoConfig.for_model(**sba_340m)
+    for key, value in sba_340m.items():        # every value of the file arrives in the config object
+        assert getattr(cfg, key) == value, key
     assert isinstance(cfg, hf.SBAConfig) and cfg.model_type == "sba"
     assert (cfg.hidden_size, cfg.num_heads, cfg.num_hidden_layers, cfg.vocab_size) == (1024, 16, 24, 32000)
     assert cfg.mlp_width() == 2816 and cfg.hidden_ratio == 4 and cfg.norm_eps == 1e-6

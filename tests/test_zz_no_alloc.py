@@ -66,6 +66,7 @@ def _run_both(shape, dtype, seed, lens=None, keep_table=True):
             p.bwd_scratch, p.bwd_scratch_bytes = None, 0      # ignored by the static entry point
         _lib.check(entry(C.byref(p)), entry.__name__)
         torch.cuda.synchronize()
+        _lib.raise_if_gave_up(p, static_scratch_used=entry is lib.sba_bwd_static)      # the error word of this call
         out.append((dq, dk, dv))
     return out
 
