@@ -288,4 +288,5 @@ def bwd_scratch_upper_bound(n_heads: int, columns: int, tab_tokens: int, head_di
     """Four tables (the recompute mode's count) or the generic path's fp32 dk|dv accumulators."""
     dp = 32 if head_dim <= 32 else (64 if head_dim <= 64 else 128)
     acc = (2 * tab_tokens * n_heads * dp * 4 + 255) & ~255
-    return max(4 * table_bytes(n_heads, columns) + 256, acc)      # + the backward's error word
+    scaled_q = (tab_tokens * n_heads * 64 * 2 + 255) & ~255      # bf16 at head_dim 64: the dQ pass's scaled copy of q
+    return max(4 * table_bytes(n_heads, columns) + scaled_q + 256, acc)      # + the backward's error word

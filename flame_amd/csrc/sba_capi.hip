@@ -73,6 +73,13 @@ int forward_tables(const SbaParams* p) { return p->dtype == SBA_DTYPE_BF16 ? 2 :
 int scratch_tables(const SbaParams* p) { return forward_tables(p) * (p->workspace ? 1 : 2); }
 // the bounded waits (and with them the error word) exist in the bf16 matrix-core backward only
 bool has_error_word(const SbaParams* p) { return use_mfma_bwd(p) && p->dtype == SBA_DTYPE_BF16; }
+// bf16 at head_dim 64: the dQ pass leaves a copy of q times the logit scale (bf16, [sequence][head][token][64], dense)
+// behind the tables, for the key-owner stream kernel, whose score MFMAs then deliver base-2 logits
+size_t scaled_q_bytes(const SbaParams* p) {
+    if (!use_mfma_bwd(p) || p->dtype != SBA_DTYPE_BF16 || p->head_dim != 64) return 0;
+    size_t b = (size_t)tab_tokens(p) * p->n_heads * 64 * 2;
+    return (b + 255) & ~(size_t)255;
+}
 
 sba::TensorArg cvt(const SbaTensor& t) { return sba::TensorArg{(char*)t.ptr, t.stride_b, t.stride_h, t.stride_t}; }
 sba::VectorArg cvt(const SbaVector& t) { return sba::VectorArg{(char*)t.ptr, t.stride_b, t.stride_h}; }
@@ -142,7 +149,13 @@ KParams make_kparams(const SbaParams* p) {
             if (two) kp.rmid = (float*)(bs + tb * slot++);
             kp.rtab = (float*)(bs + tb * slot++);
         }
-        if (has_error_word(p)) kp.gave_up = (int*)(bs + tb * slot);
+        char* tail = bs + tb * slot;
+        if (scaled_q_bytes(p)) {
+            const int64_t per_head = (p->cu_seqlens ? (int64_t)p->total_tokens : (int64_t)p->seq_len) * 64;
+            kp.q_scaled = sba::TensorArg{tail, p->cu_seqlens ? 0 : per_head * p->n_heads, per_head, 64};
+            tail += scaled_q_bytes(p);
+        }
+        if (has_error_word(p)) kp.gave_up = (int*)tail;
     } else if (bs) {
         kp.dkv32 = (float*)bs;
     }
@@ -199,7 +212,7 @@ size_t sba_bwd_scratch_bytes(const SbaParams* p) {
     if (p->cu_seqlens && p->table_cols <= 0 && use_mfma_bwd(p)) return 0;
     // without a workspace the backward recomputes the forward's tables first, into slots of its own
     if (!use_mfma_bwd(p)) return generic_acc_bytes(p);
-    return scratch_tables(p) * table_bytes(p) + (has_error_word(p) ? kErrorWordBytes : 0);
+    return scratch_tables(p) * table_bytes(p) + scaled_q_bytes(p) + (has_error_word(p) ? kErrorWordBytes : 0);
 }
 
 int sba_row_block(void) { return sba::kRowBlock; }
@@ -306,7 +319,7 @@ int sba_bwd_gave_up(const SbaParams* p, int static_scratch_used, int* gave_up) {
         if (rc) return rc;
     }
     if (!bs) return SBA_ERR_WORKSPACE;
-    const char* word = (const char*)bs + scratch_tables(p) * table_bytes(p);
+    const char* word = (const char*)bs + scratch_tables(p) * table_bytes(p) + scaled_q_bytes(p);
     hipStream_t s = (hipStream_t)p->stream;
     int host = 0;
     if (hipMemcpyAsync(&host, word, sizeof(int), hipMemcpyDeviceToHost, s) != hipSuccess) return SBA_ERR_LAUNCH;

@@ -27,6 +27,20 @@
 
 namespace sba {
 
+// The dQ pass leaves its pre-scaled Q fragments (q times scale * log2 e, rounded to bf16: the operand every
+// row-owner kernel multiplies with) behind for the key-owner stream kernel, which then needs no scaling of its
+// own and sees bit for bit the logits that the forward's carries were made from.  Row qi of q_scaled gets this
+// lane's four 16-byte chunks (columns 16 ks + 8 h ..).  head_dim 64 only, and only where the launcher asks for it.
+template <int D>
+__device__ inline void store_scaled_q(const KParams& p, const Job& job, int head, int qi, int lane,
+                                      const bf16x8 (&qf)[D / 16]) {
+    if (D != 64 || !p.q_scaled.ptr || qi >= job.len) return;
+    char* row = p.q_scaled.ptr + 2 * ((int64_t)job.seq * p.q_scaled.sb + (int64_t)head * p.q_scaled.sh +
+                                      (int64_t)(job.tok0 + qi) * p.q_scaled.st + 8 * (lane >> 5));
+#pragma unroll
+    for (int ks = 0; ks < D / 16; ++ks) *(u32x4*)(row + 32 * ks) = __builtin_bit_cast(u32x4, qf[ks]);
+}
+
 // ---------------------------------------------------------------- pass 1: dQ + prefix table
 // kLean (head_dim 64): the register-lean arrangement of the step that head_dim 128 always uses, held to three waves
 // per SIMD.  Ahead on large launches, whose SIMDs it fills better (the packed benchmark's dQ -5.6 %, short documents
@@ -58,6 +72,7 @@ __global__ __launch_bounds__(kThreads, (D == 64 && kLean) ? 3 : 2) void mfma_bwd
     bf16x8 qf[D / 16], dof[D / 16];
     load_row_frags<D>(qf, p.q, qbase, qi, job.len, lane);
     prescale_frags(qf, p.scale2);          // the score MFMAs then deliver base-2 logits
+    store_scaled_q<D>(p, job, head, qi, lane, qf);
     load_row_frags<D>(dof, p.d_o, dobase, qi, job.len, lane);
     float dr = 0.f;
     if (row_ok && p.d_rem.ptr)
@@ -240,6 +255,7 @@ __global__ __launch_bounds__(2 * kThreads, 2) void mfma_bwd_dq2_kernel(KParams p
     bf16x8 qf[D / 16], dof[D / 16];
     load_row_frags<D>(qf, p.q, qbase, qi, job.len, lane);
     prescale_frags(qf, p.scale2);          // the score MFMAs then deliver base-2 logits
+    if (grp == 0) store_scaled_q<D>(p, job, head, qi, lane, qf);
     load_row_frags<D>(dof, p.d_o, dobase, qi, job.len, lane);
     float dr = 0.f;
     if (row_ok && p.d_rem.ptr)
@@ -673,10 +689,7 @@ __global__ __launch_bounds__((NP + 4) * 64, NP == 4 ? 2 : 3) void mfma_bwd_dkv_s
         __syncthreads();                       // first item's tiles and carries visible
         int s = 0;
         bool staged_prev = false;              // the consumers staged a dK/dV in the previous iteration
-        // the logit scale in a VECTOR register: a multiply with a scalar-register operand takes a whole
-        // quad-cycle, one on vector registers half of that
-        float scale2v = p.scale2;
-        asm volatile("" : "+v"(scale2v));
+        // (no logit scale here: the Q tiles hold q times scale * log2 e, see store_scaled_q)
         if constexpr (NP == 8) {
         const int kh = wave >> 2;              // this wave's half of the 64-key block
         for (int item = 0;; ++item) {
@@ -721,7 +734,7 @@ __global__ __launch_bounds__((NP + 4) * 64, NP == 4 ? 2 : 3) void mfma_bwd_dkv_s
 #pragma unroll
                     for (int ks = 0; ks < D / 16; ++ks) acc = mfma(kfr[ks], qf[ks], acc);
 #pragma unroll
-                    for (int r = 0; r < 16; ++r) x[r] = acc[r] * scale2v;
+                    for (int r = 0; r < 16; ++r) x[r] = acc[r];
                     if (key0 + 31 + strict > q0w || q0w + 31 >= len) {        // diagonal or ragged tile
                         const int nvis = qi < len ? qi - strict - (key0 + 16 * h) + 1 : 0;
 #pragma unroll
@@ -823,7 +836,7 @@ __global__ __launch_bounds__((NP + 4) * 64, NP == 4 ? 2 : 3) void mfma_bwd_dkv_s
 #pragma unroll
                     for (int t = 0; t < 2; ++t)
 #pragma unroll
-                        for (int r = 0; r < 16; ++r) x[16 * t + r] = raw[t][r] * scale2v;
+                        for (int r = 0; r < 16; ++r) x[16 * t + r] = raw[t][r];
                     if (key0 + 63 + strict > q0w) mask_step(x, key0 + 32 * h, qi, strict);
                     // dP = dO V^T does not depend on the weights: its eight MFMAs go between the
                     // segments of the chain, where the chain's exp/rcp overlap them
@@ -913,7 +926,7 @@ __global__ __launch_bounds__((NP + 4) * 64, NP == 4 ? 2 : 3) void mfma_bwd_dkv_s
         };
         auto item_ptrs = [&](const KeyItem& t) {
             ItemPtrs r;
-            const TensorArg& xt = is_dv ? p.d_o : p.q;
+            const TensorArg& xt = is_dv ? p.d_o : p.q_scaled;      // Q as the dQ pass left it: times scale * log2 e
             r.x = xt.ptr + 2 * ((int64_t)t.job.seq * xt.sb + (int64_t)t.head * xt.sh + (int64_t)t.job.tok0 * xt.st) + cch * 16;
             const int64_t tk = tab_index(p, t.head, t.job, 0, t.kb);
             r.rt = p.rtab + tk;
@@ -926,7 +939,7 @@ __global__ __launch_bounds__((NP + 4) * 64, NP == 4 ? 2 : 3) void mfma_bwd_dkv_s
             asm volatile("" : "+v"(r.rm), "+v"(r.gm));
             return r;
         };
-        const uint32_t x_st2 = 2u * (uint32_t)(is_dv ? p.d_o.st : p.q.st);
+        const uint32_t x_st2 = 2u * (uint32_t)(is_dv ? p.d_o.st : p.q_scaled.st);
         auto request_step = [&](const ItemPtrs& t, int row0) {
             const int qi = min(row0 + (ct & (kRowBlock - 1)), t.len - 1);
             const int qb = qi >> 7;            // row block of the query: its slab starts qb*(qb+1) columns in
@@ -989,7 +1002,8 @@ __global__ __launch_bounds__((NP + 4) * 64, NP == 4 ? 2 : 3) void mfma_bwd_dkv_s
         auto stage = [&](char* staging) {
 #pragma unroll
             for (int kh = 0; kh < 2; ++kh) {
-                stage_acc_tile<D>(staging + (is_dv ? kTile : 0), 32 * kh, 32 * dbw, acc[kh], is_dv ? 1.0f : p.scale, lane);
+                // the Q rows carried scale * log2 e: dK = scale * dZ^T Q = (scale / scale2) * the sum
+                stage_acc_tile<D>(staging + (is_dv ? kTile : 0), 32 * kh, 32 * dbw, acc[kh], is_dv ? 1.0f : p.scale / p.scale2, lane);
                 acc[kh] = f32x16{0};
             }
         };
@@ -1700,6 +1714,10 @@ int sba_launch_mfma_bwd(const sba::KParams& kp_in, int phases, hipStream_t s) {
     // the stream with eight half-block producers (12 waves): measured within 1 % of the one with four
     // full-block producers (109.1 against 110.3 us at B=1 H=16 T=4096), which stays the default
     const bool stream8 = which && !strcmp(which, "stream8");
+    // the scaled copy of q is for the stream kernel: no other key-owner kernel reads it, so the dQ pass skips it
+    const bool stream = kp.head_dim == 64 && !plain && !own;
+    if (stream && !kp.q_scaled.ptr) return SBA_ERR_WORKSPACE;
+    if (!stream) kp.q_scaled.ptr = nullptr;
     if (kp.head_dim == 64) {
         // small grids last as long as their longest sweep: take the variant that halves it
         if (p1 && grid.x <= sba_two_step_max_grid()) hipLaunchKernelGGL((mfma_bwd_dq2_kernel<64>), grid, dim3(2 * kThreads), 0, s, kp);

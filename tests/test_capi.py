@@ -95,9 +95,10 @@ def test_workspace_bytes(lib):
     table = 16 * 32 * 33 * 128 * 4
     # bf16: the forward hands two tables to the backward (the carries entering the right and the left half of every 64-key step)
     assert lib.sba_workspace_bytes(C.byref(p)) == 2 * table
-    assert lib.sba_bwd_scratch_bytes(C.byref(p)) == 4 * table + 256    # no workspace: the backward recomputes those tables (+ error word)
+    scaled_q = 16 * 4096 * 64 * 2                   # head_dim 64: the dQ pass's copy of q times the logit scale, for the dK/dV stream
+    assert lib.sba_bwd_scratch_bytes(C.byref(p)) == 4 * table + scaled_q + 256    # no workspace: the backward recomputes those tables (+ error word)
     p.workspace = 1
-    assert lib.sba_bwd_scratch_bytes(C.byref(p)) == 2 * table + 256    # what the backward needs for itself
+    assert lib.sba_bwd_scratch_bytes(C.byref(p)) == 2 * table + scaled_q + 256    # what the backward needs for itself
     p.workspace = None
     p.dtype = _lib.SBA_DTYPE_F32                    # fp32 at head_dim 64 runs on the matrix cores too: one table from the forward
     assert lib.sba_workspace_bytes(C.byref(p)) == table
