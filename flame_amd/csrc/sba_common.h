@@ -137,15 +137,19 @@ template <> struct Elem<uint16_t> {   // bf16 bits
 
 }  // namespace sba
 
-// Grids of at most this many workgroups take the two-steps-per-iteration kernels (head_dim 64).
-// SBA_TWO_STEP_MAX_GRID overrides it for experiments; read once per process.
-inline unsigned sba_two_step_max_grid() {
-    static const unsigned v = [] {
+// Grids of at most this many workgroups take the kernels that split a sweep inside the workgroup (head_dim 64):
+// the segmented forward up to 640 workgroups, the two-steps-per-iteration dQ kernel up to 544 (measured at
+// H = 16: at 528 workgroups the segmented forward takes 69.9 us against the one-sweep kernel's 76.5, at 640
+// 93.8 against 94.7, at 768 122 against 114; the two-step dQ kernel 103.9 against 106.4 at 528 and 122.0
+// against 120.6 at 576).  SBA_TWO_STEP_MAX_GRID overrides both for experiments and tests; read once per process.
+inline unsigned sba_two_step_max_grid(unsigned by_default) {
+    static const int v = [] {
         const char* e = getenv("SBA_TWO_STEP_MAX_GRID");
-        return e ? (unsigned)atoi(e) : 512u;
+        return e ? atoi(e) : -1;
     }();
-    return v;
+    return v >= 0 ? (unsigned)v : by_default;
 }
+constexpr unsigned kSegmentedForwardMaxGrid = 640, kTwoStepDqMaxGrid = 544;
 
 // Launchers implemented in the kernel translation units.
 int sba_generic_padded_dim(int D);

@@ -1704,11 +1704,11 @@ int sba_launch_mfma_bwd(const sba::KParams& kp_in, int phases, hipStream_t s) {
         (const char*)kp.gmid - (const char*)kp.rtab != (const char*)kp.gtab - (const char*)kp.rmid) return SBA_ERR_WORKSPACE;
     // Key-owner pass.  head_dim 64: from about three workgroups per CU on, the kernel whose waves
     // own their keys outright is ahead; below, the resident producer/consumer stream, which splits
-    // the work into twice as many items and balances them itself.  head_dim 128: the own-keys
-    // kernel once every CU has more than one workgroup (128-key blocks); below, the kernel with
-    // 64-key blocks, which has twice as many workgroups.
+    // the work into twice as many items and balances them itself.  head_dim 128: the paired kernel at
+    // every size (on 64 ... 256 workgroups of B=1, H=16 it takes 27 / 44 / 62 / 81 us where the kernel
+    // with one workgroup per 64-key block takes 33 / 55 / 73 / 103); SBA_DKV_KERNEL=other still selects that one.
     const unsigned cus = (unsigned)sba_cu_count();
-    const bool own = own_keys_kernel(kp.head_dim == 64 ? grid.x >= 3u * cus : grid.x > cus);
+    const bool own = own_keys_kernel(kp.head_dim == 64 ? grid.x >= 3u * cus : true);
     const char* which = getenv("SBA_DKV_KERNEL");
     const bool plain = which && !strcmp(which, "plain");
     // the stream with eight half-block producers (12 waves): measured within 1 % of the one with four
@@ -1720,7 +1720,7 @@ int sba_launch_mfma_bwd(const sba::KParams& kp_in, int phases, hipStream_t s) {
     if (!stream) kp.q_scaled.ptr = nullptr;
     if (kp.head_dim == 64) {
         // small grids last as long as their longest sweep: take the variant that halves it
-        if (p1 && grid.x <= sba_two_step_max_grid()) hipLaunchKernelGGL((mfma_bwd_dq2_kernel<64>), grid, dim3(2 * kThreads), 0, s, kp);
+        if (p1 && grid.x <= sba_two_step_max_grid(kTwoStepDqMaxGrid)) hipLaunchKernelGGL((mfma_bwd_dq2_kernel<64>), grid, dim3(2 * kThreads), 0, s, kp);
         else if (p1 && lean_dq_kernel(grid.x >= 8u * cus)) hipLaunchKernelGGL((mfma_bwd_dq_kernel<64, true>), grid, dim3(kThreads), 0, s, kp);
         else if (p1) hipLaunchKernelGGL((mfma_bwd_dq_kernel<64>), grid, dim3(kThreads), 0, s, kp);
         if (p2 && plain) {

@@ -373,7 +373,7 @@ int sba_launch_mfma_fwd(const sba::KParams& kp, hipStream_t s) {
     // A grid this small cannot fill the SIMDs with one sweep per workgroup, and the launch lasts
     // as long as its longest sweep: take the kernel that cuts every sweep into segments.  Larger
     // grids are bound by throughput, where the 4-wave kernel (several workgroups per CU) is ahead.
-    const bool small_grid = grid.x <= sba_two_step_max_grid();
+    const bool small_grid = grid.x <= sba_two_step_max_grid(kSegmentedForwardMaxGrid);
     if (kp.head_dim == 64 && small_grid) {
         if (kp.carry_only) launch_seg64<true>(sba_fwd_groups(), grid, s, kp);
         else launch_seg64<false>(sba_fwd_groups(), grid, s, kp);
