@@ -9,6 +9,7 @@ import argparse
 import json
 import math
 import os
+import re
 import sys
 import time
 
@@ -20,32 +21,74 @@ BF16_MFMA_PEAK_TFLOPS = 2516.6     # 256 CU x 2.4 GHz x 4096 FLOP/clk/CU (dense 
 HBM_PEAK_GBS = 8000.0               # MI355X HBM3E
 
 KERNEL_TIMING_SAMPLES = 5      # steps of the timed region whose kernels are timed with events
-# Counters cannot be read from inside this process: the figures below are copied from the rocprofv3
-# runs summarised under profiles/ (sba_cfg{2,3,4}_hbm_traffic.txt, sba_cfg{2,3,4}_shader_counters.txt) and
-# are reported with that source next to what this run measures itself.
-# HBM bytes per launch (FETCH_SIZE + WRITE_SIZE, scaled by a copy kernel of known size):
-PROFILED_HBM_BYTES = {("cfg2", "fwd"): 68880405, ("cfg2", "bwd_dq"): 83539243, ("cfg2", "bwd_dkv"): 86576464,
-                      ("cfg3", "fwd"): 993377418, ("cfg3", "bwd_dq"): 1091328401, ("cfg3", "bwd_dkv"): 1125204967,
-                      ("cfg4", "fwd"): 817857184, ("cfg4", "bwd_dq"): 1671649641, ("cfg4", "bwd_dkv"): 1398538195}
-# wave instructions per launch: (vector incl. transcendental, transcendental, MFMA)
-PROFILED_INSTRUCTIONS = {("cfg2", "fwd"): (15223616, 2212864, 1064960), ("cfg2", "bwd_dq"): (27205633, 4334592, 1597440), ("cfg2", "bwd_dkv"): (31456645, 4334592, 2146304),
-                   ("cfg3", "fwd"): (119268016, 17871840, 8648192), ("cfg3", "bwd_dq"): (204901281, 35168224, 12972288), ("cfg3", "bwd_dkv"): (259319808, 35163264, 17564160),
-                   ("cfg4", "fwd"): (226951168, 34754560, 33685504), ("cfg4", "bwd_dq"): (405098497, 68440064, 50528256), ("cfg4", "bwd_dkv"): (516210688, 67272704, 67305472)}
-# issue time of one SIMD per instruction, ns, four waves per SIMD (profiles/gfx950_issue_rates.txt): plain vector,
-# transcendental issued while MFMAs are in flight, MFMA 32x32x16 bf16.  MFMAs and plain vector instructions do not
-# overlap on gfx950, so their times add up.
-ISSUE_NS = {"vector": 0.98, "transcendental": 0.97, "mfma": 17.0}
+# Counters cannot be read from inside this process: HBM bytes and instruction counts per launch are read from the
+# rocprofv3 summaries kept under profiles/ (sba_<workload>_hbm_traffic.txt, sba_<workload>_shader_counters.txt) and
+# are reported with that source next to what this run measures itself; a missing or unreadable file gives null.
+PROFILE_DIR = os.path.join(ROOT, "profiles")
+KERNEL_COLUMN = {"fwd": "fwd", "bwd_dq": "dq", "bwd_dkv": "dkv"}
+
+
+def profiled_hbm_bytes(workload, kernel):
+    """FETCH_SIZE + WRITE_SIZE per launch, scaled by a copy kernel of known size: the line
+    'traffic per launch (read+write) in bytes: fwd N, bwd_dq N, bwd_dkv N' of the summary."""
+    try:
+        text = open(os.path.join(PROFILE_DIR, f"sba_{workload}_hbm_traffic.txt")).read()
+    except OSError:
+        return None
+    m = re.search(r"traffic per launch \(read\+write\) in bytes:([^\n(]*)", text)
+    if not m:
+        return None
+    found = dict(re.findall(r"(\w+) (\d+)", m.group(1)))
+    return int(found[kernel]) if kernel in found else None
+
+
+def profiled_instructions(workload, kernel):
+    """Wave instructions per launch (vector incl. transcendental, transcendental, MFMA) from the counter table of
+    the summary (rows SQ_INSTS_VALU, SQ_INSTS_VALU_TRANS_F32, SQ_INSTS_MFMA; columns dkv, dq, fwd)."""
+    try:
+        lines = open(os.path.join(PROFILE_DIR, f"sba_{workload}_shader_counters.txt")).read().splitlines()
+    except OSError:
+        return None
+    cols, rows = None, {}
+    for ln in lines:
+        f = ln.split()
+        if f and f[0] == "counter":
+            cols = f[1:]
+        elif cols and len(f) == len(cols) + 1 and f[0].startswith("SQ_"):
+            rows[f[0]] = dict(zip(cols, f[1:]))
+    try:
+        c = KERNEL_COLUMN[kernel]
+        return tuple(int(float(rows[r][c])) for r in ("SQ_INSTS_VALU", "SQ_INSTS_VALU_TRANS_F32", "SQ_INSTS_MFMA"))
+    except (KeyError, ValueError):
+        return None
+
+
+# Issue time of one SIMD per instruction in cycles, four waves per SIMD (profiles/gfx950_issue_rates.txt): plain
+# vector, transcendental issued while MFMAs are in flight, MFMA 32x32x16 bf16; the chip holds about 2.0 GHz under
+# this mix.  MFMAs and plain vector instructions do not overlap on gfx950, also across waves: their times add up.
+ISSUE_CYCLES = {"vector": 2.3, "transcendental": 2.2, "mfma": 34.0}
+MIXED_CLOCK_GHZ = 2.0
 N_SIMDS = 1024
+# The fewest vector instructions per (query, key) pair the algorithm needs in each kernel (of them transcendental):
+# forward exp, two fma, a multiply and half a pack; each backward pass exp, rcp, six arithmetic instructions and a pack.
+MINIMUM_PER_PAIR = {"fwd": (4.5, 1.0), "bwd_dq": (10.5, 2.0), "bwd_dkv": (10.0, 2.0)}
 
 
-def issue_floor(workload, kernel):
-    """Secondary ceiling: the time the kernel's own instruction mix needs at the measured issue rates."""
-    c = PROFILED_INSTRUCTIONS.get((workload, kernel))
+def issue_ms(valu, trans, mfma):
+    cycles = (valu - trans) * ISSUE_CYCLES["vector"] + trans * ISSUE_CYCLES["transcendental"] + mfma * ISSUE_CYCLES["mfma"]
+    return cycles / N_SIMDS / (MIXED_CLOCK_GHZ * 1e9) * 1e3
+
+
+def issue_floors(workload, kernel, pairs):
+    """Secondary ceilings: the time the kernel's instructions need at the measured issue rates, for the counts it
+    executes today and for the algorithm's minimum vector counts (same MFMAs)."""
+    c = profiled_instructions(workload, kernel)
     if c is None:
         return None
     valu, trans, mfma = c
-    ns = ((valu - trans) * ISSUE_NS["vector"] + trans * ISSUE_NS["transcendental"] + mfma * ISSUE_NS["mfma"]) / N_SIMDS
-    return ns * 1e-6      # ms
+    per_pair, trans_per_pair = MINIMUM_PER_PAIR[kernel]
+    return {"present_counts": issue_ms(valu, trans, mfma),
+            "minimum_counts": issue_ms(per_pair * pairs / 64, trans_per_pair * pairs / 64, mfma)}
 
 
 def _lognormal_lengths(total, seed, median=600.0, sigma=1.0, lo=16, hi=4096):
@@ -327,7 +370,7 @@ def main():
         "roofline": {"bound": "mfma", "kernel": dom, "achieved": round(achieved, 2),
                      "peak": BF16_MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
                      "frac": round(achieved / BF16_MFMA_PEAK_TFLOPS, 4),
-                     "traffic": PROFILED_HBM_BYTES.get((args.workload, dom)),
+                     "traffic": profiled_hbm_bytes(args.workload, dom),
                      "traffic_source": f"profiles/sba_{args.workload}_hbm_traffic.txt (rocprofv3 --pmc, not measured by this run)"},
     }
     if args.workload == "short":
@@ -340,16 +383,27 @@ def main():
                            "frac": round(gbs[dom] / HBM_PEAK_GBS, 4), "traffic": None,
                            "per_kernel_GBps": {n: round(x, 1) for n, x in gbs.items()},
                            "step_GBps": round(15 * unit / (ms * 1e-3) / 1e9, 1)}
-    fl = issue_floor(args.workload, dom)
+    fl = issue_floors(args.workload, dom, pairs)
     if fl is not None:
-        # what the dominant kernel could reach if only instruction issue limited it: MFMA time + vector time
-        out["issue_floor"] = {"kernel": dom, "floor_ms": round(fl, 4), "measured_ms": round(kern[dom], 4),
-                              "frac_of_floor_rate": round(fl / kern[dom], 3),
-                              "tflops_at_floor": round(per_kernel_flops / (fl * 1e-3) / 1e12, 1),
-                              "frac_of_mfma_peak_at_floor": round(per_kernel_flops / (fl * 1e-3) / 1e12 / BF16_MFMA_PEAK_TFLOPS, 4),
-                              "ns_per_instruction": ISSUE_NS,
+        # what the dominant kernel could reach if only instruction issue limited it (MFMA time + vector time): with
+        # the instructions it executes today, and with the fewest the algorithm needs
+        at = lambda ms_: round(per_kernel_flops / (ms_ * 1e-3) / 1e12 / BF16_MFMA_PEAK_TFLOPS, 4)
+        out["issue_floor"] = {"kernel": dom, "measured_ms": round(kern[dom], 4),
+                              "floor_ms": round(fl["present_counts"], 4),
+                              "frac_of_floor_rate": round(fl["present_counts"] / kern[dom], 3),
+                              "frac_of_mfma_peak_at_floor": at(fl["present_counts"]),
+                              "minimum_counts_floor_ms": round(fl["minimum_counts"], 4),
+                              "frac_of_mfma_peak_at_minimum_counts": at(fl["minimum_counts"]),
+                              "cycles_per_instruction": ISSUE_CYCLES, "clock_ghz": MIXED_CLOCK_GHZ,
                               "source": f"instruction counts from profiles/sba_{args.workload}_shader_counters.txt, "
                                         "issue rates from profiles/gfx950_issue_rates.txt"}
+        every_kernel = [issue_floors(args.workload, n, pairs) for n in kern]
+        if all(every_kernel):
+            # the same two ceilings for the whole step (the three kernels one after the other)
+            for which in ("present_counts", "minimum_counts"):
+                total = sum(f[which] for f in every_kernel)
+                out["issue_floor"][f"step_pct_of_mfma_peak_at_{which}"] = round(
+                    100 * f_fb / (total * 1e-3) / 1e12 / BF16_MFMA_PEAK_TFLOPS, 1)
     if not args.no_cpu_baseline and args.workload != "short":     # (the CPU leg is defined for BASELINE's configurations)
         out["cpu_baseline"] = cpu_baseline(args.workload)
     print(json.dumps(out))

@@ -109,8 +109,8 @@ def dtype_code(dt: torch.dtype) -> int:
 def check_supported(q: torch.Tensor) -> None:
     """Say up front what the kernels do not cover instead of failing inside the library."""
     if q.dtype not in (torch.float32, torch.bfloat16):
-        raise TypeError(f"stick-breaking attention supports float32 and bfloat16, got {q.dtype} "
-                        "(float16 is not offered)")
+        raise TypeError(f"stick-breaking attention supports float32, bfloat16 and (through the float32 kernels) "
+                        f"float16, got {q.dtype}")
     if q.shape[-1] > 128:
         raise ValueError(f"head_dim {q.shape[-1]} is not supported (at most 128)")
 

@@ -63,7 +63,7 @@ def test_argument_errors_are_python_errors():
     with pytest.raises(TypeError, match="share a dtype"):
         sb_attn_varlen(q, q.float(), q, cu, 200)
     with pytest.raises(TypeError, match="float16"):
-        sb_attn_varlen(q.half(), q.half(), q.half(), cu, 200)
+        sb_attn_varlen(q.double(), q.double(), q.double(), cu, 200)
     with pytest.raises(ValueError, match="head_dim"):
         sb_attn(torch.zeros(1, 1, 8, 256, device="cuda"), torch.zeros(1, 1, 8, 256, device="cuda"),
                 torch.zeros(1, 1, 8, 256, device="cuda"))
@@ -71,6 +71,31 @@ def test_argument_errors_are_python_errors():
         sb_attn_varlen(q, q, q, cu, 150)
     with pytest.raises(ValueError, match="ends at"):
         sb_attn_varlen(q, q, q, torch.tensor([0, 100, 299], dtype=torch.int32), 200)
+
+
+def test_float16_runs_on_the_float32_kernels():
+    # float16 inputs: exact in float32, computed there, rounded to float16 on the way out; against the oracle
+    # at the float32 kernels' forward tolerance plus float16's rounding of the results (2^-11 relative)
+    from flame_amd import sb_attn, sb_attn_varlen
+    from oracle import sb_oracle as O
+    from helpers import within, max_abs, rel_l2
+    B, H, T, D = 1, 2, 300, 64
+    q, k, v, do = (randn((B, H, T, D), 425 + i, 0.5 if i < 3 else 1.0, torch.float16) for i in range(4))
+    qg, kg, vg = (x.cuda().requires_grad_(True) for x in (q, k, v))
+    o, rem = sb_attn(qg, kg, vg)
+    assert o.dtype == rem.dtype == torch.float16
+    o.backward(do.cuda())
+    o_ref, rem_ref, dq_ref, dk_ref, dv_ref = O.sb_attn_grads_oracle(q, k, v, do, None)
+    within("float16 dense T=300", "o", max_abs(o.float().cpu(), o_ref), 2e-3)
+    within("float16 dense T=300", "rem", max_abs(rem.float().cpu(), rem_ref), 2e-3)
+    for name, got, ref in (("dq", qg.grad, dq_ref), ("dk", kg.grad, dk_ref), ("dv", vg.grad, dv_ref)):
+        assert got.dtype == torch.float16
+        within("float16 dense T=300", name, rel_l2(got.float().cpu(), ref), 2e-3)
+    cu = torch.tensor([0, 100, 300], dtype=torch.int32)
+    ov, rv = sb_attn_varlen(q[0].cuda(), k[0].cuda(), v[0].cuda(), cu, 200)
+    assert ov.dtype == torch.float16
+    o_doc, _ = sb_attn(q[:, :, 100:].cuda(), k[:, :, 100:].cuda(), v[:, :, 100:].cuda())
+    assert torch.equal(ov[:, 100:], o_doc[0])
 
 
 def test_no_grad_forward_keeps_no_carry_table():
