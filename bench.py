@@ -294,6 +294,10 @@ def main():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--workload", default="cfg2", choices=["cfg2", "cfg3", "cfg4", "cfg5", "short", "copy"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--carries", default="kept", choices=["kept", "default"],
+                    help="kept: the forward keeps its carry tables whatever their size (the kernels as such); default: the "
+                         "operator's own rule, which above its workspace budget (256 MiB) keeps nothing and lets the "
+                         "backward rebuild them (cfg4: 270 MB)")
     ap.add_argument("--compile", action="store_true",
                     help="cfg5 only: torch.compile every block, as flame does with --training.compile")
     args = ap.parse_args()
@@ -320,6 +324,9 @@ def main():
         return
     desc, (q, k, v, do, cu, max_len), pairs, tokens, D, H = make_workload(args.workload, dev)
     q.requires_grad_(True), k.requires_grad_(True), v.requires_grad_(True)
+    from flame_amd import _lib
+    if args.carries == "kept":
+        _lib.set_workspace_budget(float("inf"))
 
     def step():
         q.grad = k.grad = v.grad = None
@@ -355,6 +362,7 @@ def main():
     # counted products (4*d*P); recomputed products are not counted
     per_kernel_flops = 4.0 * D * pairs
     dom = max(kern, key=kern.get)
+    desc["carries"] = "recomputed in the backward" if "bwd_carries_dq" in kern else "kept from the forward"
     achieved = per_kernel_flops / (kern[dom] * 1e-3) / 1e12
     out = {
         "metric": "sb_attn_fwd_bwd_tflops", "value": round(tflops, 2), "unit": "TFLOP/s",
@@ -383,7 +391,7 @@ def main():
                            "frac": round(gbs[dom] / HBM_PEAK_GBS, 4), "traffic": None,
                            "per_kernel_GBps": {n: round(x, 1) for n, x in gbs.items()},
                            "step_GBps": round(15 * unit / (ms * 1e-3) / 1e9, 1)}
-    fl = issue_floors(args.workload, dom, pairs)
+    fl = issue_floors(args.workload, dom, pairs) if dom in KERNEL_COLUMN else None
     if fl is not None:
         # what the dominant kernel could reach if only instruction issue limited it (MFMA time + vector time): with
         # the instructions it executes today, and with the fewest the algorithm needs
@@ -397,7 +405,7 @@ def main():
                               "cycles_per_instruction": ISSUE_CYCLES, "clock_ghz": MIXED_CLOCK_GHZ,
                               "source": f"instruction counts from profiles/sba_{args.workload}_shader_counters.txt, "
                                         "issue rates from profiles/gfx950_issue_rates.txt"}
-        every_kernel = [issue_floors(args.workload, n, pairs) for n in kern]
+        every_kernel = [issue_floors(args.workload, n, pairs) if n in KERNEL_COLUMN else None for n in kern]
         if all(every_kernel):
             # the same two ceilings for the whole step (the three kernels one after the other)
             for which in ("present_counts", "minimum_counts"):

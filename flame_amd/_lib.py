@@ -159,14 +159,14 @@ def empty_grads_like(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor):
 # forward's sweep for the carries alone (bit-identical gradients, 12-13 % more time per forward + backward).
 # The reference keeps one float per query (sb_fwd.py:146); the tables grow with the square of the sequence
 # length: 17 MB at B=1, H=16, T=4096, 270 MB at T=16384, 4.3 GB for a dense 65 536-token row.
-DEFAULT_WORKSPACE_BUDGET = 128 << 20
+DEFAULT_WORKSPACE_BUDGET = 256 << 20
 _workspace_budget = None            # set_workspace_budget(); None: SBA_WORKSPACE_BUDGET_MB or the default
 
 
 def set_workspace_budget(nbytes) -> None:
     """Largest carry-table workspace (bytes) a forward may keep for its backward; larger ones are
     recomputed in the backward instead.  None restores the default (SBA_WORKSPACE_BUDGET_MB megabytes if
-    that is set, else 128 MiB); 0 never keeps anything; float('inf') always keeps the tables."""
+    that is set, else 256 MiB); 0 never keeps anything; float('inf') always keeps the tables."""
     global _workspace_budget
     _workspace_budget = nbytes
 

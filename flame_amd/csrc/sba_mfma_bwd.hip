@@ -72,11 +72,7 @@ __global__ __launch_bounds__(kThreads, (D == 64 && kLean) ? 3 : 2) void mfma_bwd
     bf16x8 qf[D / 16], dof[D / 16];
     load_row_frags<D>(qf, p.q, qbase, qi, job.len, lane);
     prescale_frags(qf, p.scale2);          // the score MFMAs then deliver base-2 logits
-    store_scaled_q<D>(p, job, head, qi, lane, qf);
     load_row_frags<D>(dof, p.d_o, dobase, qi, job.len, lane);
-    float dr = 0.f;
-    if (row_ok && p.d_rem.ptr)
-        dr = Elem<uint16_t>::load(p.d_rem.ptr, (int64_t)job.seq * p.d_rem.sb + (int64_t)head * p.d_rem.sh + job.tok0 + qi);
 
     f32x16 dqacc[D / 32];
 #pragma unroll
@@ -108,8 +104,15 @@ __global__ __launch_bounds__(kThreads, (D == 64 && kLean) ? 3 : 2) void mfma_bwd
     float Rnext = (row_ok && n_steps > 0) ? *rcur : 1.0f;
     float Gstore = 0.f;
     bool g_pending = false;
+    // (last of the prologue's loads: its conversion waits for it, and with it for everything requested before)
+    float dr = 0.f;
+    if (row_ok && p.d_rem.ptr)
+        dr = Elem<uint16_t>::load(p.d_rem.ptr, (int64_t)job.seq * p.d_rem.sb + (int64_t)head * p.d_rem.sh + job.tok0 + qi);
     wait_global_memory();
     __syncthreads();
+    // (behind the prologue's loads: a store in front of them would keep the compiler from issuing them together,
+    // and the wait above would fall on it; here it retires under the first step)
+    store_scaled_q<D>(p, job, head, qi, lane, qf);
     auto do_step = [&](int step, auto buf_c) __attribute__((always_inline)) {
         constexpr int buf = decltype(buf_c)::value;
         constexpr TileAt ktile = {buf * 2 * kTile};
@@ -255,11 +258,7 @@ __global__ __launch_bounds__(2 * kThreads, 2) void mfma_bwd_dq2_kernel(KParams p
     bf16x8 qf[D / 16], dof[D / 16];
     load_row_frags<D>(qf, p.q, qbase, qi, job.len, lane);
     prescale_frags(qf, p.scale2);          // the score MFMAs then deliver base-2 logits
-    if (grp == 0) store_scaled_q<D>(p, job, head, qi, lane, qf);
     load_row_frags<D>(dof, p.d_o, dobase, qi, job.len, lane);
-    float dr = 0.f;
-    if (row_ok && p.d_rem.ptr)
-        dr = Elem<uint16_t>::load(p.d_rem.ptr, (int64_t)job.seq * p.d_rem.sb + (int64_t)head * p.d_rem.sh + job.tok0 + qi);
 
     f32x16 dqacc[D / 32];
 #pragma unroll
@@ -289,8 +288,13 @@ __global__ __launch_bounds__(2 * kThreads, 2) void mfma_bwd_dq2_kernel(KParams p
     float Rnext = (row_ok && grp < n_steps) ? *rcur : 1.0f;
     float Gstore = 0.f;
     bool g_pending = false;
+    // (last of the prologue's loads: its conversion waits for it, and with it for everything requested before)
+    float dr = 0.f;
+    if (row_ok && p.d_rem.ptr)
+        dr = Elem<uint16_t>::load(p.d_rem.ptr, (int64_t)job.seq * p.d_rem.sb + (int64_t)head * p.d_rem.sh + job.tok0 + qi);
     wait_global_memory();
     __syncthreads();
+    if (grp == 0) store_scaled_q<D>(p, job, head, qi, lane, qf);      // (placed as in the one-step kernel)
     // Every LDS address of the loop is a sweep-constant register plus an immediate: the lane offsets are made absolute
     // for this group's tiles once, and the loop runs in one copy per tile buffer (see the one-step kernel).
     lo.rebase(my_tiles);

@@ -74,7 +74,8 @@ def launch_bwd(lib, p):
     mark("start")
     p.bwd_phases = 1
     _lib.check(lib.sba_bwd(C.byref(p)), "sba_bwd")
-    mark("bwd_dq")
+    # without the forward's tables the first call also rebuilds them: two kernels in one span, named for both
+    mark("bwd_dq" if p.workspace else "bwd_carries_dq")
     p.bwd_phases = 2
     _lib.check(lib.sba_bwd(C.byref(p)), "sba_bwd")
     mark("bwd_dkv")

@@ -167,7 +167,7 @@ def test_workspace_budget_switch(monkeypatch):
     monkeypatch.delenv("SBA_RECOMPUTE_CARRIES", raising=False)
     monkeypatch.delenv("SBA_WORKSPACE_BUDGET_MB", raising=False)
     _lib.set_workspace_budget(None)
-    assert _lib.workspace_budget() == 128 << 20
+    assert _lib.workspace_budget() == 256 << 20
     assert not _lib.recompute_carries(17 << 20)            # B=1, H=16, T=4096: kept
     assert _lib.recompute_carries(270 << 20)               # T=16384: recomputed
     monkeypatch.setenv("SBA_WORKSPACE_BUDGET_MB", "512")

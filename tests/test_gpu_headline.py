@@ -94,7 +94,7 @@ def test_config3_pack_longest_document_gradients_against_oracle():
 
 def test_long_dense_row_switches_to_recompute_and_stays_within_memory(monkeypatch):
     # A dense row of 65 536 tokens at H=16, d=64: the forward's carry tables would be 4.3 GB, far above
-    # the workspace budget (128 MiB by default), so the operator keeps nothing and the backward recomputes
+    # the workspace budget (256 MiB by default), so the operator keeps nothing and the backward recomputes
     # the carries.  What the autograd graph holds between forward and backward is then the inputs and the
     # outputs only; the backward's transient scratch (four tables) is freed when it returns.  Gradients are
     # bit-identical to the run that keeps the tables.
