@@ -121,3 +121,53 @@ def test_carries_that_underflow_to_zero(D):
     assert max_abs(rem.detach().float().cpu(), rem_ref.float()) <= 2e-2
     for got, ref in ((qg.grad, dq), (kg.grad, dk), (vg.grad, dv)):
         assert rel_l2(got.float().cpu(), ref.float()) <= 5e-2
+
+
+def test_error_word_set_from_the_host_is_reported_and_cleared_by_the_next_backward():
+    # The error word of the bf16 matrix-core backward (last 256 bytes of its scratch) is cleared by the
+    # dQ pass and may be set by the stream kernel.  No kernel is made to give up here: the host writes the
+    # word between the two passes of a backward issued as two calls (SbaParams.bwd_phases), which is what a
+    # wave abandoning its wait in the second pass would have done.  sba_bwd_gave_up must report it, the
+    # Python check must raise, and a complete backward on the same scratch must clear it again.
+    import ctypes as C
+    import math
+    from flame_amd import _lib
+    lib = _lib.load()
+    B, H, T, D = 1, 2, 512, 64
+    q, k, v, do = (randn((B, H, T, D), 760 + i, 0.5 if i < 3 else 1.0, torch.bfloat16).cuda() for i in range(4))
+    p = _lib.SbaParams()
+    p.struct_size = C.sizeof(_lib.SbaParams)
+    p.dtype = _lib.SBA_DTYPE_BF16
+    p.n_seq, p.n_heads, p.seq_len, p.total_tokens, p.head_dim = B, H, T, T, D
+    p.scale = 1.0 / math.sqrt(D)
+    p.q, p.k, p.v = _lib.tensor4(q), _lib.tensor4(k), _lib.tensor4(v)
+    p.stream = torch.cuda.current_stream().cuda_stream
+    o, rem = torch.empty_like(q), torch.empty(B, H, T, dtype=q.dtype, device="cuda")
+    p.o, p.rem = _lib.tensor4(o), _lib.SbaVector(rem.data_ptr(), rem.stride(0), rem.stride(1))
+    ws = torch.empty(int(lib.sba_workspace_bytes(C.byref(p))), dtype=torch.uint8, device="cuda")
+    p.save_for_backward, p.workspace, p.workspace_bytes = 1, ws.data_ptr(), ws.numel()
+    _lib.check(lib.sba_fwd(C.byref(p)), "sba_fwd")
+    dq, dk, dv = (torch.empty_like(q) for _ in range(3))
+    p.d_o, p.dq, p.dk, p.dv = _lib.tensor4(do), _lib.tensor4(dq), _lib.tensor4(dk), _lib.tensor4(dv)
+    scratch = torch.empty(int(lib.sba_bwd_scratch_bytes(C.byref(p))), dtype=torch.uint8, device="cuda")
+    p.bwd_scratch, p.bwd_scratch_bytes = scratch.data_ptr(), scratch.numel()
+    word = scratch[-256:-252].view(torch.int32)
+    flag = C.c_int(-1)
+    print("error word: two-call backward with the word written by the host in between", flush=True)
+    p.bwd_phases = 1
+    _lib.check(lib.sba_bwd(C.byref(p)), "sba_bwd pass 1")
+    torch.cuda.synchronize()
+    assert int(word.item()) == 0                                   # cleared by the dQ pass
+    word.fill_(1)
+    p.bwd_phases = 2
+    _lib.check(lib.sba_bwd(C.byref(p)), "sba_bwd pass 2")          # runs normally and leaves the word alone
+    assert lib.sba_bwd_gave_up(C.byref(p), 0, C.byref(flag)) == 0 and flag.value == 1
+    with pytest.raises(RuntimeError, match="abandoned a bounded internal wait"):
+        _lib.raise_if_gave_up(p)
+    first = (dq.clone(), dk.clone(), dv.clone())
+    p.bwd_phases = 0
+    _lib.check(lib.sba_bwd(C.byref(p)), "sba_bwd")
+    assert lib.sba_bwd_gave_up(C.byref(p), 0, C.byref(flag)) == 0 and flag.value == 0
+    _lib.raise_if_gave_up(p)
+    for a, b in zip(first, (dq, dk, dv)):                          # the word changes nothing in the results
+        assert torch.equal(a, b)
