@@ -276,7 +276,11 @@ template <int D> struct TileCopy {
 // issues instructions w4, w4 + 4, ...  The per-lane byte offsets inside a tile never change, so
 // a step costs no vector address arithmetic.  Rows past the end of the sequence are clamped to
 // its last row instead of zero-filled: those keys are masked for every valid query.
-template <int D, bool kNatural = false, bool kScalarBase = true> struct TileDma {      // kNatural: rows kept in their order (query tiles)
+// kLateRagged: the lane's row and chunk for the one ragged tile of a sequence are worked out where that tile is
+// requested, from a copy of the lane index that the compiler cannot see through.  As loop invariants they are
+// otherwise computed once at the top of the kernel and occupy registers through the whole sweep: in the
+// register-lean dQ kernel that is the difference between four spilled registers and none.
+template <int D, bool kNatural = false, bool kScalarBase = true, bool kLateRagged = false> struct TileDma {      // kNatural: rows kept in their order (query tiles)
     static constexpr int kPerWave = 64 * D * 2 / 1024 / 4;    // 2 (D=64) or 4 (D=128)
     uint32_t off[kPerWave];
     const char* origin;        // row 0 of the (sequence, head) slice: uniform
@@ -340,10 +344,12 @@ template <int D, bool kNatural = false, bool kScalarBase = true> struct TileDma 
                     (__attribute__((address_space(3))) void*)(uintptr_t)(uint32_t)(uintptr_t)(tile + (w4 + 4 * i) * 1024),
                     16, 0, 0);
         } else {
+            int lane_here = lane;
+            if (kLateRagged) asm volatile("" : "+v"(lane_here));
 #pragma unroll
             for (int i = 0; i < kPerWave; ++i) {
                 int kl, c;
-                where(w4 + 4 * i, lane, kl, c);
+                where(w4 + 4 * i, lane_here, kl, c);
                 kl = min(kl, len - 1 - row0);
                 __builtin_amdgcn_global_load_lds(
                     (const __attribute__((address_space(1))) void*)(tile_base + 2 * ((int64_t)kl * st + c * 8)),

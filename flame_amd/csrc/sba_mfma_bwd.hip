@@ -83,7 +83,7 @@ __global__ __launch_bounds__(kThreads, (D == 64 && kLean) ? 3 : 2) void mfma_bwd
     const int kmax = imax - strict;
     const int n_steps = kmax >= 0 ? kmax / kKeyBlock + 1 : 0;
 
-    TileDma<D> kc, vc;
+    TileDma<D, false, true, D == 64 && kLean> kc, vc;
     kc.init(lane, wave, p.k, kbase);
     vc.init(lane, wave, p.v, vbase);
     if (n_steps > 0) {
