@@ -228,6 +228,40 @@ def cpu_baseline(name, reps=3):
             "tokens_per_s": round(tokens / (dt * full_pairs / pairs), 1)}
 
 
+def parity_sample(name, q, k, v, do, cu, o, rem):
+    """One head of the TIMED tensors against the oracle (the checker of the test-suite, here on a sample small
+    enough for a few seconds of CPU): cfg2 head 0 whole, forward and all gradients; cfg3 head 0, the first
+    documents of the pack (up to 4096 tokens), forward and all gradients; cfg4 head 0, the first 2048 tokens -
+    causality makes o, rem and dq of a prefix depend on the prefix alone (dk, dv do not: not compared there).
+    Tolerances as in the tests: o / rem max-abs 2e-2, gradients 5e-2 relative L2."""
+    import torch
+    from oracle import sb_oracle as O
+    f = lambda t: t.detach().float().cpu()
+    rel = lambda a, b: float((a - b).norm() / b.norm().clamp_min(1e-30))
+    if name == "cfg3":
+        ends = [int(e) for e in cu.cpu().tolist()]
+        n_docs = max(1, sum(1 for e in ends[1:] if e <= 4096))
+        N = ends[n_docs]
+        cut = lambda t: f(t[0:1, :N])
+        ref = O.sb_attn_grads_oracle(cut(q), cut(k), cut(v), cut(do), None, cu_seqlens=ends[:n_docs + 1])
+        got = (cut(o), f(rem[0:1, :N]), cut(q.grad), cut(k.grad), cut(v.grad))
+        what, full = f"head 0, first {n_docs} documents ({N} tokens) of the timed pack", True
+    else:
+        P = 2048 if name == "cfg4" else q.shape[2]
+        cut = lambda t: f(t[:, 0:1, :P])
+        ref = O.sb_attn_grads_oracle(cut(q), cut(k), cut(v), cut(do))
+        got = (cut(o), f(rem[:, 0:1, :P]), cut(q.grad), cut(k.grad), cut(v.grad))
+        full = name != "cfg4"
+        what = f"head 0 of the timed tensors, {'all' if full else 'the first'} {P} tokens" + ("" if full else " (o, rem, dq)")
+    res = {"what": what, "o_max_abs": float((got[0] - ref[0]).abs().max()), "rem_max_abs": float((got[1] - ref[1]).abs().max()),
+           "dq_rel_l2": rel(got[2], ref[2])}
+    if full:
+        res["dk_rel_l2"], res["dv_rel_l2"] = rel(got[3], ref[3]), rel(got[4], ref[4])
+    res["within_tolerance"] = bool(res["o_max_abs"] <= 2e-2 and res["rem_max_abs"] <= 2e-2 and
+                                   all(res[g] <= 5e-2 for g in res if g.endswith("rel_l2")))
+    return {k_: (round(v_, 6) if isinstance(v_, float) else v_) for k_, v_ in res.items()}
+
+
 def settle_clocks(step, seconds=0.3):
     """Untimed work in front of the warm-up steps: an idle GPU needs some tens of milliseconds of
     load before it runs at its sustained clocks, and ten warm-up steps of a 0.3 ms workload are
@@ -331,10 +365,11 @@ def main():
     def step():
         q.grad = k.grad = v.grad = None
         if cu is None:
-            o, _ = sb_attn(q, k, v)
+            o, rem = sb_attn(q, k, v)
         else:
-            o, _ = sb_attn_varlen(q, k, v, cu, max_len)
+            o, rem = sb_attn_varlen(q, k, v, cu, max_len)
         torch.autograd.backward([o], [do])
+        return o, rem
 
     settle_clocks(step)
     for _ in range(args.warmup):
@@ -414,6 +449,8 @@ def main():
                     100 * f_fb / (total * 1e-3) / 1e12 / BF16_MFMA_PEAK_TFLOPS, 1)
     if not args.no_cpu_baseline and args.workload != "short":     # (the CPU leg is defined for BASELINE's configurations)
         out["cpu_baseline"] = cpu_baseline(args.workload)
+        o, rem = step()          # the timed tensors once more, for the check below
+        out["parity_sample"] = parity_sample(args.workload, q, k, v, do, cu, o, rem)
     print(json.dumps(out))
 
 
