@@ -3,6 +3,7 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 #include <stdlib.h>
+#include <atomic>
 #include "../../include/sba_mi355x.h"
 
 namespace sba {
@@ -137,19 +138,34 @@ template <> struct Elem<uint16_t> {   // bf16 bits
 
 }  // namespace sba
 
-// Grids of at most this many workgroups take the kernels that split a sweep inside the workgroup (head_dim 64):
-// the segmented forward up to 640 workgroups, the two-steps-per-iteration dQ kernel up to 544 (measured at
-// H = 16: at 528 workgroups the segmented forward takes 69.9 us against the one-sweep kernel's 76.5, at 640
-// 93.8 against 94.7, at 768 122 against 114; the two-step dQ kernel 103.9 against 106.4 at 528 and 122.0
-// against 120.6 at 576).  SBA_TWO_STEP_MAX_GRID overrides both for experiments and tests; read once per process.
-inline unsigned sba_two_step_max_grid(unsigned by_default) {
+// SBA_TWO_STEP_MAX_GRID (experiments and tests; read once per process): grids of at most this many workgroups take
+// the kernels that split a sweep inside the workgroup (head_dim 64), larger ones do not.  -1: not set.
+inline int sba_two_step_env() {
     static const int v = [] {
         const char* e = getenv("SBA_TWO_STEP_MAX_GRID");
         return e ? atoi(e) : -1;
     }();
-    return v >= 0 ? (unsigned)v : by_default;
+    return v;
 }
-constexpr unsigned kSegmentedForwardMaxGrid = 640, kTwoStepDqMaxGrid = 544;
+inline unsigned sba_two_step_max_grid(unsigned by_default) {
+    return sba_two_step_env() >= 0 ? (unsigned)sba_two_step_env() : by_default;
+}
+// The two-steps-per-iteration dQ kernel up to 544 workgroups (measured at H = 16: 103.9 us against the one-step
+// kernel's 106.4 at 528 workgroups, 122.0 against 120.6 at 576).  The forward's rule is in sba_launch_mfma_fwd().
+constexpr unsigned kTwoStepDqMaxGrid = 544;
+
+// compute units of the current device (asked once per device)
+inline int sba_cu_count() {
+    static std::atomic<int> cached[64];       // zero-initialised; threads that race here store the same value
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) dev = 0;
+    int n = cached[dev].load(std::memory_order_relaxed);
+    if (n == 0) {
+        if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
+        cached[dev].store(n, std::memory_order_relaxed);
+    }
+    return n;
+}
 
 // Launchers implemented in the kernel translation units.
 int sba_generic_padded_dim(int D);

@@ -1667,19 +1667,6 @@ __global__ __launch_bounds__(2 * kThreads, 2) void mfma_bwd_dkv_pair_kernel(KPar
 
 bool sba_mfma_bwd_available() { return true; }
 
-// compute units of the current device (asked once per device)
-static int sba_cu_count() {
-    static std::atomic<int> cached[64];       // zero-initialised; threads that race here store the same value
-    int dev = 0;
-    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) dev = 0;
-    int n = cached[dev].load(std::memory_order_relaxed);
-    if (n == 0) {
-        if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
-        cached[dev].store(n, std::memory_order_relaxed);
-    }
-    return n;
-}
-
 // SBA_DKV_KERNEL=own / =other overrides the choice between the key-owner kernels (tests run
 // both on the same inputs).
 static bool own_keys_kernel(bool by_size) {

@@ -352,11 +352,43 @@ __global__ __launch_bounds__(G * kThreads) void mfma_fwd_seg_kernel(KParams p) {
 
 }  // namespace sba
 
-// Groups per workgroup of the segmented forward (SBA_FWD_GROUPS overrides it for experiments and tests).
-static int sba_fwd_groups() {
+// Key segments per sweep for the forward at head_dim 64: 4, 2, or 0 = one sweep per workgroup.
+//
+// What decides is how long the launch's longest sweep is against the work of an average workgroup slot.  With
+// one sweep per workgroup a CU holds four workgroups, so the launch has 4 x CUs slots; it cannot end before its
+// longest sweep has, and if that sweep is several times the average slot's work, most of the chip idles behind it.
+//     r = longest sweep x slots / all sweep steps of the launch
+// (steps of 64 keys; a sequence of n row blocks has n (n + 1) of them per head, which is also its number of
+// carry-table columns).  Two segments halve the longest sweep at 8 waves per workgroup (two workgroups per CU),
+// four quarter it at 16 waves (one workgroup per CU: worth it only while the grid is at most two rounds of them).
+// Measured on MI355X, forward time in us, one sweep / two segments / four segments:
+//     B=1 H=16 T=3584 (r 4.4)   64.8 / 55.8 / 51.1      B=2 H=16 T=2304 (r 3.4)   47.7 / 42.6 / 52.4
+//     B=1 H=16 T=4096 (r 3.9)   74.5 / 63.9 / 60.4      B=4 H=16 T=1024 (r 3.6, 512 workgroups)  26.2 / 26.1 / 29.7
+//     B=1 H=16 T=4224 (r 3.8)   76.5 / 66.9 / 69.6      B=8 H=16 T=512  (r 3.2, 512 workgroups)  18.5 / 18.8 / 24.9
+//     B=1 H=16 T=5120 (r 3.1)   95.7 / 82.8 / 93.3      B=1 H=32 T=4096 (r 1.9)   96.8 / 96.6 / 112.8
+//     B=1 H=16 T=6144 (r 2.6)  115.8 / 110.0 / 120.0    B=2 H=16 T=4096 (r 1.9)   98.4 / 97.3 / 112.7
+//     B=1 H=16 T=8192 (r 2.0)  179.8 / 170.9 / 181.9    B=5 H=16 T=2048 (r 1.5)   65.4 / 70.8 / -
+//     B=1 H=16 T=10240 (r 1.6) 253.7 / 248.6 / -        B=3 H=16 T=4096 (r 1.3)  127.6 / 132.5 / -
+//     packs of log-normal documents, H=16 (tokens, longest document, r): one sweep / two segments
+//         8192, 2802, r 3.2   57.7 / 51.2 (four: 69.8)     8192, 4096, r 2.8   81.5 / 72.3     4096, 1393, r 4.7   31.0 / 28.0
+//         6000, 1162, r 3.3   30.5 / 31.5                  10000, 2243, r 2.4  51.1 / 56.0     12288, 2069, r 1.9  56.4 / 64.7
+// Two segments pay from r = 1.7 on for dense batches but lose 10-16 % on packs (one long document among many short
+// ones) up to r = 2.4: the rule takes them from 2.7 on.
+// SBA_FWD_GROUPS=2|3|4 forces the number of segments where the rule picks any; SBA_TWO_STEP_MAX_GRID=n replaces
+// the rule by "segments (4, or as forced) up to n workgroups".
+static int forward_segments(const sba::KParams& kp, unsigned grid) {
+    if (kp.head_dim != 64) return 0;
     const char* e = getenv("SBA_FWD_GROUPS");
-    const int g = e ? atoi(e) : 4;
-    return g == 2 || g == 3 || g == 4 ? g : 4;
+    const int forced = e ? atoi(e) : 0;
+    const bool force = forced == 2 || forced == 3 || forced == 4;
+    if (sba_two_step_env() >= 0) return grid <= (unsigned)sba_two_step_env() ? (force ? forced : 4) : 0;
+    const double cus = sba_cu_count();
+    const double longest = 2.0 * ((kp.seq_len + sba::kRowBlock - 1) / sba::kRowBlock);
+    double steps = (double)(kp.tab_head_stride / sba::kRowBlock) * kp.n_heads;
+    if (steps <= 0) steps = (double)grid * (longest / 2 + 1);          // (no table size given: every sweep half the longest)
+    const double r = longest * 4.0 * cus / steps;
+    const int segments = (r >= 3.8 && grid <= 2 * (unsigned)cus) ? 4 : (r >= 2.7 ? 2 : 0);
+    return segments && force ? forced : segments;
 }
 
 template <bool kCarryOnly>
@@ -370,13 +402,10 @@ static void launch_seg64(int groups, dim3 grid, hipStream_t s, const sba::KParam
 int sba_launch_mfma_fwd(const sba::KParams& kp, hipStream_t s) {
     using namespace sba;
     dim3 grid((unsigned)kp.n_jobs * kp.n_heads);
-    // A grid this small cannot fill the SIMDs with one sweep per workgroup, and the launch lasts
-    // as long as its longest sweep: take the kernel that cuts every sweep into segments.  Larger
-    // grids are bound by throughput, where the 4-wave kernel (several workgroups per CU) is ahead.
-    const bool small_grid = grid.x <= sba_two_step_max_grid(kSegmentedForwardMaxGrid);
-    if (kp.head_dim == 64 && small_grid) {
-        if (kp.carry_only) launch_seg64<true>(sba_fwd_groups(), grid, s, kp);
-        else launch_seg64<false>(sba_fwd_groups(), grid, s, kp);
+    const int segments = forward_segments(kp, grid.x);
+    if (segments) {
+        if (kp.carry_only) launch_seg64<true>(segments, grid, s, kp);
+        else launch_seg64<false>(segments, grid, s, kp);
     } else if (kp.head_dim == 64) {
         if (kp.carry_only) hipLaunchKernelGGL((mfma_fwd_kernel<64, true>), grid, dim3(kThreads), 0, s, kp);
         else hipLaunchKernelGGL((mfma_fwd_kernel<64, false>), grid, dim3(kThreads), 0, s, kp);

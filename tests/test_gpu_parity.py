@@ -365,8 +365,9 @@ def test_torch_compile_fullgraph_matches_eager():
 
 
 def test_small_and_large_grids_take_different_forward_kernels_and_agree(monkeypatch):
-    # <= 512 workgroups: the segmented forward (2, 3 or 4 key segments per sweep); above: one workgroup per
-    # sweep.  Same rows computed all ways (a batch of 1 vs the same sequence repeated 40 times).
+    # A launch whose longest sweep is long against the work of an average workgroup slot takes the segmented
+    # forward (2, 3 or 4 key segments per sweep), one with many equal sweeps one workgroup per sweep.  Same rows
+    # computed all ways (a batch of 1 vs the same sequence repeated 40 times).
     sb_attn, _ = _ops()
     q, k, v = (randn((1, 4, 1000, 64), 110 + i, 0.5, torch.bfloat16).cuda() for i in range(3))
     o1, r1 = sb_attn(q, k, v)                                   # 8 row-blocks x 4 heads = 32 workgroups
