@@ -167,6 +167,18 @@ inline int sba_cu_count() {
     return n;
 }
 
+// How long a launch's longest sweep is against the work of an average workgroup slot when every workgroup runs
+// one sweep and a CU holds four of them:  r = longest sweep x (4 x CUs) / all sweep steps of the launch  (steps of
+// 64 keys; a sequence of n row blocks has n (n + 1) of them per head, which is also its number of carry-table
+// columns).  A launch cannot end before its longest sweep has; for r well above 1 most of the chip idles behind
+// it, and the kernels that cut a sweep into pieces pay.  seq_len is the longest sequence of the launch.
+inline double sba_tail_ratio(const sba::KParams& kp, unsigned grid) {
+    const double longest = 2.0 * ((kp.seq_len + sba::kRowBlock - 1) / sba::kRowBlock);
+    double steps = (double)(kp.tab_head_stride / sba::kRowBlock) * kp.n_heads;
+    if (steps <= 0) steps = (double)grid * (longest / 2 + 1);          // (no table size given: every sweep half the longest)
+    return longest * 4.0 * sba_cu_count() / steps;
+}
+
 // Launchers implemented in the kernel translation units.
 int sba_generic_padded_dim(int D);
 int sba_launch_generic_fwd(const sba::KParams& kp, int dtype, hipStream_t s);

@@ -1698,8 +1698,11 @@ int sba_launch_mfma_bwd(const sba::KParams& kp_in, int phases, hipStream_t s) {
     // the work into twice as many items and balances them itself.  head_dim 128: the paired kernel at
     // every size (on 64 ... 256 workgroups of B=1, H=16 it takes 27 / 44 / 62 / 81 us where the kernel
     // with one workgroup per 64-key block takes 33 / 55 / 73 / 103); SBA_DKV_KERNEL=other still selects that one.
+    // Batches of short sequences (sweeps of at most 16 steps) also take the own-keys kernel at any size: on
+    // 512 workgroups B=8, T=512 takes 27.3 us against the stream's 33.0, B=4, T=1024 44.0 against 45.3.
     const unsigned cus = (unsigned)sba_cu_count();
-    const bool own = own_keys_kernel(kp.head_dim == 64 ? grid.x >= 3u * cus : true);
+    const bool short_sweeps = kp.seq_len <= 8 * kRowBlock;
+    const bool own = own_keys_kernel(kp.head_dim == 64 ? grid.x >= 3u * cus || (short_sweeps && grid.x >= 2u * cus) : true);
     const char* which = getenv("SBA_DKV_KERNEL");
     const bool plain = which && !strcmp(which, "plain");
     // the stream with eight half-block producers (12 waves): measured within 1 % of the one with four
@@ -1710,8 +1713,12 @@ int sba_launch_mfma_bwd(const sba::KParams& kp_in, int phases, hipStream_t s) {
     if (stream && !kp.q_scaled.ptr) return SBA_ERR_WORKSPACE;
     if (!stream) kp.q_scaled.ptr = nullptr;
     if (kp.head_dim == 64) {
-        // small grids last as long as their longest sweep: take the variant that halves it
-        if (p1 && grid.x <= sba_two_step_max_grid(kTwoStepDqMaxGrid)) hipLaunchKernelGGL((mfma_bwd_dq2_kernel<64>), grid, dim3(2 * kThreads), 0, s, kp);
+        // Small grids that last as long as their longest sweep (tail ratio from 3.7: B=1, H=16 up to T=4096) take the
+        // variant that halves it; batches of short sequences on the same number of workgroups do not (B=8, T=512:
+        // 23.8 us with one step per iteration against 27.4, B=4, T=1024 36.0 against 37.7).
+        const bool two_steps = sba_two_step_env() >= 0 ? grid.x <= (unsigned)sba_two_step_env()
+                                                       : grid.x <= kTwoStepDqMaxGrid && sba_tail_ratio(kp, grid.x) >= 3.7;
+        if (p1 && two_steps) hipLaunchKernelGGL((mfma_bwd_dq2_kernel<64>), grid, dim3(2 * kThreads), 0, s, kp);
         else if (p1 && lean_dq_kernel(grid.x >= 8u * cus)) hipLaunchKernelGGL((mfma_bwd_dq_kernel<64, true>), grid, dim3(kThreads), 0, s, kp);
         else if (p1) hipLaunchKernelGGL((mfma_bwd_dq_kernel<64>), grid, dim3(kThreads), 0, s, kp);
         if (p2 && plain) {

@@ -354,12 +354,8 @@ __global__ __launch_bounds__(G * kThreads) void mfma_fwd_seg_kernel(KParams p) {
 
 // Key segments per sweep for the forward at head_dim 64: 4, 2, or 0 = one sweep per workgroup.
 //
-// What decides is how long the launch's longest sweep is against the work of an average workgroup slot.  With
-// one sweep per workgroup a CU holds four workgroups, so the launch has 4 x CUs slots; it cannot end before its
-// longest sweep has, and if that sweep is several times the average slot's work, most of the chip idles behind it.
-//     r = longest sweep x slots / all sweep steps of the launch
-// (steps of 64 keys; a sequence of n row blocks has n (n + 1) of them per head, which is also its number of
-// carry-table columns).  Two segments halve the longest sweep at 8 waves per workgroup (two workgroups per CU),
+// What decides is how long the launch's longest sweep is against the work of an average workgroup slot, the tail
+// ratio r of sba_tail_ratio().  Two segments halve the longest sweep at 8 waves per workgroup (two workgroups per CU),
 // four quarter it at 16 waves (one workgroup per CU: worth it only while the grid is at most two rounds of them).
 // Measured on MI355X, forward time in us, one sweep / two segments / four segments:
 //     B=1 H=16 T=3584 (r 4.4)   64.8 / 55.8 / 51.1      B=2 H=16 T=2304 (r 3.4)   47.7 / 42.6 / 52.4
@@ -382,12 +378,8 @@ static int forward_segments(const sba::KParams& kp, unsigned grid) {
     const int forced = e ? atoi(e) : 0;
     const bool force = forced == 2 || forced == 3 || forced == 4;
     if (sba_two_step_env() >= 0) return grid <= (unsigned)sba_two_step_env() ? (force ? forced : 4) : 0;
-    const double cus = sba_cu_count();
-    const double longest = 2.0 * ((kp.seq_len + sba::kRowBlock - 1) / sba::kRowBlock);
-    double steps = (double)(kp.tab_head_stride / sba::kRowBlock) * kp.n_heads;
-    if (steps <= 0) steps = (double)grid * (longest / 2 + 1);          // (no table size given: every sweep half the longest)
-    const double r = longest * 4.0 * cus / steps;
-    const int segments = (r >= 3.8 && grid <= 2 * (unsigned)cus) ? 4 : (r >= 2.7 ? 2 : 0);
+    const double r = sba_tail_ratio(kp, grid);
+    const int segments = (r >= 3.8 && grid <= 2u * (unsigned)sba_cu_count()) ? 4 : (r >= 2.7 ? 2 : 0);
     return segments && force ? forced : segments;
 }
 
