@@ -352,7 +352,7 @@ __global__ __launch_bounds__(G * kThreads) void mfma_fwd_seg_kernel(KParams p) {
 
 }  // namespace sba
 
-// Key segments per sweep for the forward at head_dim 64: 4, 2, or 0 = one sweep per workgroup.
+// Key segments per sweep for the forward: 4 or 2 (head_dim 128: 2), or 0 = one sweep per workgroup.
 //
 // What decides is how long the launch's longest sweep is against the work of an average workgroup slot, the tail
 // ratio r of sba_tail_ratio().  Two segments halve the longest sweep at 8 waves per workgroup (two workgroups per CU),
@@ -373,7 +373,14 @@ __global__ __launch_bounds__(G * kThreads) void mfma_fwd_seg_kernel(KParams p) {
 // SBA_FWD_GROUPS=2|3|4 forces the number of segments where the rule picks any; SBA_TWO_STEP_MAX_GRID=n replaces
 // the rule by "segments (4, or as forced) up to n workgroups".
 static int forward_segments(const sba::KParams& kp, unsigned grid) {
-    if (kp.head_dim != 64) return 0;
+    if (kp.head_dim == 128) {
+        // head_dim 128: the one-sweep kernel holds two workgroups per CU, the two-segment one (8 waves, 129 KB of
+        // LDS) one; it pays while the grid is at most two rounds of those and the longest sweep dominates.  B=1,
+        // H=16, one sweep / two segments in us: T=1024 29.8 / 26.2, T=2048 50.4 / 41.6, T=3072 77.2 / 60.0, T=4096
+        // 105.5 / 91.8, T=5120 131.1 / 138.7, T=8192 276.2 / 291.7; B=2 T=2048 60.0 / 57.0; H=8 T=4096 89.7 / 70.8.
+        if (sba_two_step_env() >= 0) return grid <= (unsigned)sba_two_step_env() ? 2 : 0;
+        return grid <= 2u * (unsigned)sba_cu_count() && sba_tail_ratio(kp, grid) >= 3.7 ? 2 : 0;
+    }
     const char* e = getenv("SBA_FWD_GROUPS");
     const int forced = e ? atoi(e) : 0;
     const bool force = forced == 2 || forced == 3 || forced == 4;
@@ -384,9 +391,10 @@ static int forward_segments(const sba::KParams& kp, unsigned grid) {
 }
 
 template <bool kCarryOnly>
-static void launch_seg64(int groups, dim3 grid, hipStream_t s, const sba::KParams& kp) {
+static void launch_seg(int groups, dim3 grid, hipStream_t s, const sba::KParams& kp) {
     using namespace sba;
-    if (groups == 2) hipLaunchKernelGGL((mfma_fwd_seg_kernel<64, 2, kCarryOnly>), grid, dim3(2 * kThreads), 0, s, kp);
+    if (kp.head_dim == 128) hipLaunchKernelGGL((mfma_fwd_seg_kernel<128, 2, kCarryOnly>), grid, dim3(2 * kThreads), 0, s, kp);
+    else if (groups == 2) hipLaunchKernelGGL((mfma_fwd_seg_kernel<64, 2, kCarryOnly>), grid, dim3(2 * kThreads), 0, s, kp);
     else if (groups == 3) hipLaunchKernelGGL((mfma_fwd_seg_kernel<64, 3, kCarryOnly>), grid, dim3(3 * kThreads), 0, s, kp);
     else hipLaunchKernelGGL((mfma_fwd_seg_kernel<64, 4, kCarryOnly>), grid, dim3(4 * kThreads), 0, s, kp);
 }
@@ -396,8 +404,8 @@ int sba_launch_mfma_fwd(const sba::KParams& kp, hipStream_t s) {
     dim3 grid((unsigned)kp.n_jobs * kp.n_heads);
     const int segments = forward_segments(kp, grid.x);
     if (segments) {
-        if (kp.carry_only) launch_seg64<true>(segments, grid, s, kp);
-        else launch_seg64<false>(segments, grid, s, kp);
+        if (kp.carry_only) launch_seg<true>(segments, grid, s, kp);
+        else launch_seg<false>(segments, grid, s, kp);
     } else if (kp.head_dim == 64) {
         if (kp.carry_only) hipLaunchKernelGGL((mfma_fwd_kernel<64, true>), grid, dim3(kThreads), 0, s, kp);
         else hipLaunchKernelGGL((mfma_fwd_kernel<64, false>), grid, dim3(kThreads), 0, s, kp);
