@@ -70,6 +70,9 @@ def _bind_schedule(p, q, cu_seqlens, max_seqlens):
     if max_len > max_seqlens:
         raise ValueError(f"max_seqlens={max_seqlens} is smaller than the longest document ({max_len})")
     p.cu_seqlens, p.schedule, p.n_schedule, p.table_cols = cu_dev.data_ptr(), sched.data_ptr(), n_jobs, cols
+    # the library chooses its kernels from the longest sweep of the launch: give it the real longest document,
+    # which max_seqlens may only bound
+    p.seq_len = max(max_len, 1)
     return n_jobs
 
 

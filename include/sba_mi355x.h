@@ -79,7 +79,8 @@ typedef struct SbaParams {
     int32_t  dtype;            /* SBA_DTYPE_*: element type of q,k,v,o,rem,do,drem,dq,dk,dv */
     int32_t  n_seq;            /* B (dense) or number of documents (packed) */
     int32_t  n_heads;
-    int32_t  seq_len;          /* T (dense) or max document length (packed) */
+    int32_t  seq_len;          /* T (dense) or max document length (packed: an upper bound is accepted; the kernels
+                                  are chosen from it, so the exact longest document chooses best) */
     int32_t  total_tokens;     /* T (dense) or sumT (packed) */
     int32_t  head_dim;         /* D */
     int32_t  attend_current;   /* 0: keys j < i;  1: keys j <= i */
