@@ -386,7 +386,7 @@ def test_small_and_large_grids_take_different_forward_kernels_and_agree(monkeypa
 
 @pytest.mark.parametrize("D", [64, 128])
 def test_small_and_large_grids_take_different_backward_kernels_and_agree(D):
-    # <= 512 workgroups: two-step-per-iteration dQ kernel (d = 64); above: one step per iteration.
+    # few workgroups with one dominating sweep: two-step-per-iteration dQ kernel (d = 64); many: one step per iteration.
     # Key-owner pass: the resident stream (d = 64) or the 64-key-block kernel (d = 128) on the
     # small grid, the kernel whose waves own their keys on the large one.
     sb_attn, _ = _ops()
@@ -550,7 +550,8 @@ def test_randomized_packed_batches_mfma_vs_generic_backward(dkv_kernel, D, monke
 def test_both_arrangements_of_the_one_step_dq_kernel_against_the_oracle(which, monkeypatch):
     # head_dim 64, grids above the two-step kernels' range: the library picks between the two arrangements of the
     # dQ kernel by launch size; each is forced here on a packed and a dense problem (ragged ends, both masks)
-    # (every problem has more than 512 workgroups: 36, 36 and 17 row blocks times 16, 16 and 32 heads)
+    # (576, 576 and 544 workgroups - 36, 36 and 17 row blocks times 16, 16 and 32 heads - none of which hangs on one
+    # long sweep, so none takes the two-step kernel)
     monkeypatch.setenv("SBA_DQ_KERNEL", which)
     _check_varlen(16, 64, [300, 1, 129, 64, 517, 31, 1000, 128, 77, 640, 900], torch.bfloat16, False, seed=41)
     _check_varlen(16, 64, [2100, 65, 2300], torch.bfloat16, True, seed=42)
