@@ -167,3 +167,26 @@ def test_config5_full_size_training_steps():
     print("cfg5 losses", losses, flush=True)
     assert abs(losses[0] - math.log(32000)) < 0.5            # random init: about ln(vocabulary)
     assert losses[-1] < losses[0]
+
+
+def test_mid_size_launch_with_one_long_sweep_takes_the_two_segment_forward_and_matches_the_oracle(monkeypatch):
+    # B=1, H=16, T=5120, d=64: 640 workgroups whose longest sweep is three times the work of an average workgroup
+    # slot - the library runs its forward with two key segments per workgroup (8 waves), its dQ pass with one step
+    # per iteration and its dK/dV pass as the resident stream.  One head against the oracle, forward and gradients;
+    # the forward forced to three and four segments must agree with it to the forward tolerance.
+    from flame_amd import sb_attn
+    monkeypatch.delenv("SBA_FWD_GROUPS", raising=False)
+    B, H, T, D = 1, 16, 5120, 64
+    q, k, v = (randn((B, H, T, D), 340 + i, 0.5, torch.bfloat16) for i in range(3))
+    do = randn((B, H, T, D), 343, 1.0, torch.bfloat16)
+    print("B=1 H=16 T=5120: two-segment forward", flush=True)
+    qg, kg, vg = (x.cuda().requires_grad_(True) for x in (q, k, v))
+    o, rem = sb_attn(qg, kg, vg)
+    torch.autograd.backward([o], [do.cuda()])
+    _against_oracle_per_head(q, k, v, do, None, o, rem, (qg.grad, kg.grad, vg.grad), [7],
+                             "B=1 H=16 T=5120 (two-segment forward)")
+    for groups in ("3", "4"):
+        monkeypatch.setenv("SBA_FWD_GROUPS", groups)
+        with torch.no_grad():
+            og, rg = sb_attn(qg, kg, vg)
+        assert max_abs(o.float(), og.float()) <= 2e-2 and max_abs(rem.float(), rg.float()) <= 2e-2
