@@ -315,13 +315,16 @@ __global__ __launch_bounds__(2 * kThreads, 2) void mfma_bwd_dq2_kernel(KParams p
             kc.issue((step + 2) * kKeyBlock, job.len, my_tiles + (buf ^ 1) * 4 * kTile);
             vc.issue((step + 2) * kKeyBlock, job.len, my_tiles + (buf ^ 1) * 4 * kTile + kTile);
         }
-        float x[32], beta[32], dp[32];
-        float total = 0.f, start = 0.f;
+        // (an active wave's whole step sits in one branch, exchange barrier included: were the step split around the
+        // barrier, its 64 weights and gradients would have to hold a value on the idle path too, and the compiler
+        // clears half of them at the top of every step)
         if (active) {
+            float x[32], beta[32], dp[32];
+            float total = 0.f;
             score_tiles_ps<D, true>(x, ktile, lo, qf);
             if (key0 + 63 + strict > q0w) mask_step(x, key0 + 32 * h, qi, strict);
             const float Lend = carried_weights_and_dp<D>(x, beta, dp, F, vtile, lo, dof);
-            start = logit_grads_local(x, dp, total, lane);
+            float start = logit_grads_local(x, dp, total, lane);
             // the gradient of rem rides in the prefix as the constant d_rem * rem (see the one-step
             // kernel).  The leftmost block is group 0's first step: the constant joins its total
             // (which carries it to the other group and into Gc) and its own prefix
@@ -332,14 +335,12 @@ __global__ __launch_bounds__(2 * kThreads, 2) void mfma_bwd_dq2_kernel(KParams p
                 total += c0;
                 start += c0;
             }
-        }
-        if (h == 0) xch[grp][32 * qs + n] = total;
-        __syncthreads();
-        const float other = xch[grp ^ 1][32 * qs + n];
-        // group 1 holds the right step of the pair: its prefix also contains group 0's total
-        const float Gmy = grp == 0 ? Gc : Gc + other;
-        Gc = Gc + total + other;
-        if (active) {
+            if (h == 0) xch[grp][32 * qs + n] = total;
+            __syncthreads();
+            const float other = xch[grp ^ 1][32 * qs + n];
+            // group 1 holds the right step of the pair: its prefix also contains group 0's total
+            const float Gmy = grp == 0 ? Gc : Gc + other;
+            Gc = Gc + total + other;
             const float Glane = Gmy + start;       // the prefix entering this lane's 32 keys: block edge or middle (see the one-step kernel)
             Gstore = Glane;
             g_pending = true;
@@ -352,6 +353,10 @@ __global__ __launch_bounds__(2 * kThreads, 2) void mfma_bwd_dq2_kernel(KParams p
 #pragma unroll
                 for (int c = 0; c < 4; ++c)
                     dqacc[db] = mfma(fetch_cols_o<D>(ktile, lo, db, c), zf[c], dqacc[db]);
+        } else {
+            if (h == 0) xch[grp][32 * qs + n] = 0.f;
+            __syncthreads();
+            Gc = Gc + xch[grp ^ 1][32 * qs + n];
         }
         rcur += 2 * tstride;
         wait_global_memory();                  // the next tiles have landed
@@ -720,14 +725,16 @@ __global__ __launch_bounds__((NP + 4) * 64, NP == 4 ? 2 : 3) void mfma_bwd_dkv_s
                 const int q0w = (cur.job.rb + it) * kRowBlock + 32 * w4;
                 const int qi = q0w + n;
                 const bool skip = key0 + strict > q0w + 31 || q0w >= len || key0 >= len;
-                float x[16], beta[16], dp[16];
-                float Gt = 0.f;
+                // (one branch holds the whole step of a wave that has work: split in two around barrier X, the
+                // weights would be values that "flow" through the idle path as well, and the compiler then keeps
+                // a copy of all of them across the loop)
                 if (!skip) {
+                    float x[16], beta[16], dp[16];
                     const float4 cv = *(const float4*)(carry + (s & 1) * kCarry + (32 * w4 + n) * 16);
                     // table entries of pairs that no query of the row sees are not written
                     const bool sees = qi < len && qi - strict - key0 + 1 > 0;
                     const float Rt = sees ? (kh ? cv.x : cv.z) : 1.0f;
-                    Gt = sees ? (kh ? cv.w : cv.y) : 0.0f;
+                    const float Gt = sees ? (kh ? cv.w : cv.y) : 0.0f;
                     bf16x8 qf[D / 16], dof[D / 16];
 #pragma unroll
                     for (int ks = 0; ks < D / 16; ++ks) {
@@ -753,11 +760,7 @@ __global__ __launch_bounds__((NP + 4) * 64, NP == 4 ? 2 : 3) void mfma_bwd_dkv_s
                     });
 #pragma unroll
                     for (int r = 0; r < 16; ++r) dp[r] = dacc[r];
-                }
-                if (x_now) __syncthreads();    // X
-                // (the two cases store separately: one store sequence fed from either case costs the common one a
-                // register copy per value)
-                if (!skip) {
+                    if (x_now) __syncthreads();    // X
                     own_tile_grads(x, beta, dp, Gt, lane);
 #pragma unroll
                     for (int c = 0; c < 2; ++c) {
@@ -765,6 +768,7 @@ __global__ __launch_bounds__((NP + 4) * 64, NP == 4 ? 2 : 3) void mfma_bwd_dkv_s
                         *(bf16x8*)(zd + tile_offset<64>(32 * w4 + n, 4 * kh + 2 * h + c)) = pack8(&dp[8 * c]);
                     }
                 } else {
+                    if (x_now) __syncthreads();    // X
                     const bf16x8 none = {0, 0, 0, 0, 0, 0, 0, 0};
 #pragma unroll
                     for (int c = 0; c < 2; ++c) {
@@ -809,9 +813,9 @@ __global__ __launch_bounds__((NP + 4) * 64, NP == 4 ? 2 : 3) void mfma_bwd_dkv_s
                 const int q0w = (cur.job.rb + it) * kRowBlock + 32 * w4;
                 const int qi = q0w + n;
                 const bool skip = key0 + strict > q0w + 31 || q0w >= len;
-                float x[32], beta[32], dp[32];
-                float Gc = 0.f;
+                // (one branch for the whole step, see above)
                 if (!skip) {
+                    float x[32], beta[32], dp[32];
                     // Both carries that enter this LANE's 32 keys come from the tables: the right half-wave
                     // takes the forward's block-edge product and the mid-block prefix, the left one the
                     // mid-block product and the block-edge prefix - no exchange between the halves, and the
@@ -822,7 +826,7 @@ __global__ __launch_bounds__((NP + 4) * 64, NP == 4 ? 2 : 3) void mfma_bwd_dkv_s
                     const float4 cv = *(const float4*)(carry + (s & 1) * kCarry + (32 * w4 + n) * 16);
                     const bool sees = qi < len && qi - strict - (key0 + 32 * h) + 1 > 0;
                     const float R = sees ? (h ? cv.x : cv.z) : (qi < len ? 1.0f : 0.0f);
-                    Gc = sees ? (h ? cv.w : cv.y) : 0.0f;
+                    const float Gc = sees ? (h ? cv.w : cv.y) : 0.0f;
                     bf16x8 qf[D / 16], dof[D / 16];
 #pragma unroll
                     for (int ks = 0; ks < D / 16; ++ks) {
@@ -854,11 +858,7 @@ __global__ __launch_bounds__((NP + 4) * 64, NP == 4 ? 2 : 3) void mfma_bwd_dkv_s
                     for (int t = 0; t < 2; ++t)
 #pragma unroll
                         for (int r = 0; r < 16; ++r) dp[16 * t + r] = dacc[t][r];
-                }
-                if (x_now) __syncthreads();    // X
-                // (the two cases store separately: one store sequence fed from either case costs the common one a
-                // register copy per value)
-                if (!skip) {
+                    if (x_now) __syncthreads();    // X
                     logit_grads_from<32>(x, beta, dp, Gc);
 #pragma unroll
                     for (int c = 0; c < 4; ++c) {
@@ -866,6 +866,7 @@ __global__ __launch_bounds__((NP + 4) * 64, NP == 4 ? 2 : 3) void mfma_bwd_dkv_s
                         *(bf16x8*)(zd + tile_offset<64>(32 * w4 + n, 4 * h + c)) = pack8(&dp[8 * c]);
                     }
                 } else {
+                    if (x_now) __syncthreads();    // X
                     const bf16x8 none = {0, 0, 0, 0, 0, 0, 0, 0};
 #pragma unroll
                     for (int c = 0; c < 4; ++c) {
