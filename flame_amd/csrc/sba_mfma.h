@@ -123,6 +123,18 @@ struct TileAt { int off; };
 // those waits.
 __device__ inline void wait_global_memory() { __builtin_amdgcn_s_waitcnt(0x0F70); }   // vmcnt(0)
 
+// Workgroup barrier for an exchange through LDS while tile DMAs are in flight.  __syncthreads() is a release fence
+// in front of the barrier; the compiler knows that a global -> LDS DMA writes LDS and makes the fence wait for the
+// vector-memory count to reach zero, i.e. for tiles that are only needed at the END of the step (and for every
+// outstanding global store).  Here: this wave's own LDS writes have completed (LDS count zero), then the barrier; the
+// signal fences keep the compiler from moving LDS accesses across it and emit nothing.
+__device__ inline void lds_exchange_barrier() {
+    __atomic_signal_fence(__ATOMIC_SEQ_CST);
+    __builtin_amdgcn_s_waitcnt(0xC07F);        // lgkmcnt(0), the other counts left alone
+    __builtin_amdgcn_s_barrier();
+    __atomic_signal_fence(__ATOMIC_SEQ_CST);
+}
+
 __device__ inline s16x4 lds_read_tr(const char* p) {
     return __builtin_amdgcn_ds_read_tr16_b64_v4i16(
         (__attribute__((address_space(3))) s16x4*)(uintptr_t)(uint32_t)(uintptr_t)p);
@@ -276,11 +288,25 @@ template <int D> struct TileCopy {
 // issues instructions w4, w4 + 4, ...  The per-lane byte offsets inside a tile never change, so
 // a step costs no vector address arithmetic.  Rows past the end of the sequence are clamped to
 // its last row instead of zero-filled: those keys are masked for every valid query.
+// The copy instruction is written as inline assembly.  Issued through the compiler's builtin, the compiler knows that it
+// writes LDS, cannot tell which part, and puts a wait for ALL vector-memory traffic in front of the next LDS access that
+// it cannot prove apart from the copy's destination: the first transposing fetch of every step (the V operands of the
+// forward, the K operands of the dQ pass, the Q / dO operands of the key-owner kernels) and every barrier that has a
+// release fence - all of them in the middle of a step, where the tile requested at its top (for the NEXT step) need not
+// have landed.  The kernels wait for their tiles themselves, at the end of the step (wait_global_memory() in front of
+// the barrier that publishes them).  A kernel that copies this way must not also use the builtin (the compiler would
+// not know that M0 has changed between two of its own copies).
 // kLateRagged: the lane's row and chunk for the one ragged tile of a sequence are worked out where that tile is
 // requested, from a copy of the lane index that the compiler cannot see through.  As loop invariants they are
 // otherwise computed once at the top of the kernel and occupy registers through the whole sweep: in the
 // register-lean dQ kernel that is the difference between four spilled registers and none.
-template <int D, bool kNatural = false, bool kScalarBase = true, bool kLateRagged = false> struct TileDma {      // kNatural: rows kept in their order (query tiles)
+// 64 lanes x 16 bytes from `base + off` (uniform base, 32-bit lane offset) to LDS bytes lds_addr .. lds_addr + 1023
+__device__ inline void dma16(const char* base, uint32_t off, uint32_t lds_addr) {
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %0" : : "s"(base), "v"(off), "s"(lds_addr) : "memory");
+}
+__device__ inline uint32_t lds_address(const char* p) { return (uint32_t)(uintptr_t)p; }   // (low half of the flat address)
+
+template <int D, bool kNatural = false, bool kLateRagged = false> struct TileDma {      // kNatural: rows kept in their order (query tiles)
     static constexpr int kPerWave = 64 * D * 2 / 1024 / 4;    // 2 (D=64) or 4 (D=128)
     uint32_t off[kPerWave];
     const char* origin;        // row 0 of the (sequence, head) slice: uniform
@@ -314,23 +340,11 @@ template <int D, bool kNatural = false, bool kScalarBase = true, bool kLateRagge
             off[i] = 2u * (uint32_t)(kl * st + c * 8);
         }
     }
-    // The 32-bit lane offset, opaque at each use: its widening to 64 bits then stays next to the load, which is
-    // what lets the load take "uniform base + 32-bit lane offset" as its address.  Widened once in front of the
-    // loop instead (where the compiler would move it), every load costs a 64-bit vector add.
-    // (kScalarBase = false leaves it to the compiler: the two-step dQ kernel is 1.7 % slower with it.)
-    __device__ static inline uint32_t fresh(uint32_t v) {
-        if (kScalarBase) asm volatile("" : "+v"(v));
-        return v;
-    }
     // a tile known to lie inside the sequence (every key tile of a sweep but the rightmost)
     __device__ inline void issue_full(int row0, char* tile) const {
         const char* tile_base = origin + (((uint64_t)(uint32_t)row0 * (uint32_t)st) << 1);
 #pragma unroll
-        for (int i = 0; i < kPerWave; ++i)
-            __builtin_amdgcn_global_load_lds(
-                (const __attribute__((address_space(1))) void*)(tile_base + (size_t)fresh(off[i])),
-                (__attribute__((address_space(3))) void*)(uintptr_t)(uint32_t)(uintptr_t)(tile + (w4 + 4 * i) * 1024),
-                16, 0, 0);
+        for (int i = 0; i < kPerWave; ++i) dma16(tile_base, off[i], lds_address(tile + (w4 + 4 * i) * 1024));
     }
     __device__ inline void issue(int row0, int len, char* tile) const {
         // uniform; row0 and the stride are non-negative: the unsigned product is two scalar instructions, the
@@ -338,11 +352,7 @@ template <int D, bool kNatural = false, bool kScalarBase = true, bool kLateRagge
         const char* tile_base = origin + (((uint64_t)(uint32_t)row0 * (uint32_t)st) << 1);
         if (row0 + 64 <= len) {
 #pragma unroll
-            for (int i = 0; i < kPerWave; ++i)
-                __builtin_amdgcn_global_load_lds(
-                    (const __attribute__((address_space(1))) void*)(tile_base + (size_t)fresh(off[i])),
-                    (__attribute__((address_space(3))) void*)(uintptr_t)(uint32_t)(uintptr_t)(tile + (w4 + 4 * i) * 1024),
-                    16, 0, 0);
+            for (int i = 0; i < kPerWave; ++i) dma16(tile_base, off[i], lds_address(tile + (w4 + 4 * i) * 1024));
         } else {
             int lane_here = lane;
             if (kLateRagged) asm volatile("" : "+v"(lane_here));
@@ -351,10 +361,7 @@ template <int D, bool kNatural = false, bool kScalarBase = true, bool kLateRagge
                 int kl, c;
                 where(w4 + 4 * i, lane_here, kl, c);
                 kl = min(kl, len - 1 - row0);
-                __builtin_amdgcn_global_load_lds(
-                    (const __attribute__((address_space(1))) void*)(tile_base + 2 * ((int64_t)kl * st + c * 8)),
-                    (__attribute__((address_space(3))) void*)(uintptr_t)(uint32_t)(uintptr_t)(tile + (w4 + 4 * i) * 1024),
-                    16, 0, 0);
+                dma16(tile_base, 2u * (uint32_t)(kl * st + c * 8), lds_address(tile + (w4 + 4 * i) * 1024));
             }
         }
     }
@@ -685,7 +692,11 @@ __device__ inline void stick_weights_and_dp(float (&x)[32], float (&beta)[32], f
 
 // The same from this lane's own carry F (carried_chain_with): finished weights, beta and dP; returns the carry
 // leaving the lane's keys.
-template <int D, class Tile>
+// kPaced: the wave lowers its issue priority as it moves through the chain (3 for the first two 4-key segments, then 2,
+// 1, 0).  Two waves of a SIMD that run this chain side by side otherwise issue oldest first: the older one runs as if
+// alone and then idles at the next barrier while the younger one finishes at the rate of a single wave.  With the
+// priority tied to progress, whichever wave is behind goes first and both arrive together.
+template <int D, bool kPaced = false, class Tile>
 __device__ inline float carried_weights_and_dp(float (&x)[32], float (&beta)[32], float (&dp)[32], float F,
                                                Tile vtile, const LaneOffsets<D>& o, const bf16x8 (&dof)[D / 16]) {
     constexpr int kPer = D / 64;
@@ -693,7 +704,13 @@ __device__ inline float carried_weights_and_dp(float (&x)[32], float (&beta)[32]
     bf16x8 nx[kPer];
 #pragma unroll
     for (int i = 0; i < kPer; ++i) nx[i] = fetch_rows_o<D>(vtile, o, i & 1, i >> 1);
+    if (kPaced) __builtin_amdgcn_s_setprio(3);
     const float Lend = carried_chain_with<true, 32>(x, beta, F, [&](int seg) {
+        if (kPaced) {
+            if (seg == 1) __builtin_amdgcn_s_setprio(2);
+            else if (seg == 3) __builtin_amdgcn_s_setprio(1);
+            else if (seg == 5) __builtin_amdgcn_s_setprio(0);
+        }
         bf16x8 cur[kPer];
 #pragma unroll
         for (int i = 0; i < kPer; ++i) cur[i] = nx[i];

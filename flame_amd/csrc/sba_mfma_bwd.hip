@@ -83,7 +83,7 @@ __global__ __launch_bounds__(kThreads, (D == 64 && kLean) ? 3 : 2) void mfma_bwd
     const int kmax = imax - strict;
     const int n_steps = kmax >= 0 ? kmax / kKeyBlock + 1 : 0;
 
-    TileDma<D, false, true, D == 64 && kLean> kc, vc;
+    TileDma<D, false, D == 64 && kLean> kc, vc;
     kc.init(lane, wave, p.k, kbase);
     vc.init(lane, wave, p.v, vbase);
     if (n_steps > 0) {
@@ -272,7 +272,7 @@ __global__ __launch_bounds__(2 * kThreads, 2) void mfma_bwd_dq2_kernel(KParams p
     char* my_tiles = lds + grp * 2 * kTile;          // + buf * 4 * kTile
 
     // each group copies its own tiles (256 threads per tile pair)
-    TileDma<D, false, false> kc, vc;
+    TileDma<D> kc, vc;
     kc.init(lane, qs, p.k, kbase);
     vc.init(lane, qs, p.v, vbase);
     if (grp < n_steps) {
@@ -323,7 +323,7 @@ __global__ __launch_bounds__(2 * kThreads, 2) void mfma_bwd_dq2_kernel(KParams p
             float total = 0.f;
             score_tiles_ps<D, true>(x, ktile, lo, qf);
             if (key0 + 63 + strict > q0w) mask_step(x, key0 + 32 * h, qi, strict);
-            const float Lend = carried_weights_and_dp<D>(x, beta, dp, F, vtile, lo, dof);
+            const float Lend = carried_weights_and_dp<D, true>(x, beta, dp, F, vtile, lo, dof);
             float start = logit_grads_local(x, dp, total, lane);
             // the gradient of rem rides in the prefix as the constant d_rem * rem (see the one-step
             // kernel).  The leftmost block is group 0's first step: the constant joins its total
@@ -336,7 +336,7 @@ __global__ __launch_bounds__(2 * kThreads, 2) void mfma_bwd_dq2_kernel(KParams p
                 start += c0;
             }
             if (h == 0) xch[grp][32 * qs + n] = total;
-            __syncthreads();
+            lds_exchange_barrier();            // (not __syncthreads(): that would wait here for the next tiles)
             const float other = xch[grp ^ 1][32 * qs + n];
             // group 1 holds the right step of the pair: its prefix also contains group 0's total
             const float Gmy = grp == 0 ? Gc : Gc + other;
@@ -355,7 +355,7 @@ __global__ __launch_bounds__(2 * kThreads, 2) void mfma_bwd_dq2_kernel(KParams p
                     dqacc[db] = mfma(fetch_cols_o<D>(ktile, lo, db, c), zf[c], dqacc[db]);
         } else {
             if (h == 0) xch[grp][32 * qs + n] = 0.f;
-            __syncthreads();
+            lds_exchange_barrier();
             Gc = Gc + xch[grp ^ 1][32 * qs + n];
         }
         rcur += 2 * tstride;
