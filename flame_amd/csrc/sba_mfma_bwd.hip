@@ -981,12 +981,10 @@ __global__ __launch_bounds__((NP + 4) * 64, NP == 4 ? 2 : 3) void mfma_bwd_dkv_s
                 const int kl = NP == 4 ? (((r >> 2) & 1) << 5) | (((r >> 5) & 1) << 4) | (((r >> 3) & 3) << 2) | (r & 3)
                                        : (((r >> 5) & 1) << 5) | (((r >> 2) & 1) << 4) | (((r >> 3) & 3) << 2) | (r & 3);
                 const int row = min(t.key0 + kl, t.job.len - 1);
-                __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(p.k.ptr + 2 * (kbase + (int64_t)row * p.k.st + c * 8)),
-                                                 (__attribute__((address_space(3))) void*)(uintptr_t)(uint32_t)(uintptr_t)(ktile + inst * 1024),
-                                                 16, 0, 0);
-                __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(p.v.ptr + 2 * (vbase + (int64_t)row * p.v.st + c * 8)),
-                                                 (__attribute__((address_space(3))) void*)(uintptr_t)(uint32_t)(uintptr_t)(vdst + inst * 1024),
-                                                 16, 0, 0);
+                // (the copy as inline assembly, see TileDma: through the builtin, the first LDS fetch of EVERY iteration's
+                // reduction waited for all vector-memory traffic, the tiles just requested for step s + 2 included)
+                dma16(p.k.ptr + 2 * kbase, 2u * (uint32_t)(row * (int)p.k.st + c * 8), lds_address(ktile + inst * 1024));
+                dma16(p.v.ptr + 2 * vbase, 2u * (uint32_t)(row * (int)p.v.st + c * 8), lds_address(vdst + inst * 1024));
             }
         };
         auto deposit = [&](int s) {
