@@ -123,18 +123,6 @@ struct TileAt { int off; };
 // those waits.
 __device__ inline void wait_global_memory() { __builtin_amdgcn_s_waitcnt(0x0F70); }   // vmcnt(0)
 
-// Workgroup barrier for an exchange through LDS while tile DMAs are in flight.  __syncthreads() is a release fence
-// in front of the barrier; the compiler knows that a global -> LDS DMA writes LDS and makes the fence wait for the
-// vector-memory count to reach zero, i.e. for tiles that are only needed at the END of the step (and for every
-// outstanding global store).  Here: this wave's own LDS writes have completed (LDS count zero), then the barrier; the
-// signal fences keep the compiler from moving LDS accesses across it and emit nothing.
-__device__ inline void lds_exchange_barrier() {
-    __atomic_signal_fence(__ATOMIC_SEQ_CST);
-    __builtin_amdgcn_s_waitcnt(0xC07F);        // lgkmcnt(0), the other counts left alone
-    __builtin_amdgcn_s_barrier();
-    __atomic_signal_fence(__ATOMIC_SEQ_CST);
-}
-
 __device__ inline s16x4 lds_read_tr(const char* p) {
     return __builtin_amdgcn_ds_read_tr16_b64_v4i16(
         (__attribute__((address_space(3))) s16x4*)(uintptr_t)(uint32_t)(uintptr_t)p);

@@ -336,7 +336,7 @@ __global__ __launch_bounds__(2 * kThreads, 2) void mfma_bwd_dq2_kernel(KParams p
                 start += c0;
             }
             if (h == 0) xch[grp][32 * qs + n] = total;
-            lds_exchange_barrier();            // (not __syncthreads(): that would wait here for the next tiles)
+            __syncthreads();
             const float other = xch[grp ^ 1][32 * qs + n];
             // group 1 holds the right step of the pair: its prefix also contains group 0's total
             const float Gmy = grp == 0 ? Gc : Gc + other;
@@ -355,7 +355,7 @@ __global__ __launch_bounds__(2 * kThreads, 2) void mfma_bwd_dq2_kernel(KParams p
                     dqacc[db] = mfma(fetch_cols_o<D>(ktile, lo, db, c), zf[c], dqacc[db]);
         } else {
             if (h == 0) xch[grp][32 * qs + n] = 0.f;
-            lds_exchange_barrier();
+            __syncthreads();
             Gc = Gc + xch[grp ^ 1][32 * qs + n];
         }
         rcur += 2 * tstride;
