@@ -1704,8 +1704,8 @@ int sba_launch_mfma_bwd(const sba::KParams& kp_in, int phases, hipStream_t s) {
     const bool own = own_keys_kernel(kp.head_dim == 64 ? grid.x >= 3u * cus || (short_sweeps && grid.x >= 2u * cus) : true);
     const char* which = getenv("SBA_DKV_KERNEL");
     const bool plain = which && !strcmp(which, "plain");
-    // the stream with eight half-block producers (12 waves): measured within 1 % of the one with four
-    // full-block producers (109.1 against 110.3 us at B=1 H=16 T=4096), which stays the default
+    // the stream with eight half-block producers (12 waves): behind the one with four full-block producers
+    // (107 against 99.5 us at B=1 H=16 T=4096), which stays the default
     const bool stream8 = which && !strcmp(which, "stream8");
     // the scaled copy of q is for the stream kernel: no other key-owner kernel reads it, so the dQ pass skips it
     const bool stream = kp.head_dim == 64 && !plain && !own;
