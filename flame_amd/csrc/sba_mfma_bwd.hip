@@ -1730,11 +1730,12 @@ int sba_launch_mfma_bwd(const sba::KParams& kp_in, int phases, hipStream_t s) {
         const bool two_steps = sba_two_step_env() >= 0 ? grid.x <= (unsigned)sba_two_step_env()
                                                        : grid.x <= kTwoStepDqMaxGrid && sba_tail_ratio(kp, grid.x) >= 3.7;
         if (p1 && two_steps) hipLaunchKernelGGL((mfma_bwd_dq2_kernel<64>), grid, dim3(2 * kThreads), 0, s, kp);
-        // The register-lean arrangement (three waves per SIMD) from four workgroups per CU on, unless the launch hangs on
+        // The register-lean arrangement (three waves per SIMD) from five workgroups per CU on, unless the launch hangs on
         // one long sweep (tail ratio above 2.5: there the plain arrangement's shorter step is ahead, e.g. 111 against 118 us
-        // on an 8192-token pack with a 4096-token document); from eight workgroups per CU on always.  On 1024-3232
-        // workgroups of 21 dense and packed shapes it is 1-7 % ahead of the plain one.
-        else if (p1 && lean_dq_kernel(grid.x >= 8u * cus || (grid.x >= 4u * cus && sba_tail_ratio(kp, grid.x) <= 2.5)))
+        // on an 8192-token pack with a 4096-token document); from eight workgroups per CU on always.  On 1280-3232
+        // workgroups of 15 dense and packed shapes it is 0-5 % ahead of the plain one; at four workgroups per CU (six
+        // shapes of 1024 workgroups) the plain one is, by 1-3 %.
+        else if (p1 && lean_dq_kernel(grid.x >= 8u * cus || (grid.x >= 5u * cus && sba_tail_ratio(kp, grid.x) <= 2.5)))
             hipLaunchKernelGGL((mfma_bwd_dq_kernel<64, true>), grid, dim3(kThreads), 0, s, kp);
         else if (p1) hipLaunchKernelGGL((mfma_bwd_dq_kernel<64>), grid, dim3(kThreads), 0, s, kp);
         if (p2 && plain) {
