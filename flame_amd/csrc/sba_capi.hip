@@ -74,7 +74,7 @@ int scratch_tables(const SbaParams* p) { return forward_tables(p) * (p->workspac
 // the bounded waits (and with them the error word) exist in the bf16 matrix-core backward only
 bool has_error_word(const SbaParams* p) { return use_mfma_bwd(p) && p->dtype == SBA_DTYPE_BF16; }
 // bf16 at head_dim 64: the dQ pass leaves a copy of q times the logit scale (bf16, [sequence][head][token][64], dense)
-// behind the tables, for the key-owner kernels, whose score MFMAs then deliver the same base-2 logits as the dQ pass's
+// behind the tables, for the key-owner stream kernel, whose score MFMAs then deliver base-2 logits
 size_t scaled_q_bytes(const SbaParams* p) {
     if (!use_mfma_bwd(p) || p->dtype != SBA_DTYPE_BF16 || p->head_dim != 64) return 0;
     size_t b = (size_t)tab_tokens(p) * p->n_heads * 64 * 2;

@@ -38,7 +38,7 @@ struct KParams {
     float* gmid;                   // the prefix entering the block's RIGHT 32 keys (written by the dQ pass, like gtab);
                                    //   the bf16 dQ kernels rely on gmid - rtab == gtab - rmid
     TensorArg q_scaled;            // bf16 head_dim 64 backward: q times scale2, rounded to bf16, written by the dQ pass for
-                                   //   the key-owner kernels, which read it in place of q (ptr NULL: not wanted)
+                                   //   the key-owner stream kernel (ptr NULL: not wanted)
     float* dkv32;                  // generic path: fp32 dk|dv accumulators
     int* gave_up;                  // backward error word (set if a kernel abandoned a bounded internal wait)
     int64_t tab_head_stride;       // floats per head in each carry table

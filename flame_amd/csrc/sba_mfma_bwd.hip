@@ -437,11 +437,7 @@ __global__ __launch_bounds__(kThreads, 2) void mfma_bwd_dkv_kernel(KParams p) {
     const int key0 = kb * kKeyBlock;
     if (key0 >= job.len) return;               // uniform over the workgroup
     const int strict = p.attend_current ? 0 : 1;
-    // (Q from the dQ pass's scaled copy where there is one, K then unscaled: the logits of the other passes, see the
-    // own-keys kernel)
-    const bool scaled_q = D == 64 && p.q_scaled.ptr != nullptr;
-    const TensorArg& qt = scaled_q ? p.q_scaled : p.q;
-    const int64_t qbase = (int64_t)job.seq * qt.sb + (int64_t)head * qt.sh + (int64_t)job.tok0 * qt.st;
+    const int64_t qbase = (int64_t)job.seq * p.q.sb + (int64_t)head * p.q.sh + (int64_t)job.tok0 * p.q.st;
     const int64_t kbase = (int64_t)job.seq * p.k.sb + (int64_t)head * p.k.sh + (int64_t)job.tok0 * p.k.st;
     const int64_t vbase = (int64_t)job.seq * p.v.sb + (int64_t)head * p.v.sh + (int64_t)job.tok0 * p.v.st;
     const int64_t dobase = (int64_t)job.seq * p.d_o.sb + (int64_t)head * p.d_o.sh + (int64_t)job.tok0 * p.d_o.st;
@@ -458,7 +454,7 @@ __global__ __launch_bounds__(kThreads, 2) void mfma_bwd_dkv_kernel(KParams p) {
         TileCopy<D> kc, vc;
         kc.load(p.k, kbase, key0, job.len);
         vc.load(p.v, vbase, key0, job.len);
-        if (!scaled_q) kc.scale(p.scale2);     // K times the logit scale: the score MFMAs deliver base-2 logits
+        kc.scale(p.scale2);                    // K times the logit scale: the score MFMAs deliver base-2 logits
         kc.store(ktile);
         vc.store(vtile);
     }
@@ -472,7 +468,7 @@ __global__ __launch_bounds__(kThreads, 2) void mfma_bwd_dkv_kernel(KParams p) {
     bf16x8 qfn[D / 16];
     {
         const int qi0 = qb0 * kRowBlock + 32 * wave + n;
-        load_row_frags<D>(qfn, qt, qbase, qi0, job.len, lane);
+        load_row_frags<D>(qfn, p.q, qbase, qi0, job.len, lane);
         if (qi0 < job.len) {
             const int64_t t = tab_index(p, head, job, qb0, kb) + 32 * wave + n;
             Rn = p.rtab[t]; Gn = p.gtab[t];
@@ -496,7 +492,7 @@ __global__ __launch_bounds__(kThreads, 2) void mfma_bwd_dkv_kernel(KParams p) {
         float R = Rn, Gc = Gn;
         if (qb + 1 < n_qb) {
             const int qin = qi + kRowBlock;
-            load_row_frags<D>(qfn, qt, qbase, qin, job.len, lane);
+            load_row_frags<D>(qfn, p.q, qbase, qin, job.len, lane);
             Rn = 1.0f; Gn = 0.0f;
             if (qin < job.len) {
                 const int64_t t = tab_index(p, head, job, qb + 1, kb) + 32 * wave + n;
@@ -554,7 +550,7 @@ __global__ __launch_bounds__(kThreads, 2) void mfma_bwd_dkv_kernel(KParams p) {
     char* stage_v = zd;
 #pragma unroll
     for (int i = 0; i < D / 64; ++i) {
-        stage_acc_tile<D>(stage_k, 32 * kh, 32 * (dbw + 2 * i), dkacc[i], scaled_q ? p.scale / p.scale2 : p.scale, lane);
+        stage_acc_tile<D>(stage_k, 32 * kh, 32 * (dbw + 2 * i), dkacc[i], p.scale, lane);
         stage_acc_tile<D>(stage_v, 32 * kh, 32 * (dbw + 2 * i), dvacc[i], 1.0f, lane);
     }
     __syncthreads();
@@ -1185,13 +1181,7 @@ __global__ __launch_bounds__(kThreads, D == 64 ? 2 : 1) void mfma_bwd_dkv_own_ke
     const int kb0 = q_begin + 32 * wave;               // first key of this wave
     char* ztile = lds + 2 * kNBuf * kQTile + wave * kZTile;
 
-    // Where the dQ pass has left its copy of q times scale * log2 e (bf16, head_dim 64), the Q tiles are taken from it
-    // and K stays as it is: the logits are then bit for bit those of the forward and of the dQ pass, whose carries and
-    // prefixes this kernel takes from the tables.  (With the scale folded into K instead, the logits differ from theirs
-    // by the rounding of the scaled K, and on the saturated golden vector dK's error is 0.051 instead of 0.031.)
-    const bool scaled_q = D == 64 && p.q_scaled.ptr != nullptr;
-    const TensorArg& qt = scaled_q ? p.q_scaled : p.q;
-    const int64_t qbase = (int64_t)job.seq * qt.sb + (int64_t)head * qt.sh + (int64_t)job.tok0 * qt.st;
+    const int64_t qbase = (int64_t)job.seq * p.q.sb + (int64_t)head * p.q.sh + (int64_t)job.tok0 * p.q.st;
     const int64_t kbase = (int64_t)job.seq * p.k.sb + (int64_t)head * p.k.sh + (int64_t)job.tok0 * p.k.st;
     const int64_t vbase = (int64_t)job.seq * p.v.sb + (int64_t)head * p.v.sh + (int64_t)job.tok0 * p.v.st;
     const int64_t dobase = (int64_t)job.seq * p.d_o.sb + (int64_t)head * p.d_o.sh + (int64_t)job.tok0 * p.d_o.st;
@@ -1204,7 +1194,7 @@ __global__ __launch_bounds__(kThreads, D == 64 ? 2 : 1) void mfma_bwd_dkv_own_ke
         const int key = kb0 + 16 * ((m >> 2) & 1) + 4 * (m >> 3) + (m & 3);
         load_row_frags<D>(kfr, p.k, kbase, key, job.len, lane);
         load_row_frags<D>(vfr, p.v, vbase, key, job.len, lane);
-        if (!scaled_q) prescale_frags(kfr, p.scale2);      // K times the logit scale: the score MFMAs deliver base-2 logits
+        prescale_frags(kfr, p.scale2);         // K times the logit scale: the score MFMAs deliver base-2 logits
     }
 
     f32x16 dkacc[D / 32], dvacc[D / 32];
@@ -1214,7 +1204,7 @@ __global__ __launch_bounds__(kThreads, D == 64 ? 2 : 1) void mfma_bwd_dkv_own_ke
     const int n_steps = q_begin < job.len ? (job.len - q_begin + kStep - 1) / kStep : 0;
 
     TileDma<D, true> qc, dc;
-    qc.init(lane, wave, qt, qbase);
+    qc.init(lane, wave, p.q, qbase);
     dc.init(lane, wave, p.d_o, dobase);
     if (n_steps > 0) {
         qc.issue(q_begin, job.len, lds);
@@ -1420,8 +1410,7 @@ __global__ __launch_bounds__(kThreads, D == 64 ? 2 : 1) void mfma_bwd_dkv_own_ke
         const int64_t ob = (int64_t)job.seq * out.sb + (int64_t)head * out.sh + (int64_t)job.tok0 * out.st;
 #pragma unroll
         for (int db = 0; db < D / 32; ++db)
-            stage_acc_tile<D>(ztile, 0, 32 * db, which == 0 ? dkacc[db] : dvacc[db],
-                              which == 0 ? (scaled_q ? p.scale / p.scale2 : p.scale) : 1.0f, lane);
+            stage_acc_tile<D>(ztile, 0, 32 * db, which == 0 ? dkacc[db] : dvacc[db], which == 0 ? p.scale : 1.0f, lane);
         for (int c = lane; c < 32 * D / 8; c += 64) {
             const int row = c / (D / 8), cc = c % (D / 8);
             if (kb0 + row < job.len)
@@ -1718,11 +1707,10 @@ int sba_launch_mfma_bwd(const sba::KParams& kp_in, int phases, hipStream_t s) {
     // the stream with eight half-block producers (12 waves): behind the one with four full-block producers
     // (107 against 99.5 us at B=1 H=16 T=4096), which stays the default
     const bool stream8 = which && !strcmp(which, "stream8");
-    // the scaled copy of q is for the key-owner kernels at head_dim 64 (the stream cannot do without it, the others
-    // fall back to scaling K); at head_dim 128 the dQ pass skips it
+    // the scaled copy of q is for the stream kernel: no other key-owner kernel reads it, so the dQ pass skips it
     const bool stream = kp.head_dim == 64 && !plain && !own;
     if (stream && !kp.q_scaled.ptr) return SBA_ERR_WORKSPACE;
-    if (kp.head_dim != 64) kp.q_scaled.ptr = nullptr;
+    if (!stream) kp.q_scaled.ptr = nullptr;
     if (kp.head_dim == 64) {
         // Small grids that last as long as their longest sweep (tail ratio from 3.7: B=1, H=16 up to T=4096) take the
         // variant that halves it; batches of short sequences on the same number of workgroups do not (B=8, T=512:

@@ -129,7 +129,7 @@ size_t sba_workspace_bytes(const SbaParams* p);
  * Bytes of device memory sba_bwd needs for the duration of the call only (the prefix tables that
  * its first kernel hands to its second - two in bf16, one in fp32 -, for bf16 at head_dim 64 also a
  * bf16 copy of q times the logit scale, total_tokens x n_heads x 128 bytes, which the first kernel
- * writes and the second reads in place of q (its logits are then those of the first); or the generic path's fp32 accumulators): allocate
+ * writes and the second reads in place of q; or the generic path's fp32 accumulators): allocate
  * before the call, free after it has run.  With bwd_phases 1 and 2 issued
  * as two calls, the same buffer goes to both.  For bf16 at head_dim 64 / 128 the last 256 bytes
  * hold an error word (int32): the first kernel of a backward (bwd_phases 0 or 1) clears it, and a
