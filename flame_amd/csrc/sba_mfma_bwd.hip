@@ -1565,6 +1565,7 @@ __global__ __launch_bounds__(2 * kThreads, 2) void mfma_bwd_dkv_pair_kernel(KPar
                 const float Rt = sees ? Rin : 1.0f;      // table entries of invisible pairs are not written
                 const float Gt = sees ? Gin : 0.0f;
                 float beta[16];
+                __builtin_amdgcn_s_setprio(3);     // paced like the two-step dQ kernel's chain: the wave behind goes first
                 {
                     f32x16 acc = {0};
 #pragma unroll
@@ -1596,7 +1597,9 @@ __global__ __launch_bounds__(2 * kThreads, 2) void mfma_bwd_dkv_pair_kernel(KPar
                         const int ks = kPer * seg + i;
                         dacc = mfma(vfr[ks], cur[i], ks == 0 ? f32x16{0} : dacc);
                     }
+                    if (seg == 1) __builtin_amdgcn_s_setprio(2);
                 });
+                __builtin_amdgcn_s_setprio(1);
 #pragma unroll
                 for (int i = 0; i < 16; ++i) dp[i] = dacc[i];
                 // a -> columns 16h.. of row (32r + n) now, dz -> columns 32 + 16h.. below
@@ -1605,6 +1608,7 @@ __global__ __launch_bounds__(2 * kThreads, 2) void mfma_bwd_dkv_pair_kernel(KPar
                 own_tile_grads(x, beta, dp, Gt, lane);
                 *(bf16x8*)(ztile + tile_offset<64>(32 * r + n, 4 + 2 * h)) = pack8(&dp[0]);
                 *(bf16x8*)(ztile + tile_offset<64>(32 * r + n, 4 + 2 * h + 1)) = pack8(&dp[8]);
+                __builtin_amdgcn_s_setprio(0);
             }
         }
         __syncthreads();                       // the pair's weights are complete
