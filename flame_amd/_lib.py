@@ -98,6 +98,9 @@ def check(rc: int, what: str) -> None:
         raise RuntimeError(f"{what} failed: {load().sba_error_string(rc).decode()} (code {rc})")
 
 
+MAX_HEAD_DIM = 256     # the reference pads the head dim to the next power of two (sb_attn/sb_fwd.py:199); here up to 256
+
+
 def dtype_code(dt: torch.dtype) -> int:
     if dt == torch.float32:
         return SBA_DTYPE_F32
@@ -111,8 +114,8 @@ def check_supported(q: torch.Tensor) -> None:
     if q.dtype not in (torch.float32, torch.bfloat16):
         raise TypeError(f"stick-breaking attention supports float32, bfloat16 and (through the float32 kernels) "
                         f"float16, got {q.dtype}")
-    if q.shape[-1] > 128:
-        raise ValueError(f"head_dim {q.shape[-1]} is not supported (at most 128)")
+    if q.shape[-1] > MAX_HEAD_DIM:
+        raise ValueError(f"head_dim {q.shape[-1]} is not supported (at most {MAX_HEAD_DIM})")
 
 
 def tensor4(t: torch.Tensor) -> SbaTensor:
@@ -216,14 +219,17 @@ def raise_if_gave_up(p, static_scratch_used: bool = False) -> None:
 
 def matrix_core_head_dim(t: torch.Tensor) -> int:
     """Head dim that a problem runs with.  The matrix-core kernels exist for bf16 and fp32 at 64 and
-    128; any other head dim below those rides them zero-padded (zero columns add nothing to q.k and
-    give zero output columns), which is far faster than the generic kernels.  Everything keeps its
-    head dim under SBA_FORCE_GENERIC=1 (generic kernels)."""
+    128 and for bf16 at 256; any other head dim below those rides them zero-padded (zero columns add
+    nothing to q.k and give zero output columns), which is far faster than the generic kernels
+    (float32 above 128 has only those).  Everything keeps its head dim under SBA_FORCE_GENERIC=1
+    (generic kernels)."""
     D = t.shape[-1]
-    if D > 128 or os.environ.get("SBA_FORCE_GENERIC") == "1":
+    if D > MAX_HEAD_DIM or os.environ.get("SBA_FORCE_GENERIC") == "1":
         return D
     if t.dtype not in (torch.bfloat16, torch.float32) or D in (64, 128):
         return D
+    if D > 128:
+        return 256 if t.dtype == torch.bfloat16 else D
     return 64 if D < 64 else 128
 
 
@@ -286,7 +292,7 @@ def workspace_upper_bound(n_heads: int, columns: int) -> int:
 
 def bwd_scratch_upper_bound(n_heads: int, columns: int, tab_tokens: int, head_dim: int) -> int:
     """Four tables (the recompute mode's count) or the generic path's fp32 dk|dv accumulators."""
-    dp = 32 if head_dim <= 32 else (64 if head_dim <= 64 else 128)
+    dp = 32 if head_dim <= 32 else (64 if head_dim <= 64 else (128 if head_dim <= 128 else 256))
     acc = (2 * tab_tokens * n_heads * dp * 4 + 255) & ~255
     scaled_q = (tab_tokens * n_heads * 64 * 2 + 255) & ~255      # bf16 at head_dim 64: the dQ pass's scaled copy of q
     return max(4 * table_bytes(n_heads, columns) + scaled_q + 256, acc)      # + the backward's error word

@@ -23,10 +23,11 @@ bool force_generic() {
     return e && e[0] == '1';
 }
 
-// The matrix-core kernels cover bf16 and fp32 with head_dim 64 or 128; everything else takes the
-// generic vector-ALU kernels.
+// The matrix-core kernels cover bf16 and fp32 with head_dim 64 or 128 and bf16 with head_dim 256; everything
+// else takes the generic vector-ALU kernels.
 bool use_mfma(const SbaParams* p) {
     if (force_generic()) return false;
+    if (p->dtype == SBA_DTYPE_BF16 && p->head_dim == 256) return true;
     return (p->dtype == SBA_DTYPE_F32 || p->dtype == SBA_DTYPE_BF16) && (p->head_dim == 64 || p->head_dim == 128);
 }
 
@@ -93,7 +94,7 @@ int check_common(const SbaParams* p) {
     if (p->struct_size != sizeof(SbaParams)) return SBA_ERR_ABI;
     if (p->dtype != SBA_DTYPE_F32 && p->dtype != SBA_DTYPE_BF16) return SBA_ERR_DTYPE;
     if (p->n_seq <= 0 || p->n_heads <= 0 || p->seq_len <= 0 || p->total_tokens <= 0) return SBA_ERR_SHAPE;
-    if (p->head_dim <= 0 || p->head_dim > 128) return SBA_ERR_SHAPE;
+    if (p->head_dim <= 0 || p->head_dim > sba::kMaxHeadDim) return SBA_ERR_SHAPE;
     if (!p->q.ptr || !p->k.ptr || !p->v.ptr) return SBA_ERR_NULL;
     if (p->cu_seqlens) {
         if (!p->schedule || p->n_schedule <= 0 || p->table_cols <= 0) return SBA_ERR_SCHEDULE;
@@ -190,7 +191,7 @@ const char* sba_error_string(int code) {
     switch (code) {
         case SBA_OK: return "ok";
         case SBA_ERR_NULL: return "a required pointer is NULL";
-        case SBA_ERR_SHAPE: return "bad shape: sizes must be positive, head_dim <= 128, dense total_tokens == seq_len; at head_dim 64 / 128 (the matrix-core kernels, bf16 and fp32) tensors need 16-byte aligned pointers, outer strides that are multiples of 16 bytes and a token stride below 2^23 elements";
+        case SBA_ERR_SHAPE: return "bad shape: sizes must be positive, head_dim <= 256, dense total_tokens == seq_len; at head_dim 64 / 128 (the matrix-core kernels, bf16 and fp32) and 256 (bf16) tensors need 16-byte aligned pointers, outer strides that are multiples of 16 bytes and a token stride below 2^23 elements";
         case SBA_ERR_DTYPE: return "unsupported dtype (float32 and bfloat16 only)";
         case SBA_ERR_WORKSPACE: return "workspace / bwd_scratch missing or smaller than sba_workspace_bytes() / sba_bwd_scratch_bytes()";
         case SBA_ERR_SCHEDULE: return "packed layout needs a row-block schedule from sba_build_schedule()";
@@ -202,13 +203,13 @@ const char* sba_error_string(int code) {
 }
 
 size_t sba_workspace_bytes(const SbaParams* p) {
-    if (!p || p->n_heads <= 0 || p->seq_len <= 0 || p->head_dim <= 0 || p->head_dim > 128) return 0;
+    if (!p || p->n_heads <= 0 || p->seq_len <= 0 || p->head_dim <= 0 || p->head_dim > sba::kMaxHeadDim) return 0;
     if (p->cu_seqlens && p->table_cols <= 0) return 0;
     return use_mfma(p) ? forward_tables(p) * table_bytes(p) : 0;
 }
 
 size_t sba_bwd_scratch_bytes(const SbaParams* p) {
-    if (!p || p->n_heads <= 0 || p->seq_len <= 0 || p->head_dim <= 0 || p->head_dim > 128) return 0;
+    if (!p || p->n_heads <= 0 || p->seq_len <= 0 || p->head_dim <= 0 || p->head_dim > sba::kMaxHeadDim) return 0;
     if (p->cu_seqlens && p->table_cols <= 0 && use_mfma_bwd(p)) return 0;
     // without a workspace the backward recomputes the forward's tables first, into slots of its own
     if (!use_mfma_bwd(p)) return generic_acc_bytes(p);

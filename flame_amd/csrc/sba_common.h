@@ -9,6 +9,7 @@
 namespace sba {
 
 constexpr int kRowBlock = 128;   // query rows per scheduled job (one workgroup)
+constexpr int kMaxHeadDim = 256; // bf16: matrix-core kernels at 64, 128 and 256; every other size and type up to here: generic kernels
 constexpr int kKeyBlock = 64;    // keys per sweep step of the MFMA kernels / carry-table column
 
 // Generic (fp32 / any head dim) kernels only: logits above this (in base-2 units) are clamped;

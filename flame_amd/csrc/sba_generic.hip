@@ -1,4 +1,4 @@
-// Generic stick-breaking attention kernels: any head_dim <= 128, fp32 or bf16 storage,
+// Generic stick-breaking attention kernels: any head_dim <= 256, fp32 or bf16 storage,
 // fp32 arithmetic on the vector ALUs (no matrix cores).  This is the fp32 path of the
 // operator (the 1e-4 tolerance class) and the path for head dims the MFMA kernels do
 // not cover.  One thread owns one query row; a workgroup owns a row-block of 128 queries
@@ -228,7 +228,7 @@ static int launch_bwd(const KParams& kp, hipStream_t s) {
 
 }  // namespace sba
 
-int sba_generic_padded_dim(int D) { return D <= 32 ? 32 : (D <= 64 ? 64 : 128); }
+int sba_generic_padded_dim(int D) { return D <= 32 ? 32 : (D <= 64 ? 64 : (D <= 128 ? 128 : 256)); }
 
 int sba_launch_generic_fwd(const sba::KParams& kp, int dtype, hipStream_t s) {
     using namespace sba;
@@ -236,11 +236,13 @@ int sba_launch_generic_fwd(const sba::KParams& kp, int dtype, hipStream_t s) {
     if (dtype == SBA_DTYPE_F32) {
         if (DP == 32) return launch_fwd<float, 32>(kp, s);
         if (DP == 64) return launch_fwd<float, 64>(kp, s);
-        return launch_fwd<float, 128>(kp, s);
+        if (DP == 128) return launch_fwd<float, 128>(kp, s);
+        return launch_fwd<float, 256>(kp, s);
     }
     if (DP == 32) return launch_fwd<uint16_t, 32>(kp, s);
     if (DP == 64) return launch_fwd<uint16_t, 64>(kp, s);
-    return launch_fwd<uint16_t, 128>(kp, s);
+    if (DP == 128) return launch_fwd<uint16_t, 128>(kp, s);
+    return launch_fwd<uint16_t, 256>(kp, s);
 }
 
 int sba_launch_generic_bwd(const sba::KParams& kp, int dtype, hipStream_t s) {
@@ -249,9 +251,11 @@ int sba_launch_generic_bwd(const sba::KParams& kp, int dtype, hipStream_t s) {
     if (dtype == SBA_DTYPE_F32) {
         if (DP == 32) return launch_bwd<float, 32>(kp, s);
         if (DP == 64) return launch_bwd<float, 64>(kp, s);
-        return launch_bwd<float, 128>(kp, s);
+        if (DP == 128) return launch_bwd<float, 128>(kp, s);
+        return launch_bwd<float, 256>(kp, s);
     }
     if (DP == 32) return launch_bwd<uint16_t, 32>(kp, s);
     if (DP == 64) return launch_bwd<uint16_t, 64>(kp, s);
-    return launch_bwd<uint16_t, 128>(kp, s);
+    if (DP == 128) return launch_bwd<uint16_t, 128>(kp, s);
+    return launch_bwd<uint16_t, 256>(kp, s);
 }

@@ -66,6 +66,10 @@ template <> __device__ inline int swz<128>(int row) {  // 16 chunks per row, one
     return (r1 << 3) | (r0 << 2) | ((r1 ^ r3) << 1) | r2;
 }
 
+template <> __device__ inline int swz<256>(int row) {  // 32 chunks per row: a row is two passes over the 64 banks, the bank
+    return swz<128>(row);                               // of a chunk is its index modulo 16 as at head_dim 128
+}
+
 template <int D> __device__ inline int tile_offset(int row, int chunk) {   // bytes
     return row * (D * 2) + ((chunk ^ swz<D>(row)) << 4);
 }

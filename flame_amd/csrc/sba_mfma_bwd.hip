@@ -1,4 +1,4 @@
-// bf16 MFMA backward kernels (head_dim 64 / 128): two passes, no atomics, deterministic.
+// bf16 MFMA backward kernels (head_dim 64 / 128 / 256): two passes, no atomics, deterministic.
 //
 // The reference (`_backward_one_row`, sb_varlen/sb_varlen_bwd.py:274-456) owns a query
 // row-block, keeps dq in registers and adds every dk/dv tile into global memory under a
@@ -16,7 +16,8 @@
 //           kernels, chosen by grid size and head_dim: every wave owning 32 keys outright
 //           (d = 64, large grids), two waves sharing 32 keys (d = 128, large grids), a resident
 //           producer/consumer stream over 64-key items (d = 64, small grids), one workgroup
-//           per 64-key block (d = 128, small grids).
+//           per 64-key block (d = 128, small grids).  d = 256: every wave on its own 32 keys, in two
+//           launches that each take half of the columns of dK and dV.
 //
 // Every element of the score matrix is therefore evaluated twice in the backward (once per
 // pass); in exchange nothing is reduced through memory.
@@ -46,7 +47,7 @@ __device__ inline void store_scaled_q(const KParams& p, const Job& job, int head
 // per SIMD.  Ahead on large launches, whose SIMDs it fills better (the packed benchmark's dQ -5.6 %, short documents
 // -6 %); on launches that last as long as their longest sweep the plain arrangement's shorter step is ahead.
 template <int D, bool kLean = false>
-__global__ __launch_bounds__(kThreads, (D == 64 && kLean) ? 3 : 2) void mfma_bwd_dq_kernel(KParams p) {
+__global__ __launch_bounds__(kThreads, (D == 64 && kLean) ? 3 : (D <= 128 ? 2 : 1)) void mfma_bwd_dq_kernel(KParams p) {
     constexpr int kTile = 64 * D * 2;
     __shared__ __attribute__((aligned(16))) char lds[4 * kTile];   // K0 V0 K1 V1
 
@@ -1152,8 +1153,14 @@ __global__ __launch_bounds__((NP + 4) * 64, NP == 4 ? 2 : 3) void mfma_bwd_dkv_s
 // a 64-key block that touches the edge, the mid-block ones for the other half.  Weights and
 // logit gradients go as bf16 [query][32 a | 32 dz] rows into a tile private to the wave and
 // come back transposed as the A operands of  dV += A^T dO  and  dK += dZ^T Q.
-template <int D>
+// kSplit / kPart: at head_dim 256 the [32 keys x 256] accumulators of dK and dV alone are 256 registers a lane, on top of
+// 128 for the K and V fragments.  There the kernel is launched kSplit = 2 times, launch kPart accumulating and storing
+// columns 128 * kPart .. 128 * kPart + 127 of dK and dV only; scores, weights and logit gradients are formed in both.
+template <int D, int kSplit = 1, int kPart = 0>
 __global__ __launch_bounds__(kThreads, D == 64 ? 2 : 1) void mfma_bwd_dkv_own_kernel(KParams p) {
+    constexpr int kNB = D / 32 / kSplit;         // 32-wide column blocks of dK / dV accumulated here
+    constexpr int kB0 = kPart * kNB;             // the first of them
+    static_assert(32 * (D / kSplit) * 2 <= 64 * 64 * 2, "a wave stages its [32 keys x columns] outputs in its weight tile");
     constexpr int kQTile = 64 * D * 2;           // Q or dO tile of one step (64 queries)
     constexpr int kZTile = 64 * 64 * 2;          // per wave: [64 queries][32 a | 32 dz] bf16
     constexpr int kStep = 64;
@@ -1197,9 +1204,9 @@ __global__ __launch_bounds__(kThreads, D == 64 ? 2 : 1) void mfma_bwd_dkv_own_ke
         prescale_frags(kfr, p.scale2);         // K times the logit scale: the score MFMAs deliver base-2 logits
     }
 
-    f32x16 dkacc[D / 32], dvacc[D / 32];
+    f32x16 dkacc[kNB], dvacc[kNB];
 #pragma unroll
-    for (int db = 0; db < D / 32; ++db) { dkacc[db] = f32x16{0}; dvacc[db] = f32x16{0}; }
+    for (int db = 0; db < kNB; ++db) { dkacc[db] = f32x16{0}; dvacc[db] = f32x16{0}; }
 
     const int n_steps = q_begin < job.len ? (job.len - q_begin + kStep - 1) / kStep : 0;
 
@@ -1253,9 +1260,9 @@ __global__ __launch_bounds__(kThreads, D == 64 ? 2 : 1) void mfma_bwd_dkv_own_ke
             const bf16x8 af = fetch_nat_o<64>(zt, lz, 16 * kk, 0);
             const bf16x8 zf = fetch_nat_o<64>(zt, lz, 16 * kk, 1);
 #pragma unroll
-            for (int db = 0; db < D / 32; ++db) {
-                dvacc[db] = mfma(af, fetch_nat_o<D>(dot, lo, 16 * kk, db), dvacc[db]);
-                dkacc[db] = mfma(zf, fetch_nat_o<D>(qt, lo, 16 * kk, db), dkacc[db]);
+            for (int db = 0; db < kNB; ++db) {
+                dvacc[db] = mfma(af, fetch_nat_o<D>(dot, lo, 16 * kk, kB0 + db), dvacc[db]);
+                dkacc[db] = mfma(zf, fetch_nat_o<D>(qt, lo, 16 * kk, kB0 + db), dkacc[db]);
             }
         }
     };
@@ -1312,23 +1319,23 @@ __global__ __launch_bounds__(kThreads, D == 64 ? 2 : 1) void mfma_bwd_dkv_own_ke
                     // overwritten: this step's second tile comes later) and of the previous Q / dO tiles
                     auto red_a = [&](int seg) { return fetch_nat_o<64>(zt, lz, 32 + 16 * (seg >> 1), seg & 1); };
                     auto red_b = [&](int seg, int db) {
-                        return (seg & 1) ? fetch_nat_o<D>(pqtile, lo, 32 + 16 * (seg >> 1), db) : fetch_nat_o<D>(pdotile, lo, 32 + 16 * (seg >> 1), db);
+                        return (seg & 1) ? fetch_nat_o<D>(pqtile, lo, 32 + 16 * (seg >> 1), kB0 + db) : fetch_nat_o<D>(pdotile, lo, 32 + 16 * (seg >> 1), kB0 + db);
                     };
-                    bf16x8 na = red_a(0), nb[D / 32];
+                    bf16x8 na = red_a(0), nb[kNB];
 #pragma unroll
-                    for (int db = 0; db < D / 32; ++db) nb[db] = red_b(0, db);
+                    for (int db = 0; db < kNB; ++db) nb[db] = red_b(0, db);
                     own_tile_weights(x, beta, Rt, lane, [&](int seg) {
                         const bf16x8 ca = na;
-                        bf16x8 cb[D / 32];
+                        bf16x8 cb[kNB];
 #pragma unroll
-                        for (int db = 0; db < D / 32; ++db) cb[db] = nb[db];
+                        for (int db = 0; db < kNB; ++db) cb[db] = nb[db];
                         if (seg < 3) {
                             na = red_a(seg + 1);
 #pragma unroll
-                            for (int db = 0; db < D / 32; ++db) nb[db] = red_b(seg + 1, db);
+                            for (int db = 0; db < kNB; ++db) nb[db] = red_b(seg + 1, db);
                         }
 #pragma unroll
-                        for (int db = 0; db < D / 32; ++db) {
+                        for (int db = 0; db < kNB; ++db) {
                             if (seg & 1) dkacc[db] = mfma(ca, cb[db], dkacc[db]);
                             else dvacc[db] = mfma(ca, cb[db], dvacc[db]);
                         }
@@ -1341,23 +1348,23 @@ __global__ __launch_bounds__(kThreads, D == 64 ? 2 : 1) void mfma_bwd_dkv_own_ke
                     // whose exp/rcp overlap them.  Segment 2kk: dV += A^T dO, segment 2kk + 1: dK += dZ^T Q.
                     auto red_a = [&](int seg) { return fetch_nat_o<64>(zt, lz, 16 * (seg >> 1), seg & 1); };
                     auto red_b = [&](int seg, int db) {
-                        return (seg & 1) ? fetch_nat_o<D>(qtile, lo, 16 * (seg >> 1), db) : fetch_nat_o<D>(dotile, lo, 16 * (seg >> 1), db);
+                        return (seg & 1) ? fetch_nat_o<D>(qtile, lo, 16 * (seg >> 1), kB0 + db) : fetch_nat_o<D>(dotile, lo, 16 * (seg >> 1), kB0 + db);
                     };
-                    bf16x8 na = red_a(0), nb[D / 32];
+                    bf16x8 na = red_a(0), nb[kNB];
 #pragma unroll
-                    for (int db = 0; db < D / 32; ++db) nb[db] = red_b(0, db);
+                    for (int db = 0; db < kNB; ++db) nb[db] = red_b(0, db);
                     own_tile_weights(x, beta, Rt, lane, [&](int seg) {
                         const bf16x8 ca = na;
-                        bf16x8 cb[D / 32];
+                        bf16x8 cb[kNB];
 #pragma unroll
-                        for (int db = 0; db < D / 32; ++db) cb[db] = nb[db];
+                        for (int db = 0; db < kNB; ++db) cb[db] = nb[db];
                         if (seg < 3) {
                             na = red_a(seg + 1);
 #pragma unroll
-                            for (int db = 0; db < D / 32; ++db) nb[db] = red_b(seg + 1, db);
+                            for (int db = 0; db < kNB; ++db) nb[db] = red_b(seg + 1, db);
                         }
 #pragma unroll
-                        for (int db = 0; db < D / 32; ++db) {
+                        for (int db = 0; db < kNB; ++db) {
                             if (seg & 1) dkacc[db] = mfma(ca, cb[db], dkacc[db]);
                             else dvacc[db] = mfma(ca, cb[db], dvacc[db]);
                         }
@@ -1408,13 +1415,14 @@ __global__ __launch_bounds__(kThreads, D == 64 ? 2 : 1) void mfma_bwd_dkv_own_ke
     for (int which = 0; which < 2; ++which) {
         const TensorArg& out = which == 0 ? p.dk : p.dv;
         const int64_t ob = (int64_t)job.seq * out.sb + (int64_t)head * out.sh + (int64_t)job.tok0 * out.st;
+        constexpr int kCols = D / kSplit;          // columns kPart * kCols .. of the rows
 #pragma unroll
-        for (int db = 0; db < D / 32; ++db)
-            stage_acc_tile<D>(ztile, 0, 32 * db, which == 0 ? dkacc[db] : dvacc[db], which == 0 ? p.scale : 1.0f, lane);
-        for (int c = lane; c < 32 * D / 8; c += 64) {
-            const int row = c / (D / 8), cc = c % (D / 8);
+        for (int db = 0; db < kNB; ++db)
+            stage_acc_tile<kCols>(ztile, 0, 32 * db, which == 0 ? dkacc[db] : dvacc[db], which == 0 ? p.scale : 1.0f, lane);
+        for (int c = lane; c < 32 * kCols / 8; c += 64) {
+            const int row = c / (kCols / 8), cc = c % (kCols / 8);
             if (kb0 + row < job.len)
-                *(u32x4*)(out.ptr + 2 * (ob + (int64_t)(kb0 + row) * out.st + cc * 8)) = *(const u32x4*)(ztile + row * (D * 2) + cc * 16);
+                *(u32x4*)(out.ptr + 2 * (ob + (int64_t)(kb0 + row) * out.st + kPart * kCols + cc * 8)) = *(const u32x4*)(ztile + row * (kCols * 2) + cc * 16);
         }
     }
 }
@@ -1742,6 +1750,14 @@ int sba_launch_mfma_bwd(const sba::KParams& kp_in, int phases, hipStream_t s) {
             n_wg = (n_wg + 7) & ~7u;
             if (stream8) hipLaunchKernelGGL((mfma_bwd_dkv_stream_kernel<64, 8>), dim3(n_wg), dim3(12 * 64), 0, s, kp);
             else hipLaunchKernelGGL((mfma_bwd_dkv_stream_kernel<64, 4>), dim3(n_wg), dim3(8 * 64), 0, s, kp);
+        }
+    } else if (kp.head_dim == 256) {
+        // one wave per SIMD in both passes; every wave of the key-owner pass on its own 32 keys, in two launches that
+        // each accumulate one half of the columns of dK and dV - the other key-owner kernels do not fit the CU here
+        if (p1) hipLaunchKernelGGL((mfma_bwd_dq_kernel<256>), grid, dim3(kThreads), 0, s, kp);
+        if (p2) {
+            hipLaunchKernelGGL((mfma_bwd_dkv_own_kernel<256, 2, 0>), grid, dim3(kThreads), 0, s, kp);
+            hipLaunchKernelGGL((mfma_bwd_dkv_own_kernel<256, 2, 1>), grid, dim3(kThreads), 0, s, kp);
         }
     } else {
         if (p1) hipLaunchKernelGGL((mfma_bwd_dq_kernel<128>), grid, dim3(kThreads), 0, s, kp);

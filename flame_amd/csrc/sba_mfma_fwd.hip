@@ -1,4 +1,4 @@
-// bf16 MFMA forward kernels (head_dim 64 / 128).
+// bf16 MFMA forward kernels (head_dim 64 / 128 / 256; at 256 the one-sweep kernel only: two K / V tile pairs are 128 KB of LDS).
 // Replace the reference's `_forward_one_row` sweep (sb_varlen/sb_varlen_fwd.py:81-215):
 // one workgroup per (sequence, head, 128-query row-block), keys swept right-to-left from
 // the diagonal in steps of 64, K/V tiles double-buffered in LDS, running product of
@@ -373,6 +373,7 @@ __global__ __launch_bounds__(G * kThreads) void mfma_fwd_seg_kernel(KParams p) {
 // SBA_FWD_GROUPS=2|3|4 forces the number of segments where the rule picks any; SBA_TWO_STEP_MAX_GRID=n replaces
 // the rule by "segments (4, or as forced) up to n workgroups".
 static int forward_segments(const sba::KParams& kp, unsigned grid) {
+    if (kp.head_dim == 256) return 0;      // two K / V tile pairs are 128 KB of LDS: one group of waves per workgroup
     if (kp.head_dim == 128) {
         // head_dim 128: the one-sweep kernel holds two workgroups per CU, the two-segment one (8 waves, 129 KB of
         // LDS) one; it pays while the grid is at most two rounds of those and the longest sweep dominates.  B=1,
@@ -409,9 +410,12 @@ int sba_launch_mfma_fwd(const sba::KParams& kp, hipStream_t s) {
     } else if (kp.head_dim == 64) {
         if (kp.carry_only) hipLaunchKernelGGL((mfma_fwd_kernel<64, true>), grid, dim3(kThreads), 0, s, kp);
         else hipLaunchKernelGGL((mfma_fwd_kernel<64, false>), grid, dim3(kThreads), 0, s, kp);
-    } else {
+    } else if (kp.head_dim == 128) {
         if (kp.carry_only) hipLaunchKernelGGL((mfma_fwd_kernel<128, true>), grid, dim3(kThreads), 0, s, kp);
         else hipLaunchKernelGGL((mfma_fwd_kernel<128, false>), grid, dim3(kThreads), 0, s, kp);
+    } else {
+        if (kp.carry_only) hipLaunchKernelGGL((mfma_fwd_kernel<256, true>), grid, dim3(kThreads), 0, s, kp);
+        else hipLaunchKernelGGL((mfma_fwd_kernel<256, false>), grid, dim3(kThreads), 0, s, kp);
     }
     return hipGetLastError() == hipSuccess ? SBA_OK : SBA_ERR_LAUNCH;
 }

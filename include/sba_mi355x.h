@@ -25,8 +25,9 @@
  *   packed [H, sumT, D]  : n_seq = number of documents, cu_seqlens = device int32[n_seq+1]
  *                          with cu_seqlens[0] == 0, stride_b = 0,
  *                          element (h,t,d) at    base + h*stride_h + t*stride_t + d
- * Strides are in elements; the innermost (D) stride is 1.  Problems at head_dim 64 / 128
- * (the matrix-core kernels) need 16-byte aligned tensor pointers, outer strides that are
+ * Strides are in elements; the innermost (D) stride is 1.  head_dim is at most 256 (the reference
+ * pads it to the next power of two, sb_attn/sb_fwd.py:199).  Problems at head_dim 64 / 128, and
+ * bf16 ones at 256 (the matrix-core kernels) need 16-byte aligned tensor pointers, outer strides that are
  * multiples of 16 bytes - 8 bf16 or 4 fp32 elements - and a token stride below 2^23 elements
  * (the tile copies address a 64-row tile with 32-bit byte offsets); SBA_ERR_SHAPE otherwise.
  * rem / d_rem are contiguous along tokens.
@@ -82,7 +83,7 @@ typedef struct SbaParams {
     int32_t  seq_len;          /* T (dense) or max document length (packed: an upper bound is accepted; the kernels
                                   are chosen from it, so the exact longest document chooses best) */
     int32_t  total_tokens;     /* T (dense) or sumT (packed) */
-    int32_t  head_dim;         /* D */
+    int32_t  head_dim;         /* D <= 256 */
     int32_t  attend_current;   /* 0: keys j < i;  1: keys j <= i */
     float    scale;            /* logit scale ("inv_temp") in natural-log units */
     int32_t  save_for_backward;/* forward only: also fill the carry table in workspace */
@@ -131,7 +132,7 @@ size_t sba_workspace_bytes(const SbaParams* p);
  * bf16 copy of q times the logit scale, total_tokens x n_heads x 128 bytes, which the first kernel
  * writes and the second reads in place of q; or the generic path's fp32 accumulators): allocate
  * before the call, free after it has run.  With bwd_phases 1 and 2 issued
- * as two calls, the same buffer goes to both.  For bf16 at head_dim 64 / 128 the last 256 bytes
+ * as two calls, the same buffer goes to both.  For bf16 at head_dim 64 / 128 / 256 the last 256 bytes
  * hold an error word (int32): the first kernel of a backward (bwd_phases 0 or 1) clears it, and a
  * kernel that abandoned one of its bounded internal waits sets it to 1 (the gradients are then
  * invalid); a bwd_phases = 2 call leaves what phase 1 left.  sba_bwd_gave_up() reads it.

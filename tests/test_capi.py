@@ -44,8 +44,9 @@ def test_argument_checks_without_gpu(lib):
     assert lib.sba_fwd(C.byref(p)) == -3          # dtype
     p.dtype = _lib.SBA_DTYPE_BF16
     assert lib.sba_fwd(C.byref(p)) == -2          # shape (all zero)
-    p.n_seq, p.n_heads, p.seq_len, p.total_tokens, p.head_dim = 1, 2, 64, 64, 256
-    assert lib.sba_fwd(C.byref(p)) == -2          # head_dim > 128
+    p.n_seq, p.n_heads, p.seq_len, p.total_tokens, p.head_dim = 1, 2, 64, 64, 257
+    assert lib.sba_fwd(C.byref(p)) == -2          # head_dim > 256
+    assert lib.sba_workspace_bytes(C.byref(p)) == 0 and lib.sba_bwd_scratch_bytes(C.byref(p)) == 0
     p.head_dim = 64
     assert lib.sba_fwd(C.byref(p)) == -1          # NULL q/k/v
     assert lib.sba_fwd(None) == -1
@@ -111,6 +112,15 @@ def test_workspace_bytes(lib):
     p.head_dim = 96                                 # generic kernels: nothing kept, fp32 dk|dv accumulators
     assert lib.sba_workspace_bytes(C.byref(p)) == 0
     assert lib.sba_bwd_scratch_bytes(C.byref(p)) == 2 * 4096 * 16 * 128 * 4
+    p.head_dim = 256                                # fp32 above 128: generic kernels
+    assert lib.sba_workspace_bytes(C.byref(p)) == 0
+    assert lib.sba_bwd_scratch_bytes(C.byref(p)) == 2 * 4096 * 16 * 256 * 4
+    p.dtype = _lib.SBA_DTYPE_BF16                   # bf16 at 256: matrix cores, two tables each way, the error word, no copy of q
+    assert lib.sba_workspace_bytes(C.byref(p)) == 2 * table
+    assert lib.sba_bwd_scratch_bytes(C.byref(p)) == 4 * table + 256
+    p.head_dim = 200                                # bf16 in between: generic kernels unless the caller pads to 256
+    assert lib.sba_workspace_bytes(C.byref(p)) == 0
+    assert lib.sba_bwd_scratch_bytes(C.byref(p)) == 2 * 4096 * 16 * 256 * 4
 
 
 def test_static_backward_refuses_oversize_without_gpu(lib):
@@ -227,7 +237,7 @@ def test_op_refuses_cpu_tensors():
 
 def test_python_workspace_bound_covers_the_library(lib):
     for dtype in (_lib.SBA_DTYPE_BF16, _lib.SBA_DTYPE_F32):
-        for (B, H, T, D) in [(1, 16, 4096, 64), (2, 3, 129, 128), (1, 2, 77, 80), (4, 1, 1, 8)]:
+        for (B, H, T, D) in [(1, 16, 4096, 64), (2, 3, 129, 128), (1, 2, 77, 80), (4, 1, 1, 8), (2, 3, 300, 256), (1, 2, 77, 200)]:
             p = _lib.SbaParams()
             p.struct_size = C.sizeof(_lib.SbaParams)
             p.dtype = dtype

@@ -92,7 +92,7 @@ def test_longest_dense_row_65536_tokens_invariants():
     assert max_abs(o.detach()[:, :1, T - 256:].float().cpu(), o_tail[:, :, W - 256:]) <= 2e-2
 
 
-@pytest.mark.parametrize("D", [64, 128])
+@pytest.mark.parametrize("D", [64, 128, 256])
 def test_carries_that_underflow_to_zero(D):
     # Logits around +6 in natural units (beta ~ 0.998): the product of (1 - beta) entering a key block is
     # below the fp32 range after a few tens of keys, so the carry tables hold exact zeros for almost every

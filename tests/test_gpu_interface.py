@@ -65,8 +65,8 @@ def test_argument_errors_are_python_errors():
     with pytest.raises(TypeError, match="float16"):
         sb_attn_varlen(q.double(), q.double(), q.double(), cu, 200)
     with pytest.raises(ValueError, match="head_dim"):
-        sb_attn(torch.zeros(1, 1, 8, 256, device="cuda"), torch.zeros(1, 1, 8, 256, device="cuda"),
-                torch.zeros(1, 1, 8, 256, device="cuda"))
+        sb_attn(torch.zeros(1, 1, 8, 264, device="cuda"), torch.zeros(1, 1, 8, 264, device="cuda"),
+                torch.zeros(1, 1, 8, 264, device="cuda"))
     with pytest.raises(ValueError, match="longest document"):
         sb_attn_varlen(q, q, q, cu, 150)
     with pytest.raises(ValueError, match="ends at"):

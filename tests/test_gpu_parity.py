@@ -86,7 +86,7 @@ def test_bf16_no_drem_and_no_grad():
     _check_dense(1, 2, 300, 64, torch.bfloat16, seed=22, in_scale=0.5, grads=False)
 
 
-@pytest.mark.parametrize("D", [64, 128])
+@pytest.mark.parametrize("D", [64, 128, 256])
 def test_bf16_saturated_logits(D):
     # selected keys aligned with the queries so that |z| reaches 20 and more: exercises the
     # saturated sigmoid (the reference's softplus x>15 branch, softplus.py:9-10)
@@ -410,7 +410,7 @@ def test_small_and_large_grids_take_different_backward_kernels_and_agree(D):
         assert rel_l2(a.float().cpu(), r) <= 5e-2 and rel_l2(b[39:].float().cpu(), r) <= 5e-2
 
 
-@pytest.mark.parametrize("D", [64, 128])
+@pytest.mark.parametrize("D", [64, 128, 256])
 @pytest.mark.parametrize("rep", [1, 40])
 def test_gradient_of_rem_alone(D, rep):
     # dO = 0: everything comes from d_rem, which the matrix-core backward carries as the constant
