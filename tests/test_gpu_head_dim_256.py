@@ -6,7 +6,7 @@ import pytest
 import torch
 
 from oracle import sb_oracle as O
-from helpers import randn, rel_l2, max_abs, cu_from_lengths
+from helpers import randn, rel_l2, max_abs, cu_from_lengths, within
 from test_gpu_parity import _check_dense, _check_varlen, _ops
 
 pytestmark = pytest.mark.gpu
@@ -49,7 +49,7 @@ def test_fp32_and_fp16_above_128_take_the_generic_kernels(D):
 
 
 def test_many_workgroups_and_long_sweeps_head_dim_256():
-    # 24 x 8 row blocks (every CU busy, sweeps of up to 16 steps, both tile buffers of every kernel in use) against
+    # 6 x 4 x 8 row blocks (every CU busy, sweeps of up to 16 steps, both tile buffers of every kernel in use) against
     # the oracle on the first and the last sequence; all copies of the same sequence must give the same bits
     sb_attn, _ = _ops()
     D, T, rep = 256, 1024, 6
@@ -60,9 +60,11 @@ def test_many_workgroups_and_long_sweeps_head_dim_256():
     o, rem = sb_attn(q, k, v)
     torch.autograd.backward([o, rem], [do.cuda().expand(rep, -1, -1, -1).contiguous(), drem.cuda().expand(rep, -1, -1).contiguous()])
     o_ref, rem_ref, dq, dk, dv = O.sb_attn_grads_oracle(*base, do, drem)
-    assert max_abs(o[:1].float().cpu(), o_ref) <= 2e-2 and max_abs(rem[:1].float().cpu(), rem_ref) <= 2e-2
-    for g, r in ((q.grad, dq), (k.grad, dk), (v.grad, dv)):
-        assert rel_l2(g[:1].float().cpu(), r) <= 5e-2
+    label = "head_dim 256 H=4 T=1024 (first of 6 copies)"
+    within(label, "o", max_abs(o[:1].float().cpu(), o_ref), 2e-2)
+    within(label, "rem", max_abs(rem[:1].float().cpu(), rem_ref), 2e-2)
+    for name, g, r in (("dq", q.grad, dq), ("dk", k.grad, dk), ("dv", v.grad, dv)):
+        within(label, name, rel_l2(g[:1].float().cpu(), r), 5e-2)
         assert torch.equal(g[0], g[rep - 1])
     assert torch.equal(o[0], o[rep - 1]) and torch.equal(rem[0], rem[rep - 1])
 
