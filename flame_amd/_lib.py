@@ -14,7 +14,7 @@ import torch
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "csrc", "libsba_mi355x.so")
 
-SBA_DTYPE_F32, SBA_DTYPE_BF16 = 0, 1
+SBA_DTYPE_F32, SBA_DTYPE_BF16, SBA_DTYPE_F16 = 0, 1, 2
 SBA_ABI_VERSION = 6
 
 
@@ -106,14 +106,21 @@ def dtype_code(dt: torch.dtype) -> int:
         return SBA_DTYPE_F32
     if dt == torch.bfloat16:
         return SBA_DTYPE_BF16
-    raise TypeError(f"stick-breaking attention supports float32 and bfloat16, got {dt}")
+    if dt == torch.float16:
+        return SBA_DTYPE_F16
+    raise TypeError(f"stick-breaking attention supports float32, bfloat16 and float16, got {dt}")
+
+
+def float16_needs_float32_route() -> bool:
+    """float16 has matrix-core kernels only; with the generic kernels forced (the test-suite's cross-checks) it
+    runs as float32 - exact conversion in, results rounded to float16."""
+    return os.environ.get("SBA_FORCE_GENERIC") == "1" or os.environ.get("SBA_FORCE_GENERIC_BWD") == "1"
 
 
 def check_supported(q: torch.Tensor) -> None:
     """Say up front what the kernels do not cover instead of failing inside the library."""
-    if q.dtype not in (torch.float32, torch.bfloat16):
-        raise TypeError(f"stick-breaking attention supports float32, bfloat16 and (through the float32 kernels) "
-                        f"float16, got {q.dtype}")
+    if q.dtype not in (torch.float32, torch.bfloat16, torch.float16):
+        raise TypeError(f"stick-breaking attention supports float32, bfloat16 and float16, got {q.dtype}")
     if q.shape[-1] > MAX_HEAD_DIM:
         raise ValueError(f"head_dim {q.shape[-1]} is not supported (at most {MAX_HEAD_DIM})")
 
@@ -218,18 +225,18 @@ def raise_if_gave_up(p, static_scratch_used: bool = False) -> None:
 
 
 def matrix_core_head_dim(t: torch.Tensor) -> int:
-    """Head dim that a problem runs with.  The matrix-core kernels exist for bf16 and fp32 at 64 and
-    128 and for bf16 at 256; any other head dim below those rides them zero-padded (zero columns add
+    """Head dim that a problem runs with.  The matrix-core kernels exist for bf16, float16 and fp32 at 64
+    and 128 and for the two 16-bit types at 256; any other head dim below those rides them zero-padded (zero columns add
     nothing to q.k and give zero output columns), which is far faster than the generic kernels
     (float32 above 128 has only those).  Everything keeps its head dim under SBA_FORCE_GENERIC=1
     (generic kernels)."""
     D = t.shape[-1]
     if D > MAX_HEAD_DIM or os.environ.get("SBA_FORCE_GENERIC") == "1":
         return D
-    if t.dtype not in (torch.bfloat16, torch.float32) or D in (64, 128):
+    if t.dtype not in (torch.bfloat16, torch.float16, torch.float32) or D in (64, 128):
         return D
     if D > 128:
-        return 256 if t.dtype == torch.bfloat16 else D
+        return 256 if t.dtype != torch.float32 else D
     return 64 if D < 64 else 128
 
 

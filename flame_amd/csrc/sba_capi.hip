@@ -23,12 +23,14 @@ bool force_generic() {
     return e && e[0] == '1';
 }
 
-// The matrix-core kernels cover bf16 and fp32 with head_dim 64 or 128 and bf16 with head_dim 256; everything
-// else takes the generic vector-ALU kernels.
+bool is_16bit(const SbaParams* p) { return p->dtype == SBA_DTYPE_BF16 || p->dtype == SBA_DTYPE_F16; }
+
+// The matrix-core kernels cover bf16, float16 and fp32 with head_dim 64 or 128 and the 16-bit types with head_dim
+// 256; everything else takes the generic vector-ALU kernels (which exist for bf16 and fp32).
 bool use_mfma(const SbaParams* p) {
     if (force_generic()) return false;
-    if (p->dtype == SBA_DTYPE_BF16 && p->head_dim == 256) return true;
-    return (p->dtype == SBA_DTYPE_F32 || p->dtype == SBA_DTYPE_BF16) && (p->head_dim == 64 || p->head_dim == 128);
+    if (is_16bit(p) && p->head_dim == 256) return true;
+    return (p->dtype == SBA_DTYPE_F32 || is_16bit(p)) && (p->head_dim == 64 || p->head_dim == 128);
 }
 
 // The MFMA backward is a separate switch so that the two directions can be brought up
@@ -69,15 +71,15 @@ constexpr size_t kErrorWordBytes = 256;     // tail of the bf16 matrix-core back
 // entering the right 32 keys of every 64-key step (`rtab`) and the one entering its left 32 keys (`rmid`), so
 // that every lane of the backward starts its chain from its own carry - and the dQ pass the two prefix tables
 // (`gtab`, `gmid`).  fp32, two in all: the forward writes `rtab`, the dQ pass `gtab`.
-int forward_tables(const SbaParams* p) { return p->dtype == SBA_DTYPE_BF16 ? 2 : 1; }
+int forward_tables(const SbaParams* p) { return is_16bit(p) ? 2 : 1; }
 // tables in the backward's scratch: the dQ pass's own, plus the forward's when no workspace brings them
 int scratch_tables(const SbaParams* p) { return forward_tables(p) * (p->workspace ? 1 : 2); }
 // the bounded waits (and with them the error word) exist in the bf16 matrix-core backward only
-bool has_error_word(const SbaParams* p) { return use_mfma_bwd(p) && p->dtype == SBA_DTYPE_BF16; }
+bool has_error_word(const SbaParams* p) { return use_mfma_bwd(p) && is_16bit(p); }
 // bf16 at head_dim 64: the dQ pass leaves a copy of q times the logit scale (bf16, [sequence][head][token][64], dense)
 // behind the tables, for the key-owner stream kernel, whose score MFMAs then deliver base-2 logits
 size_t scaled_q_bytes(const SbaParams* p) {
-    if (!use_mfma_bwd(p) || p->dtype != SBA_DTYPE_BF16 || p->head_dim != 64) return 0;
+    if (!use_mfma_bwd(p) || !is_16bit(p) || p->head_dim != 64) return 0;
     size_t b = (size_t)tab_tokens(p) * p->n_heads * 64 * 2;
     return (b + 255) & ~(size_t)255;
 }
@@ -92,7 +94,9 @@ constexpr int64_t kMaxTokenStride = (INT64_C(1) << 31) / (64 * 4) - 1;
 int check_common(const SbaParams* p) {
     if (!p) return SBA_ERR_NULL;
     if (p->struct_size != sizeof(SbaParams)) return SBA_ERR_ABI;
-    if (p->dtype != SBA_DTYPE_F32 && p->dtype != SBA_DTYPE_BF16) return SBA_ERR_DTYPE;
+    if (p->dtype != SBA_DTYPE_F32 && !is_16bit(p)) return SBA_ERR_DTYPE;
+    // float16 has matrix-core kernels only: head_dim 64, 128 or 256 (callers zero-pad other head dims)
+    if (p->dtype == SBA_DTYPE_F16 && !use_mfma_bwd(p)) return SBA_ERR_DTYPE;
     if (p->n_seq <= 0 || p->n_heads <= 0 || p->seq_len <= 0 || p->total_tokens <= 0) return SBA_ERR_SHAPE;
     if (p->head_dim <= 0 || p->head_dim > sba::kMaxHeadDim) return SBA_ERR_SHAPE;
     if (!p->q.ptr || !p->k.ptr || !p->v.ptr) return SBA_ERR_NULL;
@@ -192,7 +196,7 @@ const char* sba_error_string(int code) {
         case SBA_OK: return "ok";
         case SBA_ERR_NULL: return "a required pointer is NULL";
         case SBA_ERR_SHAPE: return "bad shape: sizes must be positive, head_dim <= 256, dense total_tokens == seq_len; at head_dim 64 / 128 (the matrix-core kernels, bf16 and fp32) and 256 (bf16) tensors need 16-byte aligned pointers, outer strides that are multiples of 16 bytes and a token stride below 2^23 elements";
-        case SBA_ERR_DTYPE: return "unsupported dtype (float32 and bfloat16 only)";
+        case SBA_ERR_DTYPE: return "unsupported dtype: float32, bfloat16, or float16 at head_dim 64 / 128 / 256 (float16 has matrix-core kernels only: not under SBA_FORCE_GENERIC=1 / SBA_FORCE_GENERIC_BWD=1)";
         case SBA_ERR_WORKSPACE: return "workspace / bwd_scratch missing or smaller than sba_workspace_bytes() / sba_bwd_scratch_bytes()";
         case SBA_ERR_SCHEDULE: return "packed layout needs a row-block schedule from sba_build_schedule()";
         case SBA_ERR_LAUNCH: return "kernel launch failed";
@@ -282,6 +286,7 @@ int sba_fwd(const SbaParams* p) {
     KParams kp = make_kparams(p);
     hipStream_t s = (hipStream_t)p->stream;
     if (mfma && p->dtype == SBA_DTYPE_F32) return sba_launch_mfma_f32_fwd(kp, s);
+    if (mfma && p->dtype == SBA_DTYPE_F16) return sba_launch_mfma_f16_fwd(kp, s);
     return mfma ? sba_launch_mfma_fwd(kp, s) : sba_launch_generic_fwd(kp, p->dtype, s);
 }
 
@@ -299,12 +304,14 @@ int sba_bwd(const SbaParams* p) {
         KParams carry = kp;
         carry.save = 1;
         carry.carry_only = 1;
-        rc = p->dtype == SBA_DTYPE_F32 ? sba_launch_mfma_f32_fwd(carry, s) : sba_launch_mfma_fwd(carry, s);
+        rc = p->dtype == SBA_DTYPE_F32 ? sba_launch_mfma_f32_fwd(carry, s)
+           : p->dtype == SBA_DTYPE_F16 ? sba_launch_mfma_f16_fwd(carry, s) : sba_launch_mfma_fwd(carry, s);
         if (rc) return rc;
     }
     // the generic backward is one piece: it all runs in phase 1
     if (!use_mfma_bwd(p) && p->bwd_phases == 2) return SBA_OK;
     if (use_mfma_bwd(p) && p->dtype == SBA_DTYPE_F32) return sba_launch_mfma_f32_bwd(kp, p->bwd_phases, s);
+    if (use_mfma_bwd(p) && p->dtype == SBA_DTYPE_F16) return sba_launch_mfma_f16_bwd(kp, p->bwd_phases, s);
     return use_mfma_bwd(p) ? sba_launch_mfma_bwd(kp, p->bwd_phases, s) : sba_launch_generic_bwd(kp, p->dtype, s);
 }
 

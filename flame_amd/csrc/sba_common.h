@@ -186,6 +186,8 @@ int sba_launch_generic_fwd(const sba::KParams& kp, int dtype, hipStream_t s);
 int sba_launch_generic_bwd(const sba::KParams& kp, int dtype, hipStream_t s);
 int sba_launch_mfma_fwd(const sba::KParams& kp, hipStream_t s);
 int sba_launch_mfma_bwd(const sba::KParams& kp, int phases, hipStream_t s);
+int sba_launch_mfma_f16_fwd(const sba::KParams& kp, hipStream_t s);       // the same kernels compiled for float16 elements
+int sba_launch_mfma_f16_bwd(const sba::KParams& kp, int phases, hipStream_t s);
 int sba_launch_mfma_f32_fwd(const sba::KParams& kp, hipStream_t s);
 int sba_launch_mfma_f32_bwd(const sba::KParams& kp, int phases, hipStream_t s);
 bool sba_mfma_bwd_available();

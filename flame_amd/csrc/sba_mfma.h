@@ -1,5 +1,6 @@
-// Building blocks of the bf16 MFMA kernels (gfx950): LDS tile layout, global->LDS tile
-// copies, MFMA operand fetches and the per-tile stick-breaking arithmetic.
+// Building blocks of the 16-bit MFMA kernels (gfx950): LDS tile layout, global->LDS tile
+// copies, MFMA operand fetches and the per-tile stick-breaking arithmetic.  Written for bf16,
+// which the comments speak of; the same text compiles for float16 (see SBA_ELEM_F16 below).
 //
 // Geometry.  A workgroup is 4 waves; wave w owns 32 query rows.  A sweep step covers
 // 64 keys.  All score tiles are computed TRANSPOSED, S^T = K * Q^T, with
@@ -20,10 +21,35 @@
 #pragma once
 #include "sba_common.h"
 
-namespace sba {
+// The 16-bit element type.  Everything below is compiled once per type: bf16 by default, float16 with
+// -DSBA_ELEM_F16 (same sources, second object files).  Kernels, helpers and launchers of the two builds live in
+// different inline namespaces, so both sets link into one library; code that includes this header once sees them
+// as plain sba:: names.
+#ifdef SBA_ELEM_F16
+#define SBA_ELEM_NS f16
+#else
+#define SBA_ELEM_NS bf16
+#endif
 
-typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
-typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2;
+namespace sba {
+inline namespace SBA_ELEM_NS {
+
+#ifdef SBA_ELEM_F16
+typedef _Float16 elem16;
+#else
+typedef __bf16 elem16;
+#endif
+typedef __attribute__((ext_vector_type(8))) elem16 h16x8;
+typedef __attribute__((ext_vector_type(2))) elem16 h16x2;
+// 16-bit scalars in global memory (rem, d_rem)
+#ifdef SBA_ELEM_F16
+struct Elem16 {
+    __device__ static float load(const char* p, int64_t i) { return (float)((const _Float16*)p)[i]; }
+    __device__ static void store(char* p, int64_t i, float v) { ((_Float16*)p)[i] = (_Float16)v; }
+};
+#else
+typedef Elem<uint16_t> Elem16;
+#endif
 typedef __attribute__((ext_vector_type(2))) float f32x2;
 typedef __attribute__((ext_vector_type(16))) float f32x16;
 typedef __attribute__((ext_vector_type(4))) short s16x4;
@@ -35,13 +61,13 @@ constexpr int kThreads = 256;
 // back to bf16): the score MFMAs then deliver base-2 logits directly and the per-element
 // multiplication disappears from every step.  Costs one more bf16 rounding of q (relative
 // 2^-9 per element, the size of the rounding the inputs already carry).
-template <int NF> __device__ inline void prescale_frags(bf16x8 (&f)[NF], float s) {
+template <int NF> __device__ inline void prescale_frags(h16x8 (&f)[NF], float s) {
 #pragma unroll
     for (int ks = 0; ks < NF; ++ks)
 #pragma unroll
         for (int i = 0; i < 8; i += 2) {
             const f32x2 v = {(float)f[ks][i] * s, (float)f[ks][i + 1] * s};
-            const bf16x2 b = __builtin_convertvector(v, bf16x2);
+            const h16x2 b = __builtin_convertvector(v, h16x2);
             f[ks][i] = b[0]; f[ks][i + 1] = b[1];
         }
 }
@@ -155,19 +181,19 @@ __device__ inline s16x4 lds_read_tr_at(uint32_t base, int imm) {
 //   fetch_nat_o   the same from a tile whose rows are in NATURAL order (Q, dO, and the weight
 //                 tiles of the key-owner pass): lane (m, h) gets column 32*cb + m of rows
 //                 row0 + 8*h + j, j = 0..7.
-template <int D> __device__ inline bf16x8 fetch_rows_o(const char* tile, const LaneOffsets<D>& o, int t, int ks) {
-    return *(const bf16x8*)(tile + o.rows[ks] + t * 32 * D * 2);
+template <int D> __device__ inline h16x8 fetch_rows_o(const char* tile, const LaneOffsets<D>& o, int t, int ks) {
+    return *(const h16x8*)(tile + o.rows[ks] + t * 32 * D * 2);
 }
-template <int D> __device__ inline bf16x8 fetch_rows_o(TileAt tile, const LaneOffsets<D>& o, int t, int ks) {
-    return *(const __attribute__((address_space(3))) bf16x8*)((__attribute__((address_space(3))) char*)(uintptr_t)(uint32_t)o.rows[ks] + (tile.off + t * 32 * D * 2));
+template <int D> __device__ inline h16x8 fetch_rows_o(TileAt tile, const LaneOffsets<D>& o, int t, int ks) {
+    return *(const __attribute__((address_space(3))) h16x8*)((__attribute__((address_space(3))) char*)(uintptr_t)(uint32_t)o.rows[ks] + (tile.off + t * 32 * D * 2));
 }
 // kPinBase: the sum `tile + lane offset` is pinned in a register (lds_lane_base) and the fetch's constant goes into
 // the offset field; one vector add per offset register and step instead of one per fetch, at the price of registers
 // for the pinned sums of both tile buffers (measured: forward -7 % on small grids and -3 % at head_dim 128, dQ -2 %
 // / -7 % at head_dim 64 / 128; the one-step forward at head_dim 64 would leave its four waves per SIMD).
 template <int D, bool kPinBase = true>
-__device__ inline bf16x8 fetch_cols_o(const char* tile, const LaneOffsets<D>& o, int db, int c) {
-    union { s16x4 v[2]; bf16x8 b; } u;
+__device__ inline h16x8 fetch_cols_o(const char* tile, const LaneOffsets<D>& o, int db, int c) {
+    union { s16x4 v[2]; h16x8 b; } u;
     const int add = (32 * (c >> 1) + 16 * (c & 1)) * D * 2;
     if (kPinBase) {
         u.v[0] = lds_read_tr_at(lds_lane_base(tile, o.cols[0][db]), add);
@@ -179,23 +205,23 @@ __device__ inline bf16x8 fetch_cols_o(const char* tile, const LaneOffsets<D>& o,
     return u.b;
 }
 template <int D, bool kPinBase = true>
-__device__ inline bf16x8 fetch_cols_o(TileAt tile, const LaneOffsets<D>& o, int db, int c) {
-    union { s16x4 v[2]; bf16x8 b; } u;
+__device__ inline h16x8 fetch_cols_o(TileAt tile, const LaneOffsets<D>& o, int db, int c) {
+    union { s16x4 v[2]; h16x8 b; } u;
     const int add = tile.off + (32 * (c >> 1) + 16 * (c & 1)) * D * 2;
     u.v[0] = lds_read_tr_at((uint32_t)o.cols[0][db], add);
     u.v[1] = lds_read_tr_at((uint32_t)o.cols[1][db], add);
     return u.b;
 }
 template <int D, bool kPinBase = false>
-__device__ inline bf16x8 fetch_nat_o(TileAt tile, const LaneOffsets<D>& o, int row0, int cb) {
-    union { s16x4 v[2]; bf16x8 b; } u;
+__device__ inline h16x8 fetch_nat_o(TileAt tile, const LaneOffsets<D>& o, int row0, int cb) {
+    union { s16x4 v[2]; h16x8 b; } u;
     u.v[0] = lds_read_tr_at((uint32_t)o.nat[0][cb], tile.off + row0 * D * 2);
     u.v[1] = lds_read_tr_at((uint32_t)o.nat[1][cb], tile.off + row0 * D * 2);
     return u.b;
 }
 template <int D, bool kPinBase = false>
-__device__ inline bf16x8 fetch_nat_o(const char* tile, const LaneOffsets<D>& o, int row0, int cb) {
-    union { s16x4 v[2]; bf16x8 b; } u;
+__device__ inline h16x8 fetch_nat_o(const char* tile, const LaneOffsets<D>& o, int row0, int cb) {
+    union { s16x4 v[2]; h16x8 b; } u;
     if (kPinBase) {
         u.v[0] = lds_read_tr_at(lds_lane_base(tile, o.nat[0][cb]), row0 * D * 2);
         u.v[1] = lds_read_tr_at(lds_lane_base(tile, o.nat[1][cb]), row0 * D * 2);
@@ -206,16 +232,16 @@ __device__ inline bf16x8 fetch_nat_o(const char* tile, const LaneOffsets<D>& o, 
     return u.b;
 }
 // fetch_rows_o with the pinned base (see fetch_cols_o): row 32*t + lane%32 of a tile in natural or MFMA order
-template <int D> __device__ inline bf16x8 fetch_rows_p(TileAt tile, const LaneOffsets<D>& o, int t, int ks) {
+template <int D> __device__ inline h16x8 fetch_rows_p(TileAt tile, const LaneOffsets<D>& o, int t, int ks) {
     return fetch_rows_o<D>(tile, o, t, ks);
 }
-template <int D> __device__ inline bf16x8 fetch_rows_p(const char* tile, const LaneOffsets<D>& o, int t, int ks) {
-    return *(const __attribute__((address_space(3))) bf16x8*)((__attribute__((address_space(3))) char*)(uintptr_t)lds_lane_base(tile, o.rows[ks]) + t * 32 * D * 2);
+template <int D> __device__ inline h16x8 fetch_rows_p(const char* tile, const LaneOffsets<D>& o, int t, int ks) {
+    return *(const __attribute__((address_space(3))) h16x8*)((__attribute__((address_space(3))) char*)(uintptr_t)lds_lane_base(tile, o.rows[ks]) + t * 32 * D * 2);
 }
 // The same with the two lane offsets already picked (column block chosen at run time:
 // indexing the offset table with a run-time value would push it into scratch memory).
-template <int ROWD> __device__ inline bf16x8 fetch_nat_2(const char* tile, int off0, int off1, int row0) {
-    union { s16x4 v[2]; bf16x8 b; } u;
+template <int ROWD> __device__ inline h16x8 fetch_nat_2(const char* tile, int off0, int off1, int row0) {
+    union { s16x4 v[2]; h16x8 b; } u;
     u.v[0] = lds_read_tr(tile + off0 + row0 * ROWD * 2);
     u.v[1] = lds_read_tr(tile + off1 + row0 * ROWD * 2);
     return u.b;
@@ -260,7 +286,7 @@ template <int D> struct TileCopy {
     __device__ inline void scale(float f) {      // every bf16 of the tile times f (fp32 product, rounded back)
 #pragma unroll
         for (int r = 0; r < kPerThread; ++r) {
-            bf16x8 b[1] = {__builtin_bit_cast(bf16x8, regs[r])};
+            h16x8 b[1] = {__builtin_bit_cast(h16x8, regs[r])};
             prescale_frags(b, f);
             regs[r] = __builtin_bit_cast(u32x4, b[0]);
         }
@@ -372,7 +398,7 @@ __device__ inline void stage_acc_tile(char* staging, int row0, int col0, const f
         // (round to nearest even in hardware), two 2-byte stores
         const int row = row0 + 8 * (r >> 2) + 4 * h + (r & 3);
         const f32x2 v = {acc[r] * scale, acc[r + 1] * scale};
-        const uint32_t w = __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2));
+        const uint32_t w = __builtin_bit_cast(uint32_t, __builtin_convertvector(v, h16x2));
         *(uint16_t*)(staging + row * (D * 2) + (col0 + n) * 2) = (uint16_t)w;
         *(uint16_t*)(staging + (row + 1) * (D * 2) + (col0 + n) * 2) = (uint16_t)(w >> 16);
     }
@@ -392,32 +418,36 @@ __device__ inline void store_staged_rows(const char* staging, const TensorArg& t
 // columns 16*ks + 8*h .. +7 for every ks.  Rows >= len read as zero.  One address, one
 // predicate; the ks fragments are at constant offsets from it.
 template <int D>
-__device__ inline void load_row_frags(bf16x8 (&f)[D / 16], const TensorArg& t, int64_t base, int row,
+__device__ inline void load_row_frags(h16x8 (&f)[D / 16], const TensorArg& t, int64_t base, int row,
                                       int len, int lane) {
     const int h = lane >> 5;
     const char* ptr = t.ptr + 2 * (base + (int64_t)row * t.st + 8 * h);
     if (row < len) {
 #pragma unroll
-        for (int ks = 0; ks < D / 16; ++ks) f[ks] = __builtin_bit_cast(bf16x8, *(const u32x4*)(ptr + 32 * ks));
+        for (int ks = 0; ks < D / 16; ++ks) f[ks] = __builtin_bit_cast(h16x8, *(const u32x4*)(ptr + 32 * ks));
     } else {
 #pragma unroll
-        for (int ks = 0; ks < D / 16; ++ks) f[ks] = bf16x8{0};
+        for (int ks = 0; ks < D / 16; ++ks) f[ks] = h16x8{0};
     }
 }
 
-__device__ inline bf16x8 pack8(const float* p) {
-    bf16x8 r;
+__device__ inline h16x8 pack8(const float* p) {
+    h16x8 r;
 #pragma unroll
     for (int i = 0; i < 8; i += 2) {
         f32x2 v = {p[i], p[i + 1]};
-        bf16x2 b = __builtin_convertvector(v, bf16x2);
+        h16x2 b = __builtin_convertvector(v, h16x2);
         r[i] = b[0]; r[i + 1] = b[1];
     }
     return r;
 }
 
-__device__ inline f32x16 mfma(bf16x8 a, bf16x8 b, f32x16 c) {
+__device__ inline f32x16 mfma(h16x8 a, h16x8 b, f32x16 c) {
+#ifdef SBA_ELEM_F16
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
+#else
     return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
+#endif
 }
 
 // S^T tile pair for one wave, raw MFMA accumulators (no vector-ALU instruction touches
@@ -425,14 +455,14 @@ __device__ inline f32x16 mfma(bf16x8 a, bf16x8 b, f32x16 c) {
 // raw[t][r] = (K Q^T)[key_local = 32h + 16t + r][query n].
 template <int D, bool kBatch = (D == 128), class Tile>
 __device__ inline void score_raw_o(f32x16 (&raw)[2], Tile ktile, const LaneOffsets<D>& o,
-                                   const bf16x8 (&qf)[D / 16]) {
+                                   const h16x8 (&qf)[D / 16]) {
     // tile 1 first: the product chain starts at its keys (the right half of the lane's 32), and
     // can begin while the MFMAs of tile 0 are still in flight
 #pragma unroll
     for (int t = 1; t >= 0; --t) {
         // all operands of the tile are requested before its first MFMA: at head_dim 128 the kernels
         // run one or two waves per SIMD, and nothing else hides an LDS round trip per MFMA
-        bf16x8 a[D / 16];
+        h16x8 a[D / 16];
 #pragma unroll
         for (int ks = 0; ks < D / 16; ++ks) a[ks] = fetch_rows_o<D>(ktile, o, t, ks);
         if (kBatch) __builtin_amdgcn_sched_barrier(0);
@@ -453,7 +483,7 @@ __device__ inline void scale_scores(float (&x)[32], const f32x16 (&raw)[2], floa
 
 template <int D, bool kBatch = (D == 128), class Tile>
 __device__ inline void score_tiles_o(float (&x)[32], Tile ktile, const LaneOffsets<D>& o,
-                                     const bf16x8 (&qf)[D / 16], float scale2) {
+                                     const h16x8 (&qf)[D / 16], float scale2) {
     f32x16 raw[2];
     score_raw_o<D, kBatch>(raw, ktile, o, qf);
     scale_scores(x, raw, scale2);
@@ -462,7 +492,7 @@ __device__ inline void score_tiles_o(float (&x)[32], Tile ktile, const LaneOffse
 // Score tiles from pre-scaled fragments: x[16*t + r] = raw accumulator, no vector work.
 template <int D, bool kBatch = (D == 128), class Tile>
 __device__ inline void score_tiles_ps(float (&x)[32], Tile ktile, const LaneOffsets<D>& o,
-                                      const bf16x8 (&qf)[D / 16]) {
+                                      const h16x8 (&qf)[D / 16]) {
     f32x16 raw[2];
     score_raw_o<D, kBatch>(raw, ktile, o, qf);
 #pragma unroll
@@ -591,7 +621,7 @@ template <int N> __device__ inline void scale_clamped(float (&x)[N], float f) {
 constexpr float kFastChainLimit = 0x1p96f;
 
 template <bool kWeights>
-__device__ inline bool forward_weights_fast(float (&x)[32], bf16x8 (&pf)[4], float& R, int lane, float& lane_carry) {
+__device__ inline bool forward_weights_fast(float (&x)[32], h16x8 (&pf)[4], float& R, int lane, float& lane_carry) {
     float W = 1.0f;
 #pragma unroll
     for (int idx = 31; idx >= 0; --idx) {
@@ -652,15 +682,15 @@ __device__ inline void stick_weights_hooked(float (&x)[32], float (&beta)[32], f
 template <int D, class Tile>
 __device__ inline void stick_weights_and_dp(float (&x)[32], float (&beta)[32], float (&dp)[32], float& R, int lane,
                                             float* lane_carry, Tile vtile, const LaneOffsets<D>& o,
-                                            const bf16x8 (&dof)[D / 16]) {
+                                            const h16x8 (&dof)[D / 16]) {
     constexpr int kPer = D / 64;               // MFMAs per segment: 2 tiles x D/16 slices over 8 segments
     f32x16 dacc[2];
-    bf16x8 nx[kPer];
+    h16x8 nx[kPer];
     // MFMA m (0 .. D/8 - 1): tile t = m & 1, slice ks = m >> 1 (neighbours use different accumulators)
 #pragma unroll
     for (int i = 0; i < kPer; ++i) nx[i] = fetch_rows_o<D>(vtile, o, i & 1, i >> 1);
     stick_weights_hooked(x, beta, R, lane, lane_carry, [&](int seg) {
-        bf16x8 cur[kPer];
+        h16x8 cur[kPer];
 #pragma unroll
         for (int i = 0; i < kPer; ++i) cur[i] = nx[i];
         if (seg < 7) {
@@ -690,10 +720,10 @@ __device__ inline void stick_weights_and_dp(float (&x)[32], float (&beta)[32], f
 // priority tied to progress, whichever wave is behind goes first and both arrive together.
 template <int D, bool kPaced = false, class Tile>
 __device__ inline float carried_weights_and_dp(float (&x)[32], float (&beta)[32], float (&dp)[32], float F,
-                                               Tile vtile, const LaneOffsets<D>& o, const bf16x8 (&dof)[D / 16]) {
+                                               Tile vtile, const LaneOffsets<D>& o, const h16x8 (&dof)[D / 16]) {
     constexpr int kPer = D / 64;
     f32x16 dacc[2];
-    bf16x8 nx[kPer];
+    h16x8 nx[kPer];
 #pragma unroll
     for (int i = 0; i < kPer; ++i) nx[i] = fetch_rows_o<D>(vtile, o, i & 1, i >> 1);
     if (kPaced) __builtin_amdgcn_s_setprio(3);
@@ -703,7 +733,7 @@ __device__ inline float carried_weights_and_dp(float (&x)[32], float (&beta)[32]
             else if (seg == 3) __builtin_amdgcn_s_setprio(1);
             else if (seg == 5) __builtin_amdgcn_s_setprio(0);
         }
-        bf16x8 cur[kPer];
+        h16x8 cur[kPer];
 #pragma unroll
         for (int i = 0; i < kPer; ++i) cur[i] = nx[i];
         if (seg < 7) {
@@ -752,8 +782,8 @@ __device__ inline void mask_step(float (&x)[32], int key_first, int qi, int stri
 }
 
 // Row fetch from a natural-order tile: 8 bf16 of row `row`, columns 16*ks + 8*h .. +7.
-template <int ROWD> __device__ inline bf16x8 fetch_row_nat(const char* tile, int row, int ks, int lane) {
-    return *(const bf16x8*)(tile + tile_offset<ROWD>(row, 2 * ks + (lane >> 5)));
+template <int ROWD> __device__ inline h16x8 fetch_row_nat(const char* tile, int row, int ks, int lane) {
+    return *(const h16x8*)(tile + tile_offset<ROWD>(row, 2 * ks + (lane >> 5)));
 }
 
 // dP^T tile pair: dp[16*t + r] = (V dO^T)[key_local][query].  The gradient of `rem` is not
@@ -763,7 +793,7 @@ template <int ROWD> __device__ inline bf16x8 fetch_row_nat(const char* tile, int
 // tables carry it (see the dQ kernels).  `init` is what the accumulators start from (zero).
 template <int D, class Tile>
 __device__ inline void dp_tiles_o(float (&dp)[32], Tile vtile, const LaneOffsets<D>& o,
-                                  const bf16x8 (&dof)[D / 16], float init = 0.f) {
+                                  const h16x8 (&dof)[D / 16], float init = 0.f) {
 #pragma unroll
     for (int t = 0; t < 2; ++t) {
         f32x16 acc;
@@ -862,7 +892,7 @@ __device__ inline float carried_beta_g(float (&x)[32], float (&dp)[32], float F,
 // (The running sum must stay a plain add: fused with the product that made g - which the compiler does across
 // function boundaries when allowed to - it would need the two factors of every g alive instead of g itself,
 // 32 registers more than this kernel has.)
-__device__ inline void walk_logit_grads_g(const float (&beta)[32], const float (&g)[32], float G, bf16x8 (&zf)[4]) {
+__device__ inline void walk_logit_grads_g(const float (&beta)[32], const float (&g)[32], float G, h16x8 (&zf)[4]) {
 #pragma clang fp contract(off)
 #pragma unroll
     for (int c = 0; c < 4; ++c) {
@@ -892,7 +922,7 @@ __device__ inline float chain_beta_gprime(float (&x)[32], float (&dp)[32], float
     return clamp01(L);
 }
 // Out: zf[c] = dz of keys 8c .. 8c+7 packed to bf16 (the B operand of dQ^T += K^T dZ^T).
-__device__ inline void walk_logit_grads(const float (&beta)[32], const float (&g)[32], float F, float G, bf16x8 (&zf)[4]) {
+__device__ inline void walk_logit_grads(const float (&beta)[32], const float (&g)[32], float F, float G, h16x8 (&zf)[4]) {
 #pragma unroll
     for (int c = 0; c < 4; ++c) {
         float dz[8];
@@ -930,4 +960,5 @@ __device__ inline void logit_grads_apply(const float (&beta)[32], float (&dp)[32
     }
 }
 
+}  // inline namespace SBA_ELEM_NS
 }  // namespace sba

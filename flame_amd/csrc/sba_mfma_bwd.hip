@@ -27,6 +27,7 @@
 #include "sba_mfma.h"
 
 namespace sba {
+inline namespace SBA_ELEM_NS {
 
 // The dQ pass leaves its pre-scaled Q fragments (q times scale * log2 e, rounded to bf16: the operand every
 // row-owner kernel multiplies with) behind for the key-owner stream kernel, which then needs no scaling of its
@@ -34,7 +35,7 @@ namespace sba {
 // lane's four 16-byte chunks (columns 16 ks + 8 h ..).  head_dim 64 only, and only where the launcher asks for it.
 template <int D>
 __device__ inline void store_scaled_q(const KParams& p, const Job& job, int head, int qi, int lane,
-                                      const bf16x8 (&qf)[D / 16]) {
+                                      const h16x8 (&qf)[D / 16]) {
     if (D != 64 || !p.q_scaled.ptr || qi >= job.len) return;
     char* row = p.q_scaled.ptr + 2 * ((int64_t)job.seq * p.q_scaled.sb + (int64_t)head * p.q_scaled.sh +
                                       (int64_t)(job.tok0 + qi) * p.q_scaled.st + 8 * (lane >> 5));
@@ -70,7 +71,7 @@ __global__ __launch_bounds__(kThreads, (D == 64 && kLean) ? 3 : (D <= 128 ? 2 : 
     const int64_t dobase = (int64_t)job.seq * p.d_o.sb + (int64_t)head * p.d_o.sh + (int64_t)job.tok0 * p.d_o.st;
 
     if (blockIdx.x == 0 && threadIdx.x == 0 && p.gave_up) *p.gave_up = 0;     // error word of the launch pair, see wait_for_count()
-    bf16x8 qf[D / 16], dof[D / 16];
+    h16x8 qf[D / 16], dof[D / 16];
     load_row_frags<D>(qf, p.q, qbase, qi, job.len, lane);
     prescale_frags(qf, p.scale2);          // the score MFMAs then deliver base-2 logits
     load_row_frags<D>(dof, p.d_o, dobase, qi, job.len, lane);
@@ -108,7 +109,7 @@ __global__ __launch_bounds__(kThreads, (D == 64 && kLean) ? 3 : (D <= 128 ? 2 : 
     // (last of the prologue's loads: its conversion waits for it, and with it for everything requested before)
     float dr = 0.f;
     if (row_ok && p.d_rem.ptr)
-        dr = Elem<uint16_t>::load(p.d_rem.ptr, (int64_t)job.seq * p.d_rem.sb + (int64_t)head * p.d_rem.sh + job.tok0 + qi);
+        dr = Elem16::load(p.d_rem.ptr, (int64_t)job.seq * p.d_rem.sb + (int64_t)head * p.d_rem.sh + job.tok0 + qi);
     wait_global_memory();
     __syncthreads();
     // (behind the prologue's loads: a store in front of them would keep the compiler from issuing them together,
@@ -133,7 +134,7 @@ __global__ __launch_bounds__(kThreads, (D == 64 && kLean) ? 3 : (D <= 128 ? 2 : 
             vc.issue((step + 1) * kKeyBlock, job.len, lds + (buf ^ 1) * 2 * kTile + kTile);
         }
         if (!skip) {
-            bf16x8 zf[4];
+            h16x8 zf[4];
             if constexpr (D == 128 || kLean) {
                 // Register-lean arrangement (two arrays of 32 live instead of four: two waves per SIMD
                 // instead of one): scores and dP first, then the chain over both in place.
@@ -185,7 +186,7 @@ __global__ __launch_bounds__(kThreads, (D == 64 && kLean) ? 3 : (D <= 128 ? 2 : 
             }
 #pragma unroll
             for (int c = 0; c < 4; ++c) {      // (operands of a key group requested together, see score_raw_o)
-                bf16x8 kt[D / 32];
+                h16x8 kt[D / 32];
 #pragma unroll
                 for (int db = 0; db < D / 32; ++db) kt[db] = fetch_cols_o<D>(ktile, lo, db, c);
                 if (D == 128) __builtin_amdgcn_sched_barrier(0);
@@ -211,7 +212,7 @@ __global__ __launch_bounds__(kThreads, (D == 64 && kLean) ? 3 : (D <= 128 ? 2 : 
             for (int g = 0; g < 4; ++g) {
                 f32x2 a = {dqacc[db][4 * g] * p.scale, dqacc[db][4 * g + 1] * p.scale};
                 f32x2 b = {dqacc[db][4 * g + 2] * p.scale, dqacc[db][4 * g + 3] * p.scale};
-                bf16x2 pa = __builtin_convertvector(a, bf16x2), pb = __builtin_convertvector(b, bf16x2);
+                h16x2 pa = __builtin_convertvector(a, h16x2), pb = __builtin_convertvector(b, h16x2);
                 uint2 w;
                 w.x = __builtin_bit_cast(uint32_t, pa);
                 w.y = __builtin_bit_cast(uint32_t, pb);
@@ -256,7 +257,7 @@ __global__ __launch_bounds__(2 * kThreads, 2) void mfma_bwd_dq2_kernel(KParams p
     const int64_t dobase = (int64_t)job.seq * p.d_o.sb + (int64_t)head * p.d_o.sh + (int64_t)job.tok0 * p.d_o.st;
 
     if (blockIdx.x == 0 && threadIdx.x == 0 && p.gave_up) *p.gave_up = 0;     // error word of the launch pair, see wait_for_count()
-    bf16x8 qf[D / 16], dof[D / 16];
+    h16x8 qf[D / 16], dof[D / 16];
     load_row_frags<D>(qf, p.q, qbase, qi, job.len, lane);
     prescale_frags(qf, p.scale2);          // the score MFMAs then deliver base-2 logits
     load_row_frags<D>(dof, p.d_o, dobase, qi, job.len, lane);
@@ -292,7 +293,7 @@ __global__ __launch_bounds__(2 * kThreads, 2) void mfma_bwd_dq2_kernel(KParams p
     // (last of the prologue's loads: its conversion waits for it, and with it for everything requested before)
     float dr = 0.f;
     if (row_ok && p.d_rem.ptr)
-        dr = Elem<uint16_t>::load(p.d_rem.ptr, (int64_t)job.seq * p.d_rem.sb + (int64_t)head * p.d_rem.sh + job.tok0 + qi);
+        dr = Elem16::load(p.d_rem.ptr, (int64_t)job.seq * p.d_rem.sb + (int64_t)head * p.d_rem.sh + job.tok0 + qi);
     wait_global_memory();
     __syncthreads();
     if (grp == 0) store_scaled_q<D>(p, job, head, qi, lane, qf);      // (placed as in the one-step kernel)
@@ -346,7 +347,7 @@ __global__ __launch_bounds__(2 * kThreads, 2) void mfma_bwd_dq2_kernel(KParams p
             Gstore = Glane;
             g_pending = true;
             logit_grads_apply(beta, dp, Glane);
-            bf16x8 zf[4];
+            h16x8 zf[4];
 #pragma unroll
             for (int c = 0; c < 4; ++c) zf[c] = pack8(&dp[8 * c]);
 #pragma unroll
@@ -389,7 +390,7 @@ __global__ __launch_bounds__(2 * kThreads, 2) void mfma_bwd_dq2_kernel(KParams p
             for (int g = 0; g < 4; ++g) {
                 f32x2 a = {dqacc[db][4 * g] * p.scale, dqacc[db][4 * g + 1] * p.scale};
                 f32x2 b = {dqacc[db][4 * g + 2] * p.scale, dqacc[db][4 * g + 3] * p.scale};
-                bf16x2 pa = __builtin_convertvector(a, bf16x2), pb = __builtin_convertvector(b, bf16x2);
+                h16x2 pa = __builtin_convertvector(a, h16x2), pb = __builtin_convertvector(b, h16x2);
                 uint2 w;
                 w.x = __builtin_bit_cast(uint32_t, pa);
                 w.y = __builtin_bit_cast(uint32_t, pb);
@@ -466,7 +467,7 @@ __global__ __launch_bounds__(kThreads, 2) void mfma_bwd_dkv_kernel(KParams p) {
     const int qb0 = job.rb;
     // prefetched state of the first step
     float Rn = 1.0f, Gn = 0.0f;
-    bf16x8 qfn[D / 16];
+    h16x8 qfn[D / 16];
     {
         const int qi0 = qb0 * kRowBlock + 32 * wave + n;
         load_row_frags<D>(qfn, p.q, qbase, qi0, job.len, lane);
@@ -486,7 +487,7 @@ __global__ __launch_bounds__(kThreads, 2) void mfma_bwd_dkv_kernel(KParams p) {
         //     fragments are requested now and not needed before the weights are done.  Each
         //     row is fetched from global memory exactly once: the fragments are also what the
         //     shared Q / dO tiles of the reduction are assembled from.
-        bf16x8 qf[D / 16], dof[D / 16];
+        h16x8 qf[D / 16], dof[D / 16];
 #pragma unroll
         for (int ks = 0; ks < D / 16; ++ks) qf[ks] = qfn[ks];
         load_row_frags<D>(dof, p.d_o, dobase, qi, job.len, lane);
@@ -504,7 +505,7 @@ __global__ __launch_bounds__(kThreads, 2) void mfma_bwd_dkv_kernel(KParams p) {
         //     previous step's reduction, so the tiles are free)
 #pragma unroll
         for (int ks = 0; ks < D / 16; ++ks)
-            *(bf16x8*)(qtile + tile_offset<D>(32 * wave + n, 2 * ks + h)) = qf[ks];
+            *(h16x8*)(qtile + tile_offset<D>(32 * wave + n, 2 * ks + h)) = qf[ks];
         // (3) weights of this wave's 32 queries
         float x[32], dp[32];
         const bool skip = key0 + strict > q0w + 31 || q0w >= job.len;
@@ -515,27 +516,27 @@ __global__ __launch_bounds__(kThreads, 2) void mfma_bwd_dkv_kernel(KParams p) {
             stick_weights<true>(x, beta, R, lane);
 #pragma unroll
             for (int ks = 0; ks < D / 16; ++ks)
-                *(bf16x8*)(dotile + tile_offset<D>(32 * wave + n, 2 * ks + h)) = dof[ks];
+                *(h16x8*)(dotile + tile_offset<D>(32 * wave + n, 2 * ks + h)) = dof[ks];
             dp_tiles_o<D>(dp, vtile, lo, dof);
             logit_grads<true>(x, beta, dp, Gc, lane);
         } else {
 #pragma unroll
             for (int ks = 0; ks < D / 16; ++ks)
-                *(bf16x8*)(dotile + tile_offset<D>(32 * wave + n, 2 * ks + h)) = dof[ks];
+                *(h16x8*)(dotile + tile_offset<D>(32 * wave + n, 2 * ks + h)) = dof[ks];
 #pragma unroll
             for (int idx = 0; idx < 32; ++idx) { x[idx] = 0.f; dp[idx] = 0.f; }
         }
 #pragma unroll
         for (int c = 0; c < 4; ++c) {
-            *(bf16x8*)(zp + tile_offset<64>(32 * wave + n, 4 * h + c)) = pack8(&x[8 * c]);
-            *(bf16x8*)(zd + tile_offset<64>(32 * wave + n, 4 * h + c)) = pack8(&dp[8 * c]);
+            *(h16x8*)(zp + tile_offset<64>(32 * wave + n, 4 * h + c)) = pack8(&x[8 * c]);
+            *(h16x8*)(zd + tile_offset<64>(32 * wave + n, 4 * h + c)) = pack8(&dp[8 * c]);
         }
         __syncthreads();                       // weights and tiles of all waves visible
         // (4) dK[key][d] += sum_q dz[q][key] Q[q][d];  dV[key][d] += sum_q a[q][key] dO[q][d]
 #pragma unroll
         for (int c2 = 0; c2 < 8; ++c2) {
-            bf16x8 az = fetch_nat_2<64>(zd, za0, za1, 16 * c2);
-            bf16x8 ap = fetch_nat_2<64>(zp, za0, za1, 16 * c2);
+            h16x8 az = fetch_nat_2<64>(zd, za0, za1, 16 * c2);
+            h16x8 ap = fetch_nat_2<64>(zp, za0, za1, 16 * c2);
 #pragma unroll
             for (int i = 0; i < D / 64; ++i) {
                 dkacc[i] = mfma(az, fetch_nat_2<D>(qtile, qb0o[i], qb1o[i], 16 * c2), dkacc[i]);
@@ -706,7 +707,7 @@ __global__ __launch_bounds__((NP + 4) * 64, NP == 4 ? 2 : 3) void mfma_bwd_dkv_s
             const char* vtile = vtiles + (item & 1) * kTile;
             // rows 32kh.. of the K and V tiles are this wave's keys, in the order that puts 16
             // consecutive keys into a lane's accumulator registers (see request_keys)
-            bf16x8 kfr[D / 16], vfr[D / 16];
+            h16x8 kfr[D / 16], vfr[D / 16];
 #pragma unroll
             for (int ks = 0; ks < D / 16; ++ks) {
                 kfr[ks] = fetch_rows_o<D>(ktile, lo, kh, ks);
@@ -736,7 +737,7 @@ __global__ __launch_bounds__((NP + 4) * 64, NP == 4 ? 2 : 3) void mfma_bwd_dkv_s
                     const bool sees = qi < len && qi - strict - key0 + 1 > 0;
                     const float Rt = sees ? (kh ? cv.x : cv.z) : 1.0f;
                     const float Gt = sees ? (kh ? cv.w : cv.y) : 0.0f;
-                    bf16x8 qf[D / 16], dof[D / 16];
+                    h16x8 qf[D / 16], dof[D / 16];
 #pragma unroll
                     for (int ks = 0; ks < D / 16; ++ks) {
                         qf[ks] = fetch_rows_o<D>(qtile, lo, w4, ks);
@@ -765,16 +766,16 @@ __global__ __launch_bounds__((NP + 4) * 64, NP == 4 ? 2 : 3) void mfma_bwd_dkv_s
                     own_tile_grads(x, beta, dp, Gt, lane);
 #pragma unroll
                     for (int c = 0; c < 2; ++c) {
-                        *(bf16x8*)(zp + tile_offset<64>(32 * w4 + n, 4 * kh + 2 * h + c)) = pack8(&x[8 * c]);
-                        *(bf16x8*)(zd + tile_offset<64>(32 * w4 + n, 4 * kh + 2 * h + c)) = pack8(&dp[8 * c]);
+                        *(h16x8*)(zp + tile_offset<64>(32 * w4 + n, 4 * kh + 2 * h + c)) = pack8(&x[8 * c]);
+                        *(h16x8*)(zd + tile_offset<64>(32 * w4 + n, 4 * kh + 2 * h + c)) = pack8(&dp[8 * c]);
                     }
                 } else {
                     if (x_now) __syncthreads();    // X
-                    const bf16x8 none = {0, 0, 0, 0, 0, 0, 0, 0};
+                    const h16x8 none = {0, 0, 0, 0, 0, 0, 0, 0};
 #pragma unroll
                     for (int c = 0; c < 2; ++c) {
-                        *(bf16x8*)(zp + tile_offset<64>(32 * w4 + n, 4 * kh + 2 * h + c)) = none;
-                        *(bf16x8*)(zd + tile_offset<64>(32 * w4 + n, 4 * kh + 2 * h + c)) = none;
+                        *(h16x8*)(zp + tile_offset<64>(32 * w4 + n, 4 * kh + 2 * h + c)) = none;
+                        *(h16x8*)(zd + tile_offset<64>(32 * w4 + n, 4 * kh + 2 * h + c)) = none;
                     }
                 }
                 __syncthreads();               // A
@@ -788,7 +789,7 @@ __global__ __launch_bounds__((NP + 4) * 64, NP == 4 ? 2 : 3) void mfma_bwd_dkv_s
         for (int item = 0;; ++item) {
             const char* vtile = vtiles + (item & 1) * kTile;
             // the key block of an item never changes: its score and dP operands stay in registers
-            bf16x8 kfr[2][D / 16], vfr[2][D / 16];
+            h16x8 kfr[2][D / 16], vfr[2][D / 16];
 #pragma unroll
             for (int t = 0; t < 2; ++t)
 #pragma unroll
@@ -828,7 +829,7 @@ __global__ __launch_bounds__((NP + 4) * 64, NP == 4 ? 2 : 3) void mfma_bwd_dkv_s
                     const bool sees = qi < len && qi - strict - (key0 + 32 * h) + 1 > 0;
                     const float R = sees ? (h ? cv.x : cv.z) : (qi < len ? 1.0f : 0.0f);
                     const float Gc = sees ? (h ? cv.w : cv.y) : 0.0f;
-                    bf16x8 qf[D / 16], dof[D / 16];
+                    h16x8 qf[D / 16], dof[D / 16];
 #pragma unroll
                     for (int ks = 0; ks < D / 16; ++ks) {
                         qf[ks] = fetch_rows_o<D>(qtile, lo, w4, ks);
@@ -863,16 +864,16 @@ __global__ __launch_bounds__((NP + 4) * 64, NP == 4 ? 2 : 3) void mfma_bwd_dkv_s
                     logit_grads_from<32>(x, beta, dp, Gc);
 #pragma unroll
                     for (int c = 0; c < 4; ++c) {
-                        *(bf16x8*)(zp + tile_offset<64>(32 * w4 + n, 4 * h + c)) = pack8(&x[8 * c]);
-                        *(bf16x8*)(zd + tile_offset<64>(32 * w4 + n, 4 * h + c)) = pack8(&dp[8 * c]);
+                        *(h16x8*)(zp + tile_offset<64>(32 * w4 + n, 4 * h + c)) = pack8(&x[8 * c]);
+                        *(h16x8*)(zd + tile_offset<64>(32 * w4 + n, 4 * h + c)) = pack8(&dp[8 * c]);
                     }
                 } else {
                     if (x_now) __syncthreads();    // X
-                    const bf16x8 none = {0, 0, 0, 0, 0, 0, 0, 0};
+                    const h16x8 none = {0, 0, 0, 0, 0, 0, 0, 0};
 #pragma unroll
                     for (int c = 0; c < 4; ++c) {
-                        *(bf16x8*)(zp + tile_offset<64>(32 * w4 + n, 4 * h + c)) = none;
-                        *(bf16x8*)(zd + tile_offset<64>(32 * w4 + n, 4 * h + c)) = none;
+                        *(h16x8*)(zp + tile_offset<64>(32 * w4 + n, 4 * h + c)) = none;
+                        *(h16x8*)(zd + tile_offset<64>(32 * w4 + n, 4 * h + c)) = none;
                     }
                 }
                 __syncthreads();               // A
@@ -1021,7 +1022,7 @@ __global__ __launch_bounds__((NP + 4) * 64, NP == 4 ? 2 : 3) void mfma_bwd_dkv_s
             constexpr int kBatch = NP == 8 ? 2 : 4;        // NP = 8: three waves per SIMD, fewer registers
 #pragma unroll
             for (int b = 0; b < 8 / kBatch; ++b) {
-                bf16x8 aw[kBatch][2], bx[kBatch];
+                h16x8 aw[kBatch][2], bx[kBatch];
 #pragma unroll
                 for (int j = 0; j < kBatch; ++j) {
                     const int c2 = kBatch * b + j;
@@ -1195,7 +1196,7 @@ __global__ __launch_bounds__(kThreads, D == 64 ? 2 : 1) void mfma_bwd_dkv_own_ke
 
     // A operands of the score tiles: MFMA row m holds key 16*((m>>2)&1) + 4*(m>>3) + (m&3) of
     // the wave, so that the accumulator registers of a lane are 16 consecutive keys
-    bf16x8 kfr[D / 16], vfr[D / 16];
+    h16x8 kfr[D / 16], vfr[D / 16];
     {
         const int m = lane & 31;
         const int key = kb0 + 16 * ((m >> 2) & 1) + 4 * (m >> 3) + (m & 3);
@@ -1250,15 +1251,15 @@ __global__ __launch_bounds__(kThreads, D == 64 ? 2 : 1) void mfma_bwd_dkv_own_ke
     uint32_t zst[4];              // this lane's row of the weight tile: chunks 2h, 2h + 1 (a) and 4 + 2h, 4 + 2h + 1 (dz)
 #pragma unroll
     for (int c = 0; c < 4; ++c) zst[c] = lds_lane_base(ztile, tile_offset<64>(n, (c >> 1) * 4 + 2 * h + (c & 1)));
-    auto put_z = [&](int c, int t, bf16x8 v) __attribute__((always_inline)) {
-        *(__attribute__((address_space(3))) bf16x8*)((__attribute__((address_space(3))) char*)(uintptr_t)zst[c] + t * 32 * 64 * 2) = v;
+    auto put_z = [&](int c, int t, h16x8 v) __attribute__((always_inline)) {
+        *(__attribute__((address_space(3))) h16x8*)((__attribute__((address_space(3))) char*)(uintptr_t)zst[c] + t * 32 * 64 * 2) = v;
     };
 
     auto second_tile_reduction = [&](auto qt, auto dot) __attribute__((always_inline)) {
 #pragma unroll
         for (int kk = 2; kk < 4; ++kk) {
-            const bf16x8 af = fetch_nat_o<64>(zt, lz, 16 * kk, 0);
-            const bf16x8 zf = fetch_nat_o<64>(zt, lz, 16 * kk, 1);
+            const h16x8 af = fetch_nat_o<64>(zt, lz, 16 * kk, 0);
+            const h16x8 zf = fetch_nat_o<64>(zt, lz, 16 * kk, 1);
 #pragma unroll
             for (int db = 0; db < kNB; ++db) {
                 dvacc[db] = mfma(af, fetch_nat_o<D>(dot, lo, 16 * kk, kB0 + db), dvacc[db]);
@@ -1299,7 +1300,7 @@ __global__ __launch_bounds__(kThreads, D == 64 ? 2 : 1) void mfma_bwd_dkv_own_ke
                 {
                     // with one wave on the SIMD (d = 128) nothing hides an LDS round trip in front of
                     // each MFMA: all operands of the tile are requested first
-                    bf16x8 bq[D / 16];
+                    h16x8 bq[D / 16];
 #pragma unroll
                     for (int ks = 0; ks < D / 16; ++ks) bq[ks] = fetch_rows_o<D>(qtile, lo, t, ks);
                     if (D == 128) __builtin_amdgcn_sched_barrier(0);
@@ -1321,12 +1322,12 @@ __global__ __launch_bounds__(kThreads, D == 64 ? 2 : 1) void mfma_bwd_dkv_own_ke
                     auto red_b = [&](int seg, int db) {
                         return (seg & 1) ? fetch_nat_o<D>(pqtile, lo, 32 + 16 * (seg >> 1), kB0 + db) : fetch_nat_o<D>(pdotile, lo, 32 + 16 * (seg >> 1), kB0 + db);
                     };
-                    bf16x8 na = red_a(0), nb[kNB];
+                    h16x8 na = red_a(0), nb[kNB];
 #pragma unroll
                     for (int db = 0; db < kNB; ++db) nb[db] = red_b(0, db);
                     own_tile_weights(x, beta, Rt, lane, [&](int seg) {
-                        const bf16x8 ca = na;
-                        bf16x8 cb[kNB];
+                        const h16x8 ca = na;
+                        h16x8 cb[kNB];
 #pragma unroll
                         for (int db = 0; db < kNB; ++db) cb[db] = nb[db];
                         if (seg < 3) {
@@ -1350,12 +1351,12 @@ __global__ __launch_bounds__(kThreads, D == 64 ? 2 : 1) void mfma_bwd_dkv_own_ke
                     auto red_b = [&](int seg, int db) {
                         return (seg & 1) ? fetch_nat_o<D>(qtile, lo, 16 * (seg >> 1), kB0 + db) : fetch_nat_o<D>(dotile, lo, 16 * (seg >> 1), kB0 + db);
                     };
-                    bf16x8 na = red_a(0), nb[kNB];
+                    h16x8 na = red_a(0), nb[kNB];
 #pragma unroll
                     for (int db = 0; db < kNB; ++db) nb[db] = red_b(0, db);
                     own_tile_weights(x, beta, Rt, lane, [&](int seg) {
-                        const bf16x8 ca = na;
-                        bf16x8 cb[kNB];
+                        const h16x8 ca = na;
+                        h16x8 cb[kNB];
 #pragma unroll
                         for (int db = 0; db < kNB; ++db) cb[db] = nb[db];
                         if (seg < 3) {
@@ -1371,7 +1372,7 @@ __global__ __launch_bounds__(kThreads, D == 64 ? 2 : 1) void mfma_bwd_dkv_own_ke
                     });
                 }
                 {
-                    bf16x8 bd[D / 16];
+                    h16x8 bd[D / 16];
 #pragma unroll
                     for (int ks = 0; ks < D / 16; ++ks) bd[ks] = fetch_rows_o<D>(dotile, lo, t, ks);
                     if (D == 128) __builtin_amdgcn_sched_barrier(0);
@@ -1469,7 +1470,7 @@ __global__ __launch_bounds__(2 * kThreads, 2) void mfma_bwd_dkv_pair_kernel(KPar
 
     // A operands of the score tile: MFMA row m holds key 16*((m>>2)&1) + 4*(m>>3) + (m&3) of the pair,
     // so that the accumulator registers of a lane are 16 consecutive keys (as in the own-keys kernel)
-    bf16x8 kfr[D / 16], vfr[D / 16];
+    h16x8 kfr[D / 16], vfr[D / 16];
     {
         const int m = lane & 31;
         const int key = kb0 + 16 * ((m >> 2) & 1) + 4 * (m >> 3) + (m & 3);
@@ -1532,10 +1533,10 @@ __global__ __launch_bounds__(2 * kThreads, 2) void mfma_bwd_dkv_pair_kernel(KPar
     }
     (void)lds0;
     auto rows_at = [&](uint32_t base, int imm) __attribute__((always_inline)) {
-        return *(const __attribute__((address_space(3))) bf16x8*)((__attribute__((address_space(3))) char*)(uintptr_t)base + imm);
+        return *(const __attribute__((address_space(3))) h16x8*)((__attribute__((address_space(3))) char*)(uintptr_t)base + imm);
     };
     auto nat_pair = [&](const uint32_t (&at)[2][2], int col, int imm) __attribute__((always_inline)) {
-        union { s16x4 v[2]; bf16x8 b; } u;
+        union { s16x4 v[2]; h16x8 b; } u;
         u.v[0] = lds_read_tr_at(at[0][col], imm);
         u.v[1] = lds_read_tr_at(at[1][col], imm);
         return u.b;
@@ -1548,7 +1549,7 @@ __global__ __launch_bounds__(2 * kThreads, 2) void mfma_bwd_dkv_pair_kernel(KPar
         const int q0 = q_begin + step * kStep;
         const float Rin = Rn, Gin = Gn;
         // the score operands are requested first: their LDS round trip passes under the scalar work of the tile requests
-        bf16x8 bq[D / 16];
+        h16x8 bq[D / 16];
 #pragma unroll
         for (int ks = 0; ks < D / 16; ++ks) bq[ks] = rows_at(row_at[ks], kQ);
         __builtin_amdgcn_sched_barrier(0);
@@ -1563,9 +1564,9 @@ __global__ __launch_bounds__(2 * kThreads, 2) void mfma_bwd_dkv_pair_kernel(KPar
             const int qt0 = q0 + 32 * r;
             const int qi = qt0 + n;
             if (kb0 + strict > qt0 + 31) {             // this wave's query tile sees none of the keys (the other one does)
-                const bf16x8 none = {0, 0, 0, 0, 0, 0, 0, 0};
+                const h16x8 none = {0, 0, 0, 0, 0, 0, 0, 0};
 #pragma unroll
-                for (int c = 0; c < 4; ++c) *(bf16x8*)(ztile + tile_offset<64>(32 * r + n, 2 * c + h)) = none;
+                for (int c = 0; c < 4; ++c) *(h16x8*)(ztile + tile_offset<64>(32 * r + n, 2 * c + h)) = none;
             } else {
                 float x[16], dp[16];
                 const int nvis = qi < job.len ? qi - strict - (kb0 + 16 * h) + 1 : 0;
@@ -1588,12 +1589,12 @@ __global__ __launch_bounds__(2 * kThreads, 2) void mfma_bwd_dkv_pair_kernel(KPar
                 }
                 // dP = dO V^T between the segments of the chain, its operands fetched one segment ahead
                 constexpr int kPer = D / 64;
-                bf16x8 nx[kPer];
+                h16x8 nx[kPer];
 #pragma unroll
                 for (int i = 0; i < kPer; ++i) nx[i] = rows_at(row_at[i], kDO);
                 f32x16 dacc;
                 own_tile_weights(x, beta, Rt, lane, [&](int seg) {
-                    bf16x8 cur[kPer];
+                    h16x8 cur[kPer];
 #pragma unroll
                     for (int i = 0; i < kPer; ++i) cur[i] = nx[i];
                     if (seg < 3) {
@@ -1611,11 +1612,11 @@ __global__ __launch_bounds__(2 * kThreads, 2) void mfma_bwd_dkv_pair_kernel(KPar
 #pragma unroll
                 for (int i = 0; i < 16; ++i) dp[i] = dacc[i];
                 // a -> columns 16h.. of row (32r + n) now, dz -> columns 32 + 16h.. below
-                *(bf16x8*)(ztile + tile_offset<64>(32 * r + n, 2 * h)) = pack8(&x[0]);
-                *(bf16x8*)(ztile + tile_offset<64>(32 * r + n, 2 * h + 1)) = pack8(&x[8]);
+                *(h16x8*)(ztile + tile_offset<64>(32 * r + n, 2 * h)) = pack8(&x[0]);
+                *(h16x8*)(ztile + tile_offset<64>(32 * r + n, 2 * h + 1)) = pack8(&x[8]);
                 own_tile_grads(x, beta, dp, Gt, lane);
-                *(bf16x8*)(ztile + tile_offset<64>(32 * r + n, 4 + 2 * h)) = pack8(&dp[0]);
-                *(bf16x8*)(ztile + tile_offset<64>(32 * r + n, 4 + 2 * h + 1)) = pack8(&dp[8]);
+                *(h16x8*)(ztile + tile_offset<64>(32 * r + n, 4 + 2 * h)) = pack8(&dp[0]);
+                *(h16x8*)(ztile + tile_offset<64>(32 * r + n, 4 + 2 * h + 1)) = pack8(&dp[8]);
                 __builtin_amdgcn_s_setprio(0);
             }
         }
@@ -1624,8 +1625,8 @@ __global__ __launch_bounds__(2 * kThreads, 2) void mfma_bwd_dkv_pair_kernel(KPar
             // dV += A^T dO, dK += dZ^T Q over the step's 64 queries, this wave's column blocks.  The operands of
             // 16 queries are requested while the MFMAs of the 16 before them run (left to itself the compiler
             // requests them right before their MFMA, which then waits for the LDS round trip: 16 per step).
-            bf16x8 w[2][2], o[2][2 * kBlocks];
-            auto fetch_kk = [&](int kk, bf16x8 (&ww)[2], bf16x8 (&oo)[2 * kBlocks]) __attribute__((always_inline)) {
+            h16x8 w[2][2], o[2][2 * kBlocks];
+            auto fetch_kk = [&](int kk, h16x8 (&ww)[2], h16x8 (&oo)[2 * kBlocks]) __attribute__((always_inline)) {
                 ww[0] = nat_pair(z_at, 0, 16 * kk * 64 * 2);
                 ww[1] = nat_pair(z_at, 1, 16 * kk * 64 * 2);
 #pragma unroll
@@ -1674,9 +1675,12 @@ __global__ __launch_bounds__(2 * kThreads, 2) void mfma_bwd_dkv_pair_kernel(KPar
     }
 }
 
+}  // inline namespace SBA_ELEM_NS
 }  // namespace sba
 
+#ifndef SBA_ELEM_F16
 bool sba_mfma_bwd_available() { return true; }
+#endif
 
 // SBA_DKV_KERNEL=own / =other overrides the choice between the key-owner kernels (tests run
 // both on the same inputs).
@@ -1696,7 +1700,11 @@ static bool lean_dq_kernel(bool by_size) {
     return by_size;
 }
 
+#ifdef SBA_ELEM_F16
+int sba_launch_mfma_f16_bwd(const sba::KParams& kp_in, int phases, hipStream_t s) {
+#else
 int sba_launch_mfma_bwd(const sba::KParams& kp_in, int phases, hipStream_t s) {
+#endif
     using namespace sba;
     KParams kp = kp_in;
     dim3 grid((unsigned)kp.n_jobs * kp.n_heads);

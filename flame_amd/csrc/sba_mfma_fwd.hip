@@ -6,6 +6,7 @@
 #include "sba_mfma.h"
 
 namespace sba {
+inline namespace SBA_ELEM_NS {
 
 // One sweep step of one wave: 32 queries x 64 keys.  Scores (from the pre-scaled Q fragments),
 // mask on the diagonal, weights, O^T += V^T P^T.  kFast: the one-reciprocal chain; it may refuse
@@ -14,13 +15,13 @@ namespace sba {
 // the step), which is what the carry tables keep.
 template <int D, bool kCarryOnly, bool kFast, bool kPinBase>
 __device__ inline bool fwd_step(const char* ktile, const char* vtile, const LaneOffsets<D>& lo,
-                                const bf16x8 (&qf)[D / 16], f32x16 (&oacc)[D / 32], float& R, int lane,
+                                const h16x8 (&qf)[D / 16], f32x16 (&oacc)[D / 32], float& R, int lane,
                                 int key0, int q0w, int qi, int strict, float& lane_carry) {
     const int h = lane >> 5;
     float x[32];
     score_tiles_ps<D>(x, ktile, lo, qf);
     if (key0 + 63 + strict > q0w) mask_step(x, key0 + 32 * h, qi, strict);     // diagonal region
-    bf16x8 pf[4];
+    h16x8 pf[4];
     if (kFast) {
         if (!forward_weights_fast<!kCarryOnly>(x, pf, R, lane, lane_carry)) return false;
     } else {
@@ -34,7 +35,7 @@ __device__ inline bool fwd_step(const char* ktile, const char* vtile, const Lane
     if (!kCarryOnly) {
 #pragma unroll
         for (int c2 = 0; c2 < 2; ++c2) {   // operands of two key groups requested together, ahead of their MFMAs
-            bf16x8 vt[2][D / 32];
+            h16x8 vt[2][D / 32];
 #pragma unroll
             for (int cc = 0; cc < 2; ++cc)
 #pragma unroll
@@ -61,7 +62,7 @@ __device__ inline void store_o_row(const KParams& p, const Job& job, int head, i
         for (int g = 0; g < 4; ++g) {
             f32x2 a = {oacc[db][4 * g], oacc[db][4 * g + 1]};
             f32x2 b = {oacc[db][4 * g + 2], oacc[db][4 * g + 3]};
-            bf16x2 pa = __builtin_convertvector(a, bf16x2), pb = __builtin_convertvector(b, bf16x2);
+            h16x2 pa = __builtin_convertvector(a, h16x2), pb = __builtin_convertvector(b, h16x2);
             uint2 w;
             w.x = __builtin_bit_cast(uint32_t, pa);
             w.y = __builtin_bit_cast(uint32_t, pb);
@@ -92,7 +93,7 @@ __global__ __launch_bounds__(kThreads) void mfma_fwd_kernel(KParams p) {
     const int64_t kbase = (int64_t)job.seq * p.k.sb + (int64_t)head * p.k.sh + (int64_t)job.tok0 * p.k.st;
     const int64_t vbase = (int64_t)job.seq * p.v.sb + (int64_t)head * p.v.sh + (int64_t)job.tok0 * p.v.st;
 
-    bf16x8 qf[D / 16];
+    h16x8 qf[D / 16];
     load_row_frags<D>(qf, p.q, qbase, qi, job.len, lane);
     prescale_frags(qf, p.scale2);
 
@@ -179,7 +180,7 @@ __global__ __launch_bounds__(kThreads) void mfma_fwd_kernel(KParams p) {
     if (qi < job.len && !kCarryOnly) {
         store_o_row<D>(p, job, head, qi, lane, oacc);
         if (h == 0)
-            Elem<uint16_t>::store(p.rem.ptr, (int64_t)job.seq * p.rem.sb + (int64_t)head * p.rem.sh + job.tok0 + qi, R);
+            Elem16::store(p.rem.ptr, (int64_t)job.seq * p.rem.sb + (int64_t)head * p.rem.sh + job.tok0 + qi, R);
     }
 }
 
@@ -218,7 +219,7 @@ __global__ __launch_bounds__(G * kThreads) void mfma_fwd_seg_kernel(KParams p) {
     const int64_t kbase = (int64_t)job.seq * p.k.sb + (int64_t)head * p.k.sh + (int64_t)job.tok0 * p.k.st;
     const int64_t vbase = (int64_t)job.seq * p.v.sb + (int64_t)head * p.v.sh + (int64_t)job.tok0 * p.v.st;
 
-    bf16x8 qf[D / 16];
+    h16x8 qf[D / 16];
     load_row_frags<D>(qf, p.q, qbase, qi, job.len, lane);
     prescale_frags(qf, p.scale2);
     f32x16 oacc[D / 32];
@@ -346,10 +347,11 @@ __global__ __launch_bounds__(G * kThreads) void mfma_fwd_seg_kernel(KParams p) {
                     oacc[db][r] += park[((((g - 1) * 4 + qs) * (D / 32) + db) * 16 + r) * 64 + lane];
         store_o_row<D>(p, job, head, qi, lane, oacc);
         if (h == 0)
-            Elem<uint16_t>::store(p.rem.ptr, (int64_t)job.seq * p.rem.sb + (int64_t)head * p.rem.sh + job.tok0 + qi, all);
+            Elem16::store(p.rem.ptr, (int64_t)job.seq * p.rem.sb + (int64_t)head * p.rem.sh + job.tok0 + qi, all);
     }
 }
 
+}  // inline namespace SBA_ELEM_NS
 }  // namespace sba
 
 // Key segments per sweep for the forward: 4 or 2 (head_dim 128: 2), or 0 = one sweep per workgroup.
@@ -400,7 +402,11 @@ static void launch_seg(int groups, dim3 grid, hipStream_t s, const sba::KParams&
     else hipLaunchKernelGGL((mfma_fwd_seg_kernel<64, 4, kCarryOnly>), grid, dim3(4 * kThreads), 0, s, kp);
 }
 
+#ifdef SBA_ELEM_F16
+int sba_launch_mfma_f16_fwd(const sba::KParams& kp, hipStream_t s) {
+#else
 int sba_launch_mfma_fwd(const sba::KParams& kp, hipStream_t s) {
+#endif
     using namespace sba;
     dim3 grid((unsigned)kp.n_jobs * kp.n_heads);
     const int segments = forward_segments(kp, grid.x);

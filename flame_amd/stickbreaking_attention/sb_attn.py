@@ -156,9 +156,9 @@ def sb_attn_(q, k, v, inv_temp, attend_current):
     if not torch.is_grad_enabled():
         # no backward can follow: detached inputs tell the forward to keep no carry table
         q, k, v = q.detach(), k.detach(), v.detach()
-    if q.dtype == k.dtype == v.dtype == torch.float16:
-        # float16 has no kernels of its own: its values are exact in float32, so it runs on the float32
-        # matrix-core kernels (more precise than float16 arithmetic, at their speed) and comes back rounded
+    if q.dtype == k.dtype == v.dtype == torch.float16 and _lib.float16_needs_float32_route():
+        # float16 has matrix-core kernels of its own (the bf16 sources compiled for float16 elements) and no generic
+        # ones: with those forced its values, exact in float32, run as float32 and come back rounded
         o, rem = StickBreakingAttention.apply(q.float(), k.float(), v.float(), inv_temp, attend_current)
         return o.half(), rem.half()
     return StickBreakingAttention.apply(q, k, v, inv_temp, attend_current)

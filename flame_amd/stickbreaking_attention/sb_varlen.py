@@ -247,8 +247,8 @@ def _apply(q, k, v, cu_seqlens, max_seqlens, inv_temp, attend_current):
     if not torch.is_grad_enabled():
         # no backward can follow: detached inputs tell the forward to keep no carry table
         q, k, v = q.detach(), k.detach(), v.detach()
-    if q.dtype == k.dtype == v.dtype == torch.float16:
-        # float16 runs on the float32 kernels (see sb_attn.sb_attn_) and is rounded on the way out
+    if q.dtype == k.dtype == v.dtype == torch.float16 and _lib.float16_needs_float32_route():
+        # with the generic kernels forced float16 runs as float32 (see sb_attn.sb_attn_) and is rounded on the way out
         o, rem = StickBreakingAttention.apply(q.float(), k.float(), v.float(), cu_seqlens, max_seqlens, inv_temp,
                                               attend_current)
         return o.half(), rem.half()

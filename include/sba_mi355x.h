@@ -27,10 +27,11 @@
  *                          element (h,t,d) at    base + h*stride_h + t*stride_t + d
  * Strides are in elements; the innermost (D) stride is 1.  head_dim is at most 256 (the reference
  * pads it to the next power of two, sb_attn/sb_fwd.py:199).  Problems at head_dim 64 / 128, and
- * bf16 ones at 256 (the matrix-core kernels) need 16-byte aligned tensor pointers, outer strides that are
- * multiples of 16 bytes - 8 bf16 or 4 fp32 elements - and a token stride below 2^23 elements
+ * bf16 / float16 ones at 256 (the matrix-core kernels) need 16-byte aligned tensor pointers, outer strides that are
+ * multiples of 16 bytes - 8 bf16 / float16 or 4 fp32 elements - and a token stride below 2^23 elements
  * (the tile copies address a 64-row tile with 32-bit byte offsets); SBA_ERR_SHAPE otherwise.
  * rem / d_rem are contiguous along tokens.
+ * Wherever the comments below say bf16, float16 (SBA_DTYPE_F16) is sized and handled the same way.
  */
 #ifndef SBA_MI355X_H
 #define SBA_MI355X_H
@@ -46,13 +47,13 @@ extern "C" {
 #define SBA_SCHEDULE_INTS 8   /* int32 per scheduled job, see sba_build_schedule() */
 #define SBA_DOC_MAJOR_GRID 8192 /* workgroups from which the schedule is document-major */
 
-enum { SBA_DTYPE_F32 = 0, SBA_DTYPE_BF16 = 1 };
+enum { SBA_DTYPE_F32 = 0, SBA_DTYPE_BF16 = 1, SBA_DTYPE_F16 = 2 };   /* float16: head_dim 64, 128 or 256 only (the reference's kernels take whatever dtype the tensors have, sb_attn/sb_fwd.py:144-146) */
 
 enum {
     SBA_OK = 0,
     SBA_ERR_NULL = -1,        /* a required pointer is NULL */
     SBA_ERR_SHAPE = -2,       /* non-positive size, head_dim unsupported, bad strides */
-    SBA_ERR_DTYPE = -3,       /* unknown dtype */
+    SBA_ERR_DTYPE = -3,       /* unknown dtype, or float16 at a head_dim other than 64 / 128 / 256 */
     SBA_ERR_WORKSPACE = -4,   /* workspace or bwd_scratch missing or too small */
     SBA_ERR_SCHEDULE = -5,    /* packed layout without a row-block schedule */
     SBA_ERR_LAUNCH = -6,      /* hipGetLastError() after a launch was not hipSuccess */

@@ -49,6 +49,11 @@ def test_argument_checks_without_gpu(lib):
     assert lib.sba_workspace_bytes(C.byref(p)) == 0 and lib.sba_bwd_scratch_bytes(C.byref(p)) == 0
     p.head_dim = 64
     assert lib.sba_fwd(C.byref(p)) == -1          # NULL q/k/v
+    p.dtype = _lib.SBA_DTYPE_F16                  # float16: matrix-core head dims only
+    assert lib.sba_fwd(C.byref(p)) == -1
+    p.head_dim = 96
+    assert lib.sba_fwd(C.byref(p)) == -3
+    p.dtype, p.head_dim = _lib.SBA_DTYPE_BF16, 64
     assert lib.sba_fwd(None) == -1
     assert lib.sba_row_block() == 128
 
@@ -118,6 +123,12 @@ def test_workspace_bytes(lib):
     p.dtype = _lib.SBA_DTYPE_BF16                   # bf16 at 256: matrix cores, two tables each way, the error word, no copy of q
     assert lib.sba_workspace_bytes(C.byref(p)) == 2 * table
     assert lib.sba_bwd_scratch_bytes(C.byref(p)) == 4 * table + 256
+    p.dtype = _lib.SBA_DTYPE_F16                    # float16 is sized like bf16
+    assert lib.sba_workspace_bytes(C.byref(p)) == 2 * table
+    assert lib.sba_bwd_scratch_bytes(C.byref(p)) == 4 * table + 256
+    p.head_dim = 64
+    assert lib.sba_bwd_scratch_bytes(C.byref(p)) == 4 * table + scaled_q + 256
+    p.dtype, p.head_dim = _lib.SBA_DTYPE_BF16, 256
     p.head_dim = 200                                # bf16 in between: generic kernels unless the caller pads to 256
     assert lib.sba_workspace_bytes(C.byref(p)) == 0
     assert lib.sba_bwd_scratch_bytes(C.byref(p)) == 2 * 4096 * 16 * 256 * 4
@@ -236,7 +247,7 @@ def test_op_refuses_cpu_tensors():
 
 
 def test_python_workspace_bound_covers_the_library(lib):
-    for dtype in (_lib.SBA_DTYPE_BF16, _lib.SBA_DTYPE_F32):
+    for dtype in (_lib.SBA_DTYPE_BF16, _lib.SBA_DTYPE_F32, _lib.SBA_DTYPE_F16):
         for (B, H, T, D) in [(1, 16, 4096, 64), (2, 3, 129, 128), (1, 2, 77, 80), (4, 1, 1, 8), (2, 3, 300, 256), (1, 2, 77, 200)]:
             p = _lib.SbaParams()
             p.struct_size = C.sizeof(_lib.SbaParams)

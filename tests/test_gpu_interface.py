@@ -73,9 +73,8 @@ def test_argument_errors_are_python_errors():
         sb_attn_varlen(q, q, q, torch.tensor([0, 100, 299], dtype=torch.int32), 200)
 
 
-def test_float16_runs_on_the_float32_kernels():
-    # float16 inputs: exact in float32, computed there, rounded to float16 on the way out; against the oracle
-    # at the float32 kernels' forward tolerance plus float16's rounding of the results (2^-11 relative)
+def test_float16_results_and_gradients_come_back_as_float16():
+    # float16 inputs run on the float16 matrix-core kernels; against the oracle at bf16's bounds divided by 8
     from flame_amd import sb_attn, sb_attn_varlen
     from oracle import sb_oracle as O
     from helpers import within, max_abs, rel_l2
@@ -86,11 +85,11 @@ def test_float16_runs_on_the_float32_kernels():
     assert o.dtype == rem.dtype == torch.float16
     o.backward(do.cuda())
     o_ref, rem_ref, dq_ref, dk_ref, dv_ref = O.sb_attn_grads_oracle(q, k, v, do, None)
-    within("float16 dense T=300", "o", max_abs(o.float().cpu(), o_ref), 2e-3)
-    within("float16 dense T=300", "rem", max_abs(rem.float().cpu(), rem_ref), 2e-3)
+    within("float16 dense T=300", "o", max_abs(o.float().cpu(), o_ref), 2.5e-3)
+    within("float16 dense T=300", "rem", max_abs(rem.float().cpu(), rem_ref), 2.5e-3)
     for name, got, ref in (("dq", qg.grad, dq_ref), ("dk", kg.grad, dk_ref), ("dv", vg.grad, dv_ref)):
         assert got.dtype == torch.float16
-        within("float16 dense T=300", name, rel_l2(got.float().cpu(), ref), 2e-3)
+        within("float16 dense T=300", name, rel_l2(got.float().cpu(), ref), 6.25e-3)
     cu = torch.tensor([0, 100, 300], dtype=torch.int32)
     ov, rv = sb_attn_varlen(q[0].cuda(), k[0].cuda(), v[0].cuda(), cu, 200)
     assert ov.dtype == torch.float16

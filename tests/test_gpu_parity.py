@@ -1,6 +1,7 @@
 """GPU parity: the HIP operator (through the C ABI) against the CPU oracle on identical
 seeded inputs.  Tolerances are the ones the task states: forward o / rem max-abs
-2e-2 (bf16) and 1e-4 (fp32); gradients 5e-2 relative L2 (bf16; fp32 is held to 2e-3)."""
+2e-2 (bf16) and 1e-4 (fp32); gradients 5e-2 relative L2 (bf16; fp32 is held to 2e-3).
+float16 (tests/test_gpu_float16.py) is held to bf16's bounds divided by 8, the ratio of the unit roundoffs."""
 import math
 import os
 
@@ -12,8 +13,9 @@ from helpers import randn, rel_l2, max_abs, cu_from_lengths, lognormal_lengths
 
 pytestmark = pytest.mark.gpu
 
-FWD_TOL = {torch.bfloat16: 2e-2, torch.float32: 1e-4}
-GRAD_TOL = {torch.bfloat16: 5e-2, torch.float32: 2e-3}
+# float16: bf16's bounds times the ratio of the unit roundoffs (2^-11 against 2^-8)
+FWD_TOL = {torch.bfloat16: 2e-2, torch.float32: 1e-4, torch.float16: 2.5e-3}
+GRAD_TOL = {torch.bfloat16: 5e-2, torch.float32: 2e-3, torch.float16: 6.25e-3}
 
 
 def _ops():
