@@ -16,8 +16,8 @@
 //           kernels, chosen by grid size and head_dim: every wave owning 32 keys outright
 //           (d = 64, large grids), two waves sharing 32 keys (d = 128, large grids), a resident
 //           producer/consumer stream over 64-key items (d = 64, small grids), one workgroup
-//           per 64-key block (d = 128, small grids).  d = 256: every wave on its own 32 keys, in two
-//           launches that each take half of the columns of dK and dV.
+//           per 64-key block (d = 128, small grids).  d = 256: every wave on its own 32 keys, two
+//           workgroups per key block that each take half of the columns of dK and dV.
 //
 // Every element of the score matrix is therefore evaluated twice in the backward (once per
 // pass); in exchange nothing is reduced through memory.
@@ -1154,13 +1154,14 @@ __global__ __launch_bounds__((NP + 4) * 64, NP == 4 ? 2 : 3) void mfma_bwd_dkv_s
 // a 64-key block that touches the edge, the mid-block ones for the other half.  Weights and
 // logit gradients go as bf16 [query][32 a | 32 dz] rows into a tile private to the wave and
 // come back transposed as the A operands of  dV += A^T dO  and  dK += dZ^T Q.
-// kSplit / kPart: at head_dim 256 the [32 keys x 256] accumulators of dK and dV alone are 256 registers a lane, on top of
-// 128 for the K and V fragments.  There the kernel is launched kSplit = 2 times, launch kPart accumulating and storing
-// columns 128 * kPart .. 128 * kPart + 127 of dK and dV only; scores, weights and logit gradients are formed in both.
-template <int D, int kSplit = 1, int kPart = 0>
+// kSplit: at head_dim 256 the [32 keys x 256] accumulators of dK and dV alone are 256 registers a lane, on top of 128
+// for the K and V fragments.  There the grid has kSplit = 2 workgroups per (key block, head), blockIdx.y = 0, 1, and
+// workgroup `part` accumulates and stores columns 128 * part .. 128 * part + 127 of dK and dV only; scores, weights and
+// logit gradients are formed in both.
+template <int D, int kSplit = 1>
 __global__ __launch_bounds__(kThreads, D == 64 ? 2 : 1) void mfma_bwd_dkv_own_kernel(KParams p) {
     constexpr int kNB = D / 32 / kSplit;         // 32-wide column blocks of dK / dV accumulated here
-    constexpr int kB0 = kPart * kNB;             // the first of them
+    const int part = kSplit > 1 ? (int)blockIdx.y : 0;
     static_assert(32 * (D / kSplit) * 2 <= 64 * 64 * 2, "a wave stages its [32 keys x columns] outputs in its weight tile");
     constexpr int kQTile = 64 * D * 2;           // Q or dO tile of one step (64 queries)
     constexpr int kZTile = 64 * 64 * 2;          // per wave: [64 queries][32 a | 32 dz] bf16
@@ -1245,6 +1246,15 @@ __global__ __launch_bounds__(kThreads, D == 64 ? 2 : 1) void mfma_bwd_dkv_own_ke
     // runs in one copy per tile buffer, so that buffer and row offsets are compile-time numbers in the offset fields of
     // the fetches (with the tile address in a scalar register each fetch or pinned sum costs a vector add with a scalar
     // operand: 25 of them per step here).
+    if (kSplit > 1) {
+        // this workgroup's column blocks: kNB blocks are 4 * kNB sixteen-byte chunks, a multiple of 16, and the swizzle
+        // only touches chunk bits 0..3, so block b + part * kNB lies part * kNB * 64 bytes further along the same row
+        static_assert(kSplit == 1 || kNB % 4 == 0, "the shift must not meet the swizzled chunk bits");
+#pragma unroll
+        for (int a = 0; a < 2; ++a)
+#pragma unroll
+            for (int b = 0; b < kNB; ++b) lo.nat[a][b] += part * (kNB * 64);
+    }
     lo.rebase(lds);
     lz.rebase(ztile);
     constexpr TileAt zt{0};
@@ -1262,8 +1272,8 @@ __global__ __launch_bounds__(kThreads, D == 64 ? 2 : 1) void mfma_bwd_dkv_own_ke
             const h16x8 zf = fetch_nat_o<64>(zt, lz, 16 * kk, 1);
 #pragma unroll
             for (int db = 0; db < kNB; ++db) {
-                dvacc[db] = mfma(af, fetch_nat_o<D>(dot, lo, 16 * kk, kB0 + db), dvacc[db]);
-                dkacc[db] = mfma(zf, fetch_nat_o<D>(qt, lo, 16 * kk, kB0 + db), dkacc[db]);
+                dvacc[db] = mfma(af, fetch_nat_o<D>(dot, lo, 16 * kk, db), dvacc[db]);
+                dkacc[db] = mfma(zf, fetch_nat_o<D>(qt, lo, 16 * kk, db), dkacc[db]);
             }
         }
     };
@@ -1320,7 +1330,7 @@ __global__ __launch_bounds__(kThreads, D == 64 ? 2 : 1) void mfma_bwd_dkv_own_ke
                     // overwritten: this step's second tile comes later) and of the previous Q / dO tiles
                     auto red_a = [&](int seg) { return fetch_nat_o<64>(zt, lz, 32 + 16 * (seg >> 1), seg & 1); };
                     auto red_b = [&](int seg, int db) {
-                        return (seg & 1) ? fetch_nat_o<D>(pqtile, lo, 32 + 16 * (seg >> 1), kB0 + db) : fetch_nat_o<D>(pdotile, lo, 32 + 16 * (seg >> 1), kB0 + db);
+                        return (seg & 1) ? fetch_nat_o<D>(pqtile, lo, 32 + 16 * (seg >> 1), db) : fetch_nat_o<D>(pdotile, lo, 32 + 16 * (seg >> 1), db);
                     };
                     h16x8 na = red_a(0), nb[kNB];
 #pragma unroll
@@ -1349,7 +1359,7 @@ __global__ __launch_bounds__(kThreads, D == 64 ? 2 : 1) void mfma_bwd_dkv_own_ke
                     // whose exp/rcp overlap them.  Segment 2kk: dV += A^T dO, segment 2kk + 1: dK += dZ^T Q.
                     auto red_a = [&](int seg) { return fetch_nat_o<64>(zt, lz, 16 * (seg >> 1), seg & 1); };
                     auto red_b = [&](int seg, int db) {
-                        return (seg & 1) ? fetch_nat_o<D>(qtile, lo, 16 * (seg >> 1), kB0 + db) : fetch_nat_o<D>(dotile, lo, 16 * (seg >> 1), kB0 + db);
+                        return (seg & 1) ? fetch_nat_o<D>(qtile, lo, 16 * (seg >> 1), db) : fetch_nat_o<D>(dotile, lo, 16 * (seg >> 1), db);
                     };
                     h16x8 na = red_a(0), nb[kNB];
 #pragma unroll
@@ -1416,14 +1426,14 @@ __global__ __launch_bounds__(kThreads, D == 64 ? 2 : 1) void mfma_bwd_dkv_own_ke
     for (int which = 0; which < 2; ++which) {
         const TensorArg& out = which == 0 ? p.dk : p.dv;
         const int64_t ob = (int64_t)job.seq * out.sb + (int64_t)head * out.sh + (int64_t)job.tok0 * out.st;
-        constexpr int kCols = D / kSplit;          // columns kPart * kCols .. of the rows
+        constexpr int kCols = D / kSplit;          // columns part * kCols .. of the rows
 #pragma unroll
         for (int db = 0; db < kNB; ++db)
             stage_acc_tile<kCols>(ztile, 0, 32 * db, which == 0 ? dkacc[db] : dvacc[db], which == 0 ? p.scale : 1.0f, lane);
         for (int c = lane; c < 32 * kCols / 8; c += 64) {
             const int row = c / (kCols / 8), cc = c % (kCols / 8);
             if (kb0 + row < job.len)
-                *(u32x4*)(out.ptr + 2 * (ob + (int64_t)(kb0 + row) * out.st + kPart * kCols + cc * 8)) = *(const u32x4*)(ztile + row * (kCols * 2) + cc * 16);
+                *(u32x4*)(out.ptr + 2 * (ob + (int64_t)(kb0 + row) * out.st + part * kCols + cc * 8)) = *(const u32x4*)(ztile + row * (kCols * 2) + cc * 16);
         }
     }
 }
@@ -1760,12 +1770,12 @@ int sba_launch_mfma_bwd(const sba::KParams& kp_in, int phases, hipStream_t s) {
             else hipLaunchKernelGGL((mfma_bwd_dkv_stream_kernel<64, 4>), dim3(n_wg), dim3(8 * 64), 0, s, kp);
         }
     } else if (kp.head_dim == 256) {
-        // one wave per SIMD in both passes; every wave of the key-owner pass on its own 32 keys, in two launches that
-        // each accumulate one half of the columns of dK and dV - the other key-owner kernels do not fit the CU here
+        // one wave per SIMD in both passes; every wave of the key-owner pass on its own 32 keys, two workgroups per
+        // key block that each accumulate one half of the columns of dK and dV - the other key-owner kernels do not
+        // fit the CU here
         if (p1) hipLaunchKernelGGL((mfma_bwd_dq_kernel<256>), grid, dim3(kThreads), 0, s, kp);
         if (p2) {
-            hipLaunchKernelGGL((mfma_bwd_dkv_own_kernel<256, 2, 0>), grid, dim3(kThreads), 0, s, kp);
-            hipLaunchKernelGGL((mfma_bwd_dkv_own_kernel<256, 2, 1>), grid, dim3(kThreads), 0, s, kp);
+            hipLaunchKernelGGL((mfma_bwd_dkv_own_kernel<256, 2>), dim3(grid.x, 2), dim3(kThreads), 0, s, kp);
         }
     } else {
         if (p1) hipLaunchKernelGGL((mfma_bwd_dq_kernel<128>), grid, dim3(kThreads), 0, s, kp);
