@@ -1,6 +1,6 @@
 """Benchmark of the stick-breaking attention hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload cfg2|cfg3|cfg4]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload cfg2|cfg3|cfg4|cfg5|short|d256] [--dtype bf16|f16]
 
 A step is one forward + backward of the operator through its public autograd API on
 synthetic inputs already resident in HBM.  Prints ONE JSON line.
@@ -107,20 +107,30 @@ def _lognormal_lengths(total, seed, median=600.0, sigma=1.0, lo=16, hi=4096):
     return lens
 
 
-def make_workload(name, device):
+def make_workload(name, device, dtype_name="bf16"):
     """Returns (description, step_fn inputs, number of allowed pairs P, tokens, d)."""
     import torch
     g = torch.Generator().manual_seed(0)
+    dtype = {"bf16": torch.bfloat16, "f16": torch.float16}[dtype_name]
 
     def rn(shape, scale):
-        return (torch.randn(shape, generator=g) * scale).to(torch.bfloat16).to(device)
+        return (torch.randn(shape, generator=g) * scale).to(dtype).to(device)
+
+    if name == "d256":
+        # head_dim 256 (no configuration of BASELINE.json; the size the reference would run with BLOCK_D = 256)
+        B, H, T, D = 1, 8, 8192, 256
+        q, k, v = rn((B, H, T, D), 0.5), rn((B, H, T, D), 0.5), rn((B, H, T, D), 0.5)
+        do = rn((B, H, T, D), 1.0)
+        pairs = B * H * T * (T - 1) // 2
+        desc = {"workload": f"d256: dense causal fwd+bwd B=1 H=8 T=8192 d=256 {dtype_name}", "B": B, "H": H, "T": T, "d": D}
+        return desc, (q, k, v, do, None, None), pairs, B * T, D, H
 
     if name == "cfg2":
         B, H, T, D = 1, 16, 4096, 64
         q, k, v = rn((B, H, T, D), 0.5), rn((B, H, T, D), 0.5), rn((B, H, T, D), 0.5)
         do = rn((B, H, T, D), 1.0)
         pairs = B * H * T * (T - 1) // 2
-        desc = {"workload": "cfg2: dense causal fwd+bwd B=1 H=16 T=4096 d=64 bf16", "B": B, "H": H, "T": T, "d": D}
+        desc = {"workload": f"cfg2: dense causal fwd+bwd B=1 H=16 T=4096 d=64 {dtype_name}", "B": B, "H": H, "T": T, "d": D}
         return desc, (q, k, v, do, None, None), pairs, B * T, D, H
     if name == "cfg4":
         B, H, T, D = 1, 16, 16384, 128
@@ -130,11 +140,11 @@ def make_workload(name, device):
         for h in range(H):
             sel = torch.randperm(T, generator=g)[:n_sel].to(device)
             u = torch.randn(D, generator=g)
-            u = (3.0 * u / u.norm()).to(torch.bfloat16).to(device)
+            u = (3.0 * u / u.norm()).to(dtype).to(device)
             k[0, h, sel] += u
         do = rn((B, H, T, D), 1.0)
         pairs = B * H * T * (T - 1) // 2
-        desc = {"workload": "cfg4: dense causal fwd+bwd B=1 H=16 T=16384 d=128 bf16, 1% boosted keys",
+        desc = {"workload": f"cfg4: dense causal fwd+bwd B=1 H=16 T=16384 d=128 {dtype_name}, 1% boosted keys",
                 "B": B, "H": H, "T": T, "d": D}
         return desc, (q, k, v, do, None, None), pairs, B * T, D, H
     if name == "cfg3":
@@ -147,7 +157,7 @@ def make_workload(name, device):
         do = rn((H, N, D), 1.0)
         pairs = H * sum(L * (L - 1) // 2 for L in lens)
         cu_t = torch.tensor(cu, dtype=torch.int32, device=device)
-        desc = {"workload": "cfg3: packed varlen fwd+bwd H=16 d=64 bf16, 65536 tokens, lognormal docs",
+        desc = {"workload": f"cfg3: packed varlen fwd+bwd H=16 d=64 {dtype_name}, 65536 tokens, lognormal docs",
                 "H": H, "tokens": N, "d": D, "n_docs": len(lens), "max_len": max(lens)}
         return desc, (q, k, v, do, cu_t, max(lens)), pairs, N, D, H
     if name == "short":
@@ -166,7 +176,7 @@ def make_workload(name, device):
         do = rn((H, N, D), 1.0)
         pairs = H * sum(L * (L - 1) // 2 for L in lens)
         cu_t = torch.tensor(cu, dtype=torch.int32, device=device)
-        desc = {"workload": "short: packed varlen fwd+bwd H=16 d=64 bf16, 65536 tokens in documents of 16..128 tokens",
+        desc = {"workload": f"short: packed varlen fwd+bwd H=16 d=64 {dtype_name}, 65536 tokens in documents of 16..128 tokens",
                 "H": H, "tokens": N, "d": D, "n_docs": len(lens), "max_len": max(lens)}
         return desc, (q, k, v, do, cu_t, max(lens)), pairs, N, D, H
     raise SystemExit(f"unknown workload {name}")
@@ -326,7 +336,10 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--workload", default="cfg2", choices=["cfg2", "cfg3", "cfg4", "cfg5", "short", "copy"])
+    ap.add_argument("--workload", default="cfg2", choices=["cfg2", "cfg3", "cfg4", "cfg5", "short", "copy", "d256"])
+    ap.add_argument("--dtype", default="bf16", choices=["bf16", "f16"],
+                    help="element type of the operator workloads (f16: the same kernels compiled for float16; "
+                         "BASELINE.json's configurations are bf16, the default)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--carries", default="kept", choices=["kept", "default"],
                     help="kept: the forward keeps its carry tables whatever their size (the kernels as such); default: the "
@@ -356,7 +369,7 @@ def main():
         torch.cuda.synchronize()
         print(json.dumps({"workload": "copy", "bytes_read": 256 << 20, "bytes_written": 256 << 20}))
         return
-    desc, (q, k, v, do, cu, max_len), pairs, tokens, D, H = make_workload(args.workload, dev)
+    desc, (q, k, v, do, cu, max_len), pairs, tokens, D, H = make_workload(args.workload, dev, args.dtype)
     q.requires_grad_(True), k.requires_grad_(True), v.requires_grad_(True)
     from flame_amd import _lib
     if args.carries == "kept":
@@ -402,7 +415,7 @@ def main():
     out = {
         "metric": "sb_attn_fwd_bwd_tflops", "value": round(tflops, 2), "unit": "TFLOP/s",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms, 4),
-        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16",
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": args.dtype,
         "data": "synthetic", "config": desc,
         "pct_of_bf16_mfma_peak": round(100 * tflops / BF16_MFMA_PEAK_TFLOPS, 2),
         "tokens_per_s": round(tokens / (ms * 1e-3), 1),
@@ -447,7 +460,8 @@ def main():
                 total = sum(f[which] for f in every_kernel)
                 out["issue_floor"][f"step_pct_of_mfma_peak_at_{which}"] = round(
                     100 * f_fb / (total * 1e-3) / 1e12 / BF16_MFMA_PEAK_TFLOPS, 1)
-    if not args.no_cpu_baseline and args.workload != "short":     # (the CPU leg is defined for BASELINE's configurations)
+    # (the CPU leg is defined for BASELINE's configurations, which are bf16)
+    if not args.no_cpu_baseline and args.workload not in ("short", "d256") and args.dtype == "bf16":
         out["cpu_baseline"] = cpu_baseline(args.workload)
         o, rem = step()          # the timed tensors once more, for the check below
         out["parity_sample"] = parity_sample(args.workload, q, k, v, do, cu, o, rem)
