@@ -76,6 +76,8 @@ def load() -> C.CDLL:
         lib.sba_fwd.argtypes = [C.POINTER(SbaParams)]
         lib.sba_bwd.restype = C.c_int
         lib.sba_bwd.argtypes = [C.POINTER(SbaParams)]
+        lib.sba_attention_weights.restype = C.c_int
+        lib.sba_attention_weights.argtypes = [C.POINTER(SbaParams), C.c_void_p]
         lib.sba_bwd_static.restype = C.c_int
         lib.sba_bwd_static.argtypes = [C.POINTER(SbaParams)]
         lib.sba_bwd_gave_up.restype = C.c_int

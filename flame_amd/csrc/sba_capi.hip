@@ -290,6 +290,16 @@ int sba_fwd(const SbaParams* p) {
     return mfma ? sba_launch_mfma_fwd(kp, s) : sba_launch_generic_fwd(kp, p->dtype, s);
 }
 
+int sba_attention_weights(const SbaParams* p, float* weights) {
+    int rc = check_common(p);
+    if (rc) return rc;
+    if (!weights) return SBA_ERR_NULL;
+    if (p->dtype == SBA_DTYPE_F16) return SBA_ERR_DTYPE;      // vector-ALU kernel: bf16 and fp32 (float16 is exact in fp32)
+    KParams kp = make_kparams(p);
+    kp.weights = weights;
+    return sba_launch_generic_weights(kp, p->dtype, (hipStream_t)p->stream);
+}
+
 int sba_bwd(const SbaParams* p) {
     int rc = check_common(p);
     if (rc) return rc;

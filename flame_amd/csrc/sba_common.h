@@ -41,6 +41,7 @@ struct KParams {
     TensorArg q_scaled;            // bf16 head_dim 64 backward: q times scale2, rounded to bf16, written by the dQ pass for
                                    //   the key-owner stream kernel (ptr NULL: not wanted)
     float* dkv32;                  // generic path: fp32 dk|dv accumulators
+    float* weights;                // sba_attention_weights(): the attention weights, fp32 (debug output)
     int* gave_up;                  // backward error word (set if a kernel abandoned a bounded internal wait)
     int64_t tab_head_stride;       // floats per head in each carry table
     int64_t tab_tokens;            // generic path: tokens per head in the fp32 accumulators (n_seq*T dense, sumT packed)
@@ -184,6 +185,7 @@ inline double sba_tail_ratio(const sba::KParams& kp, unsigned grid) {
 int sba_generic_padded_dim(int D);
 int sba_launch_generic_fwd(const sba::KParams& kp, int dtype, hipStream_t s);
 int sba_launch_generic_bwd(const sba::KParams& kp, int dtype, hipStream_t s);
+int sba_launch_generic_weights(const sba::KParams& kp, int dtype, hipStream_t s);
 int sba_launch_mfma_fwd(const sba::KParams& kp, hipStream_t s);
 int sba_launch_mfma_bwd(const sba::KParams& kp, int phases, hipStream_t s);
 int sba_launch_mfma_f16_fwd(const sba::KParams& kp, hipStream_t s);       // the same kernels compiled for float16 elements

@@ -84,6 +84,52 @@ __global__ __launch_bounds__(kGenThreads) void generic_fwd_kernel(KParams p) {
     }
 }
 
+// The attention weights A_ij themselves, the reference's `return_attention` debug output (sb_attn/sb_fwd.py:141-172,
+// sb_varlen/sb_varlen_fwd.py:195-201 and :409-446): fp32, dense [B, H, T, T], packed [H, sum T, sum T] (a document's
+// block on the diagonal); entries of pairs that are not allowed are left as they are (the caller zero-fills, as the
+// reference does).  The forward sweep of generic_fwd_kernel without V.
+template <typename T, int DP>
+__global__ __launch_bounds__(kGenThreads) void generic_weights_kernel(KParams p) {
+    __shared__ float Ks[kGenChunk * DP];
+    const int head = blockIdx.x % p.n_heads;
+    const Job job = decode_job(p, blockIdx.x / p.n_heads);
+    const int D = p.head_dim;
+    const int i = job.rb * kRowBlock + threadIdx.x;
+    const bool active = i < job.len;
+    const int strict = p.attend_current ? 0 : 1;
+    const int64_t qbase = (int64_t)job.seq * p.q.sb + (int64_t)head * p.q.sh + (int64_t)job.tok0 * p.q.st;
+    const int64_t kbase = (int64_t)job.seq * p.k.sb + (int64_t)head * p.k.sh + (int64_t)job.tok0 * p.k.st;
+    // row (token i) of this head's [tokens x tokens] matrix, first column of the sequence
+    const int64_t side = p.cu_seqlens ? (int64_t)p.total_tokens : (int64_t)p.seq_len;
+    const int64_t plane = p.cu_seqlens ? (int64_t)head : (int64_t)job.seq * p.n_heads + head;
+    float* const wrow = p.weights + (plane * side + job.tok0 + i) * side + job.tok0;
+
+    float q[DP];
+#pragma unroll
+    for (int d = 0; d < DP; ++d)
+        q[d] = (active && d < D) ? Elem<T>::load(p.q.ptr, qbase + (int64_t)i * p.q.st + d) * p.scale : 0.f;
+    float R = 1.f;
+    const int imax = min(job.rb * kRowBlock + kRowBlock - 1, job.len - 1);
+    const int kmax = imax - strict;
+    for (int c = (kmax >= 0 ? kmax / kGenChunk : -1); c >= 0; --c) {
+        __syncthreads();
+        load_rows_to_lds<T, DP>(Ks, p.k, kbase, c * kGenChunk, job.len, D);
+        __syncthreads();
+        for (int jj = kGenChunk - 1; jj >= 0; --jj) {
+            const int j = c * kGenChunk + jj;
+            float z = 0.f;
+#pragma unroll
+            for (int d = 0; d < DP; ++d) z = __builtin_fmaf(q[d], Ks[jj * DP + d], z);
+            if (active && (j + strict <= i)) {
+                const float e = expf(fminf(z, kMaxLogitNat));
+                const float u = 1.0f / (1.0f + e);
+                wrow[j] = e * u * R;
+                R *= u;
+            }
+        }
+    }
+}
+
 // fp32 accumulators for dk and dv: [2][tab_tokens][H][DP] -> index helper
 __device__ inline int64_t acc_index(const KParams& p, int which, int64_t tok, int head, int DP) {
     return (((int64_t)which * p.tab_tokens + tok) * p.n_heads + head) * DP;
@@ -243,6 +289,21 @@ int sba_launch_generic_fwd(const sba::KParams& kp, int dtype, hipStream_t s) {
     if (DP == 64) return launch_fwd<uint16_t, 64>(kp, s);
     if (DP == 128) return launch_fwd<uint16_t, 128>(kp, s);
     return launch_fwd<uint16_t, 256>(kp, s);
+}
+
+template <typename T> static int launch_weights(const sba::KParams& kp, int DP, hipStream_t s) {
+    using namespace sba;
+    dim3 grid((unsigned)kp.n_jobs * kp.n_heads);
+    if (DP == 32) hipLaunchKernelGGL((generic_weights_kernel<T, 32>), grid, dim3(kGenThreads), 0, s, kp);
+    else if (DP == 64) hipLaunchKernelGGL((generic_weights_kernel<T, 64>), grid, dim3(kGenThreads), 0, s, kp);
+    else if (DP == 128) hipLaunchKernelGGL((generic_weights_kernel<T, 128>), grid, dim3(kGenThreads), 0, s, kp);
+    else hipLaunchKernelGGL((generic_weights_kernel<T, 256>), grid, dim3(kGenThreads), 0, s, kp);
+    return hipGetLastError() == hipSuccess ? SBA_OK : SBA_ERR_LAUNCH;
+}
+
+int sba_launch_generic_weights(const sba::KParams& kp, int dtype, hipStream_t s) {
+    const int DP = sba_generic_padded_dim(kp.head_dim);
+    return dtype == SBA_DTYPE_F32 ? launch_weights<float>(kp, DP, s) : launch_weights<uint16_t>(kp, DP, s);
 }
 
 int sba_launch_generic_bwd(const sba::KParams& kp, int dtype, hipStream_t s) {

@@ -84,7 +84,31 @@ def _compileable_backward(do: torch.Tensor, dr: Optional[torch.Tensor], q: torch
     profiling.launch_bwd(lib, p)
 
 
-def _fwd(q, k, v, logit_scale, attend_current=False, no_grad=False):
+def attention_weights(q, k, inv_temp=None, attend_current=False):
+    """The attention weights A_ij as float32 [B, H, T, T] (zero where j may not be attended): what the reference's
+    forward returns as `W` under `return_attention=True` (sb_fwd.py:141-172).  For inspection and tests: a
+    vector-ALU kernel, T x T floats per head."""
+    if not q.is_cuda:
+        raise RuntimeError("stick-breaking attention runs on the GPU only (HIP kernels); there is no CPU path")
+    if q.shape != k.shape or q.dim() != 4 or q.dtype != k.dtype:
+        raise ValueError("q, k must both be [B, H, T, D] of one dtype")
+    _lib.check_supported(q)
+    if inv_temp is None:
+        inv_temp = 1 / math.sqrt(q.size(-1))
+    if q.dtype == torch.float16:          # exact in float32; the kernel takes bf16 and float32
+        q, k = q.float(), k.float()
+    B, H, T, _ = q.shape
+    W = torch.zeros((B, H, T, T), dtype=torch.float32, device=q.device)
+    if W.numel():
+        q, k = _lib.usable(q.detach()), _lib.usable(k.detach())
+        p = _params(q, k, k, inv_temp, attend_current)
+        _lib.check(_lib.load().sba_attention_weights(C.byref(p), W.data_ptr()), "sba_attention_weights")
+    return W
+
+
+def _fwd(q, k, v, logit_scale, attend_current=False, no_grad=False, return_attention=False):
+    if return_attention:                 # the reference's debug output rides along as a fourth result
+        return (*_fwd(q, k, v, logit_scale, attend_current, no_grad), attention_weights(q, k, logit_scale, attend_current))
     o = torch.empty_like(q)              # same strides as q (sb_fwd.py:144 does the same)
     rem = torch.empty(q.shape[:-1], dtype=q.dtype, device=q.device)
     # above the workspace budget nothing is kept and the backward recomputes the carries (_lib.recompute_carries)

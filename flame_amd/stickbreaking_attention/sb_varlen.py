@@ -146,7 +146,34 @@ def _compileable_backward(do: torch.Tensor, dr: Optional[torch.Tensor], q: torch
     profiling.launch_bwd(lib, p)
 
 
-def varlen_fwd(q, k, v, cu_seqlens, max_seqlens, logit_scale, attend_current=False, no_grad=False):
+def attention_weights_varlen(q, k, cu_seqlens, max_seqlens, inv_temp=None, attend_current=False):
+    """The attention weights of a packed batch as float32 [H, sum T, sum T], every document's block on the diagonal,
+    zero elsewhere: what the reference's `varlen_fwd` returns as `W` under `return_attention=True`
+    (sb_varlen_fwd.py:409-446).  For inspection and tests: a vector-ALU kernel, (sum T)^2 floats per head."""
+    if not q.is_cuda:
+        raise RuntimeError("stick-breaking attention runs on the GPU only (HIP kernels); there is no CPU path")
+    if q.shape != k.shape or q.dim() != 3 or q.dtype != k.dtype:
+        raise ValueError("q, k must both be [H, sum T, D] of one dtype")
+    _lib.check_supported(q)
+    if inv_temp is None:
+        inv_temp = 1 / math.sqrt(q.size(-1))
+    if q.dtype == torch.float16:          # exact in float32; the kernel takes bf16 and float32
+        q, k = q.float(), k.float()
+    H, N, _ = q.shape
+    W = torch.zeros((H, N, N), dtype=torch.float32, device=q.device)
+    if W.numel():
+        q, k = _lib.usable(q.detach()), _lib.usable(k.detach())
+        p = _params(q, k, k, cu_seqlens.numel() - 1, max_seqlens, inv_temp, attend_current)
+        if _bind_schedule(p, q, cu_seqlens, max_seqlens) != 0:
+            _lib.check(_lib.load().sba_attention_weights(C.byref(p), W.data_ptr()), "sba_attention_weights")
+    return W
+
+
+def varlen_fwd(q, k, v, cu_seqlens, max_seqlens, logit_scale, attend_current=False, no_grad=False,
+               return_attention=False):
+    if return_attention:                 # the reference's debug output rides along as a fourth result
+        return (*varlen_fwd(q, k, v, cu_seqlens, max_seqlens, logit_scale, attend_current, no_grad),
+                attention_weights_varlen(q, k, cu_seqlens, max_seqlens, logit_scale, attend_current))
     o = torch.empty_like(q)
     rem = torch.empty(q.shape[:-1], dtype=q.dtype, device=q.device)
     # above the workspace budget nothing is kept and the backward recomputes the carries (_lib.recompute_carries)

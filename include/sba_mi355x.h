@@ -185,6 +185,18 @@ int sba_fwd(const SbaParams* p);
 int sba_bwd(const SbaParams* p);
 
 /*
+ * The attention weights A_ij themselves, in fp32: the reference forward's `return_attention` debug output
+ * (sb_attn/sb_fwd.py:141-172 `W`, sb_varlen/sb_varlen_fwd.py:195-201 and :409-446).  Reads q, k, scale,
+ * attend_current and the layout fields of *p (dtype bf16 or fp32, any head_dim; o, rem and the workspace are not
+ * touched) and writes weights[b][h][i][j] (dense, [n_seq, n_heads, seq_len, seq_len] contiguous) or
+ * weights[h][i][j] (packed, [n_heads, total_tokens, total_tokens] contiguous, i and j token positions in the
+ * pack) for every allowed pair; all other entries are left as they are (zero-fill first, as the reference does).
+ * A vector-ALU kernel: for inspection and tests, not for speed; its logits are the fp32 products of the inputs,
+ * where the 16-bit matrix-core kernels round q times the logit scale to 16 bits first.
+ */
+int sba_attention_weights(const SbaParams* p, float* weights);
+
+/*
  * Error word of the last backward that ran on this problem's scratch: *gave_up = 1 if one of its
  * kernels abandoned a bounded internal wait (its gradients are invalid), else 0.  `p` is the
  * SbaParams of that backward (sizes, workspace, bwd_scratch, stream); pass static_scratch_used = 1
