@@ -90,7 +90,7 @@ def load() -> C.CDLL:
 
 EXPORTED_SYMBOLS = ("sba_abi_version", "sba_error_string", "sba_workspace_bytes", "sba_bwd_scratch_bytes",
                     "sba_build_schedule", "sba_row_block", "sba_table_columns", "sba_fwd", "sba_bwd",
-                    "sba_bwd_static", "sba_bwd_gave_up")
+                    "sba_bwd_static", "sba_bwd_gave_up", "sba_attention_weights")
 
 STATIC_SCRATCH_BYTES = 64 << 20     # SBA_STATIC_SCRATCH_BYTES: what sba_bwd_static() holds per GPU
 
