@@ -89,7 +89,7 @@ def test_static_backward_matches_sba_bwd_on_two_calls_in_a_row():
 
 
 def test_static_backward_other_paths():
-    print("static bwd: d128, recompute mode, packed, fp32", flush=True)
+    print("static bwd: d128, recompute mode, packed, fp32, d256, float16", flush=True)
     a, b = _run_both((2, 2, 520, 128), torch.bfloat16, seed=20)
     _same(a, b, exact=True)
     a, b = _run_both((1, 2, 777, 64), torch.bfloat16, seed=30, keep_table=False)   # no table kept: the backward recomputes it
@@ -99,6 +99,10 @@ def test_static_backward_other_paths():
     a, b = _run_both((1, 2, 200, 32), torch.float32, seed=50)
     _same(a, b, exact=False)
     a, b = _run_both((1, 2, 90, 64), torch.bfloat16, seed=60)
+    _same(a, b, exact=True)
+    a, b = _run_both((1, 2, 300, 256), torch.bfloat16, seed=70)         # head_dim 256
+    _same(a, b, exact=True)
+    a, b = _run_both((2, 2, 520, 64), torch.float16, seed=80)           # the float16 build of the kernels
     _same(a, b, exact=True)
 
 
