@@ -1,5 +1,6 @@
 """Writes the golden vectors of this folder (``sb_*.npz``).  Run: python tests/golden/make_vectors.py
-(``python tests/golden/make_vectors.py overflow`` writes only ``sb_packed_overflow.npz``)
+(``python tests/golden/make_vectors.py overflow`` writes only ``sb_packed_overflow.npz``,
+``python tests/golden/make_vectors.py d256`` only ``sbdir_dense_d256.npz``)
 
 The reference ships no fixtures for stick-breaking attention, so these come from the
 mathematics alone, evaluated with 50-digit arithmetic (mpmath) and sharing no code with the
@@ -198,6 +199,10 @@ if __name__ == "__main__":
     import sys
     if sys.argv[1:] == ["overflow"]:       # only the case added last
         run_overflow_case("sb_packed_overflow")
+        sys.exit(0)
+    if sys.argv[1:] == ["d256"]:           # head_dim 256, added later: a generator of its own leaves the other files as they are
+        run_directional_case("sbdir_dense_d256", np.random.default_rng(20250311), lens=[150], D=256, scale=1 / 16.0,
+                             attend_current=False, in_scale=1.0, packed=False)
         sys.exit(0)
     rng = np.random.default_rng(20240607)
     run_case("sb_dense_strict", rng, H=2, lens=[9], D=4, scale=0.7, attend_current=False, in_scale=1.0, packed=False)

@@ -17,6 +17,11 @@ GOLDEN = sorted(glob.glob(os.path.join(os.path.dirname(__file__), "golden", "sb_
 OUTPUTS = ("o", "rem", "dq", "dk", "dv")
 
 
+# o / rem max-abs, gradients relative L2; float16: bf16's bounds times the ratio of the unit roundoffs (1/8)
+_TOL = {torch.bfloat16: (2e-2, 5e-2), torch.float32: (1e-4, 2e-3), torch.float16: (2.5e-3, 6.25e-3)}
+_NAME = {torch.bfloat16: "bf16", torch.float32: "fp32", torch.float16: "f16"}
+
+
 def _load(path):
     z = np.load(path, allow_pickle=False)
     t = {n: torch.from_numpy(z[n]) for n in ("q", "k", "v", "do", "drem") + OUTPUTS}
@@ -61,13 +66,13 @@ def test_closed_form_gradients_reproduce_golden_vectors(path):
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["fp32", "bf16"])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16], ids=["fp32", "bf16", "f16"])
 @pytest.mark.parametrize("path", GOLDEN, ids=os.path.basename)
 def test_hip_operator_reproduces_golden_vectors(path, dtype):
     from flame_amd import sb_attn, sb_attn_varlen
     t, cu, scale, ac = _load(path)
     print(f"golden {os.path.basename(path)} {dtype}", flush=True)
-    fwd_tol, grad_tol = (2e-2, 5e-2) if dtype == torch.bfloat16 else (1e-4, 2e-3)   # inputs are bf16-exact
+    fwd_tol, grad_tol = _TOL[dtype]   # inputs are bf16-exact (and with that float16-exact, down to values of 2^-15)
     q, k, v = (t[n].to(dtype).cuda().requires_grad_(True) for n in ("q", "k", "v"))
     if cu is None:
         o, rem = sb_attn(q, k, v, scale, attend_current=ac)
@@ -76,7 +81,7 @@ def test_hip_operator_reproduces_golden_vectors(path, dtype):
         o, rem = sb_attn_varlen(q, k, v, cu.cuda(), max(lens), scale, attend_current=ac)
     loss = (o.float() * t["do"].float().cuda()).sum() + (rem.float() * t["drem"].float().cuda()).sum()
     loss.backward()
-    label = f"golden {os.path.basename(path)} {'bf16' if dtype == torch.bfloat16 else 'fp32'}"
+    label = f"golden {os.path.basename(path)} {_NAME[dtype]}"
     within(label, "o", max_abs(o.float().cpu(), t["o"]), fwd_tol)
     within(label, "rem", max_abs(rem.float().cpu(), t["rem"]), fwd_tol)
     for name, g in (("dq", q.grad), ("dk", k.grad), ("dv", v.grad)):
@@ -101,7 +106,7 @@ def _slopes(grads, directions):
 
 
 def test_directional_fixtures_present():
-    assert len(DIRECTIONAL) == 3
+    assert len(DIRECTIONAL) == 4
 
 
 @pytest.mark.parametrize("path", DIRECTIONAL, ids=os.path.basename)
@@ -116,14 +121,14 @@ def test_oracle_reproduces_directional_vectors(path):
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["fp32", "bf16"])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16], ids=["fp32", "bf16", "f16"])
 @pytest.mark.parametrize("path", DIRECTIONAL, ids=os.path.basename)
 def test_hip_operator_reproduces_directional_vectors(path, dtype):
-    # D = 64 / 128: the matrix-core kernels in both dtypes (bf16 and fp32 MFMA)
+    # D = 64 / 128 / 256: the matrix-core kernels (bf16, float16 and, up to 128, fp32 MFMA; fp32 at 256: generic)
     from flame_amd import sb_attn, sb_attn_varlen
     t, cu, scale, ac = _load_directional(path)
     print(f"golden {os.path.basename(path)} {dtype}", flush=True)
-    fwd_tol, grad_tol = (2e-2, 5e-2) if dtype == torch.bfloat16 else (1e-4, 2e-3)
+    fwd_tol, grad_tol = _TOL[dtype]
     q, k, v = (t[n].to(dtype).cuda().requires_grad_(True) for n in ("q", "k", "v"))
     if cu is None:
         o, rem = sb_attn(q, k, v, scale, attend_current=ac)
@@ -132,7 +137,7 @@ def test_hip_operator_reproduces_directional_vectors(path, dtype):
         o, rem = sb_attn_varlen(q, k, v, cu.cuda(), max(lens), scale, attend_current=ac)
     loss = (o.float() * t["do"].float().cuda()).sum() + (rem.float() * t["drem"].float().cuda()).sum()
     loss.backward()
-    label = f"golden {os.path.basename(path)} {'bf16' if dtype == torch.bfloat16 else 'fp32'}"
+    label = f"golden {os.path.basename(path)} {_NAME[dtype]}"
     within(label, "o", max_abs(o.detach().float().cpu(), t["o"]), fwd_tol)
     within(label, "rem", max_abs(rem.detach().float().cpu(), t["rem"]), fwd_tol)
     grads = [g.detach().float().cpu() for g in (q.grad, k.grad, v.grad)]
