@@ -54,6 +54,13 @@ def test_argument_checks_without_gpu(lib):
     p.head_dim = 96
     assert lib.sba_fwd(C.byref(p)) == -3
     p.dtype, p.head_dim = _lib.SBA_DTYPE_BF16, 64
+    assert lib.sba_attention_weights(C.byref(p), None) == -1      # NULL q/k/v come first
+    p.q.ptr = p.k.ptr = p.v.ptr = 256                             # never dereferenced: the checks below come before any launch
+    assert lib.sba_attention_weights(C.byref(p), None) == -1      # no output
+    p.dtype = _lib.SBA_DTYPE_F16
+    assert lib.sba_attention_weights(C.byref(p), 256) == -3       # bf16 and fp32 only
+    p.dtype = _lib.SBA_DTYPE_BF16
+    p.q.ptr = p.k.ptr = p.v.ptr = None
     assert lib.sba_fwd(None) == -1
     assert lib.sba_row_block() == 128
 
