@@ -1731,7 +1731,11 @@ int sba_launch_mfma_bwd(const sba::KParams& kp_in, int phases, hipStream_t s) {
     // 512 workgroups B=8, T=512 takes 27.3 us against the stream's 33.0, B=4, T=1024 44.0 against 45.3.
     const unsigned cus = (unsigned)sba_cu_count();
     const bool short_sweeps = kp.seq_len <= 8 * kRowBlock;
-    const bool own = own_keys_kernel(kp.head_dim == 64 ? grid.x >= 3u * cus || (short_sweeps && grid.x >= 2u * cus) : true);
+    // One dense sequence per head from 4096 tokens on keeps the stream up to four and a half workgroups per CU (B=1, H=16:
+    // T=7168 297 against 309 us, T=8192 363 against 391, T=9216 445 against 460; from T=10240 on, and for batches of
+    // shorter sequences and packs on the same grids, the own-keys kernel is ahead by 2-5 %).
+    const bool long_dense = !kp.cu_seqlens && kp.seq_len >= 4096 && 2u * grid.x <= 9u * cus;
+    const bool own = own_keys_kernel(kp.head_dim == 64 ? (grid.x >= 3u * cus && !long_dense) || (short_sweeps && grid.x >= 2u * cus) : true);
     const char* which = getenv("SBA_DKV_KERNEL");
     const bool plain = which && !strcmp(which, "plain");
     // the stream with eight half-block producers (12 waves): behind the one with four full-block producers
