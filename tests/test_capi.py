@@ -267,3 +267,25 @@ def test_python_workspace_bound_covers_the_library(lib):
     for lens in ([1, 130, 500, 64, 205], [4096] * 3 + [16] * 40, [127, 128, 129], [1]):
         cu = torch.tensor([0] + list(torch.tensor(lens).cumsum(0)), dtype=torch.int32)
         assert _lib.packed_columns_bound(sum(lens), len(lens), max(lens)) >= _lib.table_columns(cu)
+
+
+def test_head_dim_routing_of_the_python_layer(monkeypatch):
+    # which head dim a problem runs with: matrix-core sizes as they are, everything else zero-padded up to the next one
+    # (16-bit types up to 256, float32 up to 128); the generic kernels keep every head dim
+    monkeypatch.delenv("SBA_FORCE_GENERIC", raising=False)
+    monkeypatch.delenv("SBA_FORCE_GENERIC_BWD", raising=False)
+    expect = {torch.bfloat16: {8: 64, 64: 64, 80: 128, 128: 128, 129: 256, 200: 256, 256: 256},
+              torch.float16: {8: 64, 64: 64, 80: 128, 128: 128, 129: 256, 200: 256, 256: 256},
+              torch.float32: {8: 64, 64: 64, 80: 128, 128: 128, 129: 129, 200: 200, 256: 256}}
+    for dtype, table in expect.items():
+        for D, Dp in table.items():
+            assert _lib.matrix_core_head_dim(torch.empty(1, 1, 1, D, dtype=dtype)) == Dp, (dtype, D)
+    assert _lib.dtype_code(torch.float16) == _lib.SBA_DTYPE_F16 == 2
+    assert not _lib.float16_needs_float32_route()
+    with pytest.raises(ValueError, match="head_dim"):
+        _lib.check_supported(torch.empty(1, 1, 1, 257, dtype=torch.bfloat16))
+    with pytest.raises(TypeError, match="float16"):
+        _lib.check_supported(torch.empty(1, 1, 1, 64, dtype=torch.float64))
+    monkeypatch.setenv("SBA_FORCE_GENERIC", "1")
+    assert _lib.matrix_core_head_dim(torch.empty(1, 1, 1, 80, dtype=torch.bfloat16)) == 80
+    assert _lib.float16_needs_float32_route()
