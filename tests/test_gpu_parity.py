@@ -342,13 +342,15 @@ def test_varlen_rejects_too_small_max_seqlens():
         sb_attn_varlen(q, q, q, torch.tensor([0, 100, 300], dtype=torch.int32).cuda(), 150)
 
 
-def test_torch_compile_fullgraph_matches_eager():
+@pytest.mark.parametrize("D,dtype", [(64, torch.bfloat16), (96, torch.float16), (256, torch.bfloat16)])
+def test_torch_compile_fullgraph_matches_eager(D, dtype):
     # the launchers are registered as stickbreaking_attention::{attn_fwd,attn_bwd,varlen_fwd,
-    # varlen_bwd} custom ops (as the reference does, utils.py:20-39), so the op traces
+    # varlen_bwd} custom ops (as the reference does, utils.py:20-39), so the op traces - also through the
+    # zero-padding of a head dim and in float16
     sb_attn, sb_attn_varlen = _ops()
     assert hasattr(torch.ops.stickbreaking_attention, "attn_fwd")
     assert hasattr(torch.ops.stickbreaking_attention, "varlen_bwd")
-    q, k, v, do = (randn((1, 2, 200, 64), 100 + i, 0.5, torch.bfloat16).cuda() for i in range(4))
+    q, k, v, do = (randn((1, 2, 200, D), 100 + i, 0.5, dtype).cuda() for i in range(4))
 
     def f(q, k, v):
         o, rem = sb_attn(q, k, v)
