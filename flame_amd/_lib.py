@@ -113,12 +113,6 @@ def dtype_code(dt: torch.dtype) -> int:
     raise TypeError(f"stick-breaking attention supports float32, bfloat16 and float16, got {dt}")
 
 
-def float16_needs_float32_route() -> bool:
-    """float16 has matrix-core kernels only; with the generic kernels forced (the test-suite's cross-checks) it
-    runs as float32 - exact conversion in, results rounded to float16."""
-    return os.environ.get("SBA_FORCE_GENERIC") == "1" or os.environ.get("SBA_FORCE_GENERIC_BWD") == "1"
-
-
 def check_supported(q: torch.Tensor) -> None:
     """Say up front what the kernels do not cover instead of failing inside the library."""
     if q.dtype not in (torch.float32, torch.bfloat16, torch.float16):

@@ -26,7 +26,7 @@ bool force_generic() {
 bool is_16bit(const SbaParams* p) { return p->dtype == SBA_DTYPE_BF16 || p->dtype == SBA_DTYPE_F16; }
 
 // The matrix-core kernels cover bf16, float16 and fp32 with head_dim 64 or 128 and the 16-bit types with head_dim
-// 256; everything else takes the generic vector-ALU kernels (which exist for bf16 and fp32).
+// 256; everything else takes the generic vector-ALU kernels.
 bool use_mfma(const SbaParams* p) {
     if (force_generic()) return false;
     if (is_16bit(p) && p->head_dim == 256) return true;
@@ -95,8 +95,6 @@ int check_common(const SbaParams* p) {
     if (!p) return SBA_ERR_NULL;
     if (p->struct_size != sizeof(SbaParams)) return SBA_ERR_ABI;
     if (p->dtype != SBA_DTYPE_F32 && !is_16bit(p)) return SBA_ERR_DTYPE;
-    // float16 has matrix-core kernels only: head_dim 64, 128 or 256 (callers zero-pad other head dims)
-    if (p->dtype == SBA_DTYPE_F16 && !use_mfma_bwd(p)) return SBA_ERR_DTYPE;
     if (p->n_seq <= 0 || p->n_heads <= 0 || p->seq_len <= 0 || p->total_tokens <= 0) return SBA_ERR_SHAPE;
     if (p->head_dim <= 0 || p->head_dim > sba::kMaxHeadDim) return SBA_ERR_SHAPE;
     if (!p->q.ptr || !p->k.ptr || !p->v.ptr) return SBA_ERR_NULL;
@@ -196,7 +194,7 @@ const char* sba_error_string(int code) {
         case SBA_OK: return "ok";
         case SBA_ERR_NULL: return "a required pointer is NULL";
         case SBA_ERR_SHAPE: return "bad shape: sizes must be positive, head_dim <= 256, dense total_tokens == seq_len; at head_dim 64 / 128 (the matrix-core kernels, bf16 and fp32) and 256 (bf16) tensors need 16-byte aligned pointers, outer strides that are multiples of 16 bytes and a token stride below 2^23 elements";
-        case SBA_ERR_DTYPE: return "unsupported dtype: float32, bfloat16, or float16 at head_dim 64 / 128 / 256 (float16 has matrix-core kernels only: not under SBA_FORCE_GENERIC=1 / SBA_FORCE_GENERIC_BWD=1)";
+        case SBA_ERR_DTYPE: return "unsupported dtype (SBA_DTYPE_F32, SBA_DTYPE_BF16 or SBA_DTYPE_F16)";
         case SBA_ERR_WORKSPACE: return "workspace / bwd_scratch missing or smaller than sba_workspace_bytes() / sba_bwd_scratch_bytes()";
         case SBA_ERR_SCHEDULE: return "packed layout needs a row-block schedule from sba_build_schedule()";
         case SBA_ERR_LAUNCH: return "kernel launch failed";
@@ -294,7 +292,6 @@ int sba_attention_weights(const SbaParams* p, float* weights) {
     int rc = check_common(p);
     if (rc) return rc;
     if (!weights) return SBA_ERR_NULL;
-    if (p->dtype == SBA_DTYPE_F16) return SBA_ERR_DTYPE;      // vector-ALU kernel: bf16 and fp32 (float16 is exact in fp32)
     KParams kp = make_kparams(p);
     kp.weights = weights;
     return sba_launch_generic_weights(kp, p->dtype, (hipStream_t)p->stream);

@@ -133,6 +133,10 @@ template <> struct Elem<float> {
     __device__ static float load(const char* p, int64_t i) { return ((const float*)p)[i]; }
     __device__ static void store(char* p, int64_t i, float v) { ((float*)p)[i] = v; }
 };
+template <> struct Elem<_Float16> {
+    __device__ static float load(const char* p, int64_t i) { return (float)((const _Float16*)p)[i]; }
+    __device__ static void store(char* p, int64_t i, float v) { ((_Float16*)p)[i] = (_Float16)v; }
+};
 template <> struct Elem<uint16_t> {   // bf16 bits
     __device__ static float load(const char* p, int64_t i) { return bf16_to_f32(((const uint16_t*)p)[i]); }
     __device__ static void store(char* p, int64_t i, float v) { ((uint16_t*)p)[i] = f32_to_bf16(v); }

@@ -1,4 +1,4 @@
-// Generic stick-breaking attention kernels: any head_dim <= 256, fp32 or bf16 storage,
+// Generic stick-breaking attention kernels: any head_dim <= 256, fp32, bf16 or float16 storage,
 // fp32 arithmetic on the vector ALUs (no matrix cores).  This is the fp32 path of the
 // operator (the 1e-4 tolerance class) and the path for head dims the MFMA kernels do
 // not cover.  One thread owns one query row; a workgroup owns a row-block of 128 queries
@@ -285,6 +285,12 @@ int sba_launch_generic_fwd(const sba::KParams& kp, int dtype, hipStream_t s) {
         if (DP == 128) return launch_fwd<float, 128>(kp, s);
         return launch_fwd<float, 256>(kp, s);
     }
+    if (dtype == SBA_DTYPE_F16) {
+        if (DP == 32) return launch_fwd<_Float16, 32>(kp, s);
+        if (DP == 64) return launch_fwd<_Float16, 64>(kp, s);
+        if (DP == 128) return launch_fwd<_Float16, 128>(kp, s);
+        return launch_fwd<_Float16, 256>(kp, s);
+    }
     if (DP == 32) return launch_fwd<uint16_t, 32>(kp, s);
     if (DP == 64) return launch_fwd<uint16_t, 64>(kp, s);
     if (DP == 128) return launch_fwd<uint16_t, 128>(kp, s);
@@ -303,6 +309,7 @@ template <typename T> static int launch_weights(const sba::KParams& kp, int DP, 
 
 int sba_launch_generic_weights(const sba::KParams& kp, int dtype, hipStream_t s) {
     const int DP = sba_generic_padded_dim(kp.head_dim);
+    if (dtype == SBA_DTYPE_F16) return launch_weights<_Float16>(kp, DP, s);
     return dtype == SBA_DTYPE_F32 ? launch_weights<float>(kp, DP, s) : launch_weights<uint16_t>(kp, DP, s);
 }
 
@@ -314,6 +321,12 @@ int sba_launch_generic_bwd(const sba::KParams& kp, int dtype, hipStream_t s) {
         if (DP == 64) return launch_bwd<float, 64>(kp, s);
         if (DP == 128) return launch_bwd<float, 128>(kp, s);
         return launch_bwd<float, 256>(kp, s);
+    }
+    if (dtype == SBA_DTYPE_F16) {
+        if (DP == 32) return launch_bwd<_Float16, 32>(kp, s);
+        if (DP == 64) return launch_bwd<_Float16, 64>(kp, s);
+        if (DP == 128) return launch_bwd<_Float16, 128>(kp, s);
+        return launch_bwd<_Float16, 256>(kp, s);
     }
     if (DP == 32) return launch_bwd<uint16_t, 32>(kp, s);
     if (DP == 64) return launch_bwd<uint16_t, 64>(kp, s);

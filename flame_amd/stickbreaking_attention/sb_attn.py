@@ -95,8 +95,6 @@ def attention_weights(q, k, inv_temp=None, attend_current=False):
     _lib.check_supported(q)
     if inv_temp is None:
         inv_temp = 1 / math.sqrt(q.size(-1))
-    if q.dtype == torch.float16:          # exact in float32; the kernel takes bf16 and float32
-        q, k = q.float(), k.float()
     B, H, T, _ = q.shape
     W = torch.zeros((B, H, T, T), dtype=torch.float32, device=q.device)
     if W.numel():
@@ -180,9 +178,4 @@ def sb_attn_(q, k, v, inv_temp, attend_current):
     if not torch.is_grad_enabled():
         # no backward can follow: detached inputs tell the forward to keep no carry table
         q, k, v = q.detach(), k.detach(), v.detach()
-    if q.dtype == k.dtype == v.dtype == torch.float16 and _lib.float16_needs_float32_route():
-        # float16 has matrix-core kernels of its own (the bf16 sources compiled for float16 elements) and no generic
-        # ones: with those forced its values, exact in float32, run as float32 and come back rounded
-        o, rem = StickBreakingAttention.apply(q.float(), k.float(), v.float(), inv_temp, attend_current)
-        return o.half(), rem.half()
     return StickBreakingAttention.apply(q, k, v, inv_temp, attend_current)

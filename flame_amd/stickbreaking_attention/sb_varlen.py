@@ -157,8 +157,6 @@ def attention_weights_varlen(q, k, cu_seqlens, max_seqlens, inv_temp=None, atten
     _lib.check_supported(q)
     if inv_temp is None:
         inv_temp = 1 / math.sqrt(q.size(-1))
-    if q.dtype == torch.float16:          # exact in float32; the kernel takes bf16 and float32
-        q, k = q.float(), k.float()
     H, N, _ = q.shape
     W = torch.zeros((H, N, N), dtype=torch.float32, device=q.device)
     if W.numel():
@@ -274,11 +272,6 @@ def _apply(q, k, v, cu_seqlens, max_seqlens, inv_temp, attend_current):
     if not torch.is_grad_enabled():
         # no backward can follow: detached inputs tell the forward to keep no carry table
         q, k, v = q.detach(), k.detach(), v.detach()
-    if q.dtype == k.dtype == v.dtype == torch.float16 and _lib.float16_needs_float32_route():
-        # with the generic kernels forced float16 runs as float32 (see sb_attn.sb_attn_) and is rounded on the way out
-        o, rem = StickBreakingAttention.apply(q.float(), k.float(), v.float(), cu_seqlens, max_seqlens, inv_temp,
-                                              attend_current)
-        return o.half(), rem.half()
     return StickBreakingAttention.apply(q, k, v, cu_seqlens, max_seqlens, inv_temp, attend_current)
 
 

@@ -47,13 +47,13 @@ extern "C" {
 #define SBA_SCHEDULE_INTS 8   /* int32 per scheduled job, see sba_build_schedule() */
 #define SBA_DOC_MAJOR_GRID 8192 /* workgroups from which the schedule is document-major */
 
-enum { SBA_DTYPE_F32 = 0, SBA_DTYPE_BF16 = 1, SBA_DTYPE_F16 = 2 };   /* float16: head_dim 64, 128 or 256 only (the reference's kernels take whatever dtype the tensors have, sb_attn/sb_fwd.py:144-146) */
+enum { SBA_DTYPE_F32 = 0, SBA_DTYPE_BF16 = 1, SBA_DTYPE_F16 = 2 };   /* (the reference's kernels take whatever dtype the tensors have, sb_attn/sb_fwd.py:144-146) */
 
 enum {
     SBA_OK = 0,
     SBA_ERR_NULL = -1,        /* a required pointer is NULL */
     SBA_ERR_SHAPE = -2,       /* non-positive size, head_dim unsupported, bad strides */
-    SBA_ERR_DTYPE = -3,       /* unknown dtype, or float16 at a head_dim other than 64 / 128 / 256 */
+    SBA_ERR_DTYPE = -3,       /* unknown dtype */
     SBA_ERR_WORKSPACE = -4,   /* workspace or bwd_scratch missing or too small */
     SBA_ERR_SCHEDULE = -5,    /* packed layout without a row-block schedule */
     SBA_ERR_LAUNCH = -6,      /* hipGetLastError() after a launch was not hipSuccess */
@@ -187,7 +187,7 @@ int sba_bwd(const SbaParams* p);
 /*
  * The attention weights A_ij themselves, in fp32: the reference forward's `return_attention` debug output
  * (sb_attn/sb_fwd.py:141-172 `W`, sb_varlen/sb_varlen_fwd.py:195-201 and :409-446).  Reads q, k, scale,
- * attend_current and the layout fields of *p (dtype bf16 or fp32, any head_dim; o, rem and the workspace are not
+ * attend_current and the layout fields of *p (any dtype and head_dim; o, rem and the workspace are not
  * touched) and writes weights[b][h][i][j] (dense, [n_seq, n_heads, seq_len, seq_len] contiguous) or
  * weights[h][i][j] (packed, [n_heads, total_tokens, total_tokens] contiguous, i and j token positions in the
  * pack) for every allowed pair; all other entries are left as they are (zero-fill first, as the reference does).

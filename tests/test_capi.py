@@ -49,17 +49,14 @@ def test_argument_checks_without_gpu(lib):
     assert lib.sba_workspace_bytes(C.byref(p)) == 0 and lib.sba_bwd_scratch_bytes(C.byref(p)) == 0
     p.head_dim = 64
     assert lib.sba_fwd(C.byref(p)) == -1          # NULL q/k/v
-    p.dtype = _lib.SBA_DTYPE_F16                  # float16: matrix-core head dims only
+    p.dtype = _lib.SBA_DTYPE_F16                  # float16: every head dim, like bf16
     assert lib.sba_fwd(C.byref(p)) == -1
     p.head_dim = 96
-    assert lib.sba_fwd(C.byref(p)) == -3
+    assert lib.sba_fwd(C.byref(p)) == -1
     p.dtype, p.head_dim = _lib.SBA_DTYPE_BF16, 64
     assert lib.sba_attention_weights(C.byref(p), None) == -1      # NULL q/k/v come first
     p.q.ptr = p.k.ptr = p.v.ptr = 256                             # never dereferenced: the checks below come before any launch
     assert lib.sba_attention_weights(C.byref(p), None) == -1      # no output
-    p.dtype = _lib.SBA_DTYPE_F16
-    assert lib.sba_attention_weights(C.byref(p), 256) == -3       # bf16 and fp32 only
-    p.dtype = _lib.SBA_DTYPE_BF16
     p.q.ptr = p.k.ptr = p.v.ptr = None
     assert lib.sba_fwd(None) == -1
     assert lib.sba_row_block() == 128
@@ -136,6 +133,10 @@ def test_workspace_bytes(lib):
     p.head_dim = 64
     assert lib.sba_bwd_scratch_bytes(C.byref(p)) == 4 * table + scaled_q + 256
     p.dtype, p.head_dim = _lib.SBA_DTYPE_BF16, 256
+    p.dtype, p.head_dim = _lib.SBA_DTYPE_F16, 200   # float16 on the generic kernels: sized like bf16 there too
+    assert lib.sba_workspace_bytes(C.byref(p)) == 0
+    assert lib.sba_bwd_scratch_bytes(C.byref(p)) == 2 * 4096 * 16 * 256 * 4
+    p.dtype = _lib.SBA_DTYPE_BF16
     p.head_dim = 200                                # bf16 in between: generic kernels unless the caller pads to 256
     assert lib.sba_workspace_bytes(C.byref(p)) == 0
     assert lib.sba_bwd_scratch_bytes(C.byref(p)) == 2 * 4096 * 16 * 256 * 4
@@ -281,11 +282,9 @@ def test_head_dim_routing_of_the_python_layer(monkeypatch):
         for D, Dp in table.items():
             assert _lib.matrix_core_head_dim(torch.empty(1, 1, 1, D, dtype=dtype)) == Dp, (dtype, D)
     assert _lib.dtype_code(torch.float16) == _lib.SBA_DTYPE_F16 == 2
-    assert not _lib.float16_needs_float32_route()
     with pytest.raises(ValueError, match="head_dim"):
         _lib.check_supported(torch.empty(1, 1, 1, 257, dtype=torch.bfloat16))
     with pytest.raises(TypeError, match="float16"):
         _lib.check_supported(torch.empty(1, 1, 1, 64, dtype=torch.float64))
     monkeypatch.setenv("SBA_FORCE_GENERIC", "1")
     assert _lib.matrix_core_head_dim(torch.empty(1, 1, 1, 80, dtype=torch.bfloat16)) == 80
-    assert _lib.float16_needs_float32_route()

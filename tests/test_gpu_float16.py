@@ -112,8 +112,12 @@ def test_float16_saturated_logits_stay_finite_and_accurate():
         assert torch.isfinite(g_).all() and rel_l2(g_.float().cpu(), r) <= GRAD_TOL[F16]
 
 
-def test_float16_with_the_generic_kernels_forced_runs_as_float32(monkeypatch):
-    # float16 has no generic kernels: under SBA_FORCE_GENERIC=1 its values, exact in float32, run there
+def test_float16_on_the_generic_kernels(monkeypatch):
+    # the vector-ALU kernels in float16 storage (fp32 arithmetic): forced for everything, and for the backward alone
     monkeypatch.setenv("SBA_FORCE_GENERIC", "1")
     _check_dense(1, 2, 200, 64, F16, seed=90, in_scale=0.5)
+    _check_dense(1, 2, 130, 200, F16, attend_current=True, seed=92, in_scale=0.5)
     _check_varlen(2, 80, [130, 45], F16, seed=91)
+    monkeypatch.delenv("SBA_FORCE_GENERIC")
+    monkeypatch.setenv("SBA_FORCE_GENERIC_BWD", "1")
+    _check_dense(1, 2, 300, 128, F16, seed=93, in_scale=0.5)
