@@ -121,6 +121,16 @@ def check_supported(q: torch.Tensor) -> None:
         raise ValueError(f"head_dim {q.shape[-1]} is not supported (at most {MAX_HEAD_DIM})")
 
 
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+
+
+def current_stream_handle(device: torch.device) -> int:
+    """hipStream_t of torch's current stream on `device` (the stream the kernels are launched on)."""
+    if _raw_stream is not None and device.index is not None:
+        return _raw_stream(device.index)          # the same handle, without building a torch.cuda.Stream object
+    return torch.cuda.current_stream(device).cuda_stream
+
+
 def tensor4(t: torch.Tensor) -> SbaTensor:
     """[B, H, T, D] view -> descriptor."""
     return SbaTensor(t.data_ptr(), t.stride(0), t.stride(1), t.stride(2))
@@ -146,7 +156,9 @@ def empty_grads_like(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor):
     """Uninitialised dq, dk, dv.  When q, k and v are the three column slices of one [.., 3*H*D] tensor (the
     output of a stacked q/k/v projection), the gradients are laid out the same way in ONE allocation, so that
     the caller's backward can hand the whole of it to the projection without concatenating."""
-    if not torch.compiler.is_compiling() and q.shape == k.shape == v.shape and q.stride() == k.stride() == v.stride():
+    # (three tensors at the same offset of their storages cannot be slices of one buffer: the usual case, decided first)
+    if (k.storage_offset() != q.storage_offset() and not torch.compiler.is_compiling()
+            and q.shape == k.shape == v.shape and q.stride() == k.stride() == v.stride()):
         n = q.numel()
         span = sum((sz - 1) * st for sz, st in zip(q.shape, q.stride())) + 1      # elements from q's first to its last
         base = q.untyped_storage().data_ptr()

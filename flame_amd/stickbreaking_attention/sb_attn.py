@@ -8,6 +8,7 @@ entry points sba_fwd / sba_bwd of libsba_mi355x.so.
 from __future__ import annotations
 
 import ctypes as C
+import os
 import math
 from typing import Optional
 
@@ -27,8 +28,17 @@ def _params(q, k, v, inv_temp, attend_current):
     p.attend_current = int(bool(attend_current))
     p.scale = float(inv_temp)
     p.q, p.k, p.v = _lib.tensor4(q), _lib.tensor4(k), _lib.tensor4(v)
-    p.stream = torch.cuda.current_stream(q.device).cuda_stream
+    p.stream = _lib.current_stream_handle(q.device)
     return p
+
+
+# The two sizes depend on dtype, shape and the two switches that route a problem to the generic kernels: asked of the
+# library once per such key (a size query costs as much host time as a launch, and a training step asks twice per layer).
+_SIZES = {}
+
+
+def _size_key(q, what):
+    return (what, q.dtype, tuple(q.shape), os.environ.get("SBA_FORCE_GENERIC"), os.environ.get("SBA_FORCE_GENERIC_BWD"))
 
 
 def workspace_bytes(q, inv_temp=1.0) -> int:
@@ -36,7 +46,11 @@ def workspace_bytes(q, inv_temp=1.0) -> int:
     if torch.compiler.is_compiling():
         B, H, T, D = q.shape
         return _lib.workspace_upper_bound(H, _lib.dense_columns(B, T))
-    return int(_lib.load().sba_workspace_bytes(C.byref(_params(q, q, q, inv_temp, False))))
+    key = _size_key(q, 0)
+    n = _SIZES.get(key)
+    if n is None:
+        n = _SIZES[key] = int(_lib.load().sba_workspace_bytes(C.byref(_params(q, q, q, inv_temp, False))))
+    return n
 
 
 def bwd_scratch_bytes(q, have_workspace=True) -> int:
@@ -45,9 +59,13 @@ def bwd_scratch_bytes(q, have_workspace=True) -> int:
     if torch.compiler.is_compiling():
         B, H, T, D = q.shape
         return _lib.bwd_scratch_upper_bound(H, _lib.dense_columns(B, T), B * T, D)
-    p = _params(q, q, q, 1.0, False)
-    p.workspace = 1 if have_workspace else None       # only NULL or not is looked at
-    return int(_lib.load().sba_bwd_scratch_bytes(C.byref(p)))
+    key = _size_key(q, 1 if have_workspace else 2)
+    n = _SIZES.get(key)
+    if n is None:
+        p = _params(q, q, q, 1.0, False)
+        p.workspace = 1 if have_workspace else None       # only NULL or not is looked at
+        n = _SIZES[key] = int(_lib.load().sba_bwd_scratch_bytes(C.byref(p)))
+    return n
 
 
 # Same registered names as the reference (sb_fwd.py:177, sb_bwd.py:207); outputs are

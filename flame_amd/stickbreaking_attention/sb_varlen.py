@@ -59,7 +59,7 @@ def _params(q, k, v, n_docs, max_seqlens, inv_temp, attend_current):
     p.attend_current = int(bool(attend_current))
     p.scale = float(inv_temp)
     p.q, p.k, p.v = _lib.tensor3(q), _lib.tensor3(k), _lib.tensor3(v)
-    p.stream = torch.cuda.current_stream(q.device).cuda_stream
+    p.stream = _lib.current_stream_handle(q.device)
     return p
 
 
