@@ -157,7 +157,7 @@ def empty_grads_like(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor):
     output of a stacked q/k/v projection), the gradients are laid out the same way in ONE allocation, so that
     the caller's backward can hand the whole of it to the projection without concatenating."""
     # (three tensors at the same offset of their storages cannot be slices of one buffer: the usual case, decided first)
-    if (k.storage_offset() != q.storage_offset() and not torch.compiler.is_compiling()
+    if (not torch.compiler.is_compiling() and k.storage_offset() != q.storage_offset()
             and q.shape == k.shape == v.shape and q.stride() == k.stride() == v.stride()):
         n = q.numel()
         span = sum((sz - 1) * st for sz, st in zip(q.shape, q.stride())) + 1      # elements from q's first to its last
