@@ -345,6 +345,9 @@ def main():
                     help="kept: the forward keeps its carry tables whatever their size (the kernels as such); default: the "
                          "operator's own rule, which above its workspace budget (256 MiB) keeps nothing and lets the "
                          "backward rebuild them (cfg4: 270 MB)")
+    ap.add_argument("--autograd-thread", default="off", choices=["off", "on"],
+                    help="off (default): torch.autograd.set_multithreading_enabled(False), the backward is issued from the "
+                         "calling thread; on: PyTorch's default worker thread per device")
     ap.add_argument("--compile", action="store_true",
                     help="cfg5 only: torch.compile every block, as flame does with --training.compile")
     args = ap.parse_args()
@@ -357,6 +360,11 @@ def main():
     from flame_amd.stickbreaking_attention import profiling
 
     dev = torch.device("cuda:0")
+    if args.autograd_thread == "off":
+        # The backward runs in the calling thread instead of autograd's per-device worker: a forward + backward of the
+        # operator then costs the host about 80 us instead of 160-200, which on a box with a slow host is the
+        # difference between timing the kernels and timing Python.  Same graph, same kernels, same results.
+        torch.autograd.set_multithreading_enabled(False)
     if args.workload == "cfg5":
         return bench_model(args, dev)
     if args.workload == "copy":
